@@ -1,0 +1,33 @@
+"""CPU oracle for the quantized RWKV inference hot path.  TEST INFRASTRUCTURE ONLY.
+
+This package restates, in numpy, the arithmetic of the reference path
+``RWKV(model, strategy).forward(tokens, state)``
+(rwkv_pip_package/src/rwkv/model.py:612-1677 and the kernels under
+rwkv_pip_package/src/rwkv/cuda/).  It exists to check the HIP path and to be
+timed as the CPU baseline.  Only ``tests/``, ``__graft_entry__.smoke()`` and the
+``cpu_baseline`` leg of ``bench.py`` may import it; the product package
+``chatrwkv_amd`` never does and fails loudly when its HIP library is missing.
+
+Modules
+  quant.py   uint8 quantizer + dequantisation          (model.py:818-847, 91-97)
+  ops.py     LayerNorm/GroupNorm, mm8, WKV v4/v5/v6     (model.py:984-1340, cuda/*.cu)
+  model.py   checkpoint conversion + forward            (model.py:613-903, 1443-1677)
+
+How each function is pinned (what a wrong sign / index / dropped term would trip):
+  quantize_u8          golden vectors written by the reference's own loader
+                       (tests/golden/quant_*.npz) + invariants (0 and 255 in
+                       every row and column, reconstruction bound).
+  mm8 / dequant        fp64 ``x @ W'`` library matmul; factorised identity.
+  wkv4_*               O(T^2) closed form in fp64; zero-state T=1 => wkv = v;
+                       golden end-to-end logits + state from the reference.
+  wkv5/6 recurrences   O(T^2) closed form in fp64; v5 parallel form vs recurrent
+                       form; non-symmetric state for the [h][key][value] layout;
+                       golden end-to-end logits + state from the reference.
+  layer_norm/group_norm  torch CPU library routines.
+  forward (all versions) golden logits and final state from the reference's CPU
+                       path ('cpu fp32i8', 'cpu fp32'); chunk invariance.
+The fp16 rounding points of the reference's 'cuda fp16i8' path cannot be run
+anywhere in this build (needs nvcc + an NVIDIA GPU): for that emulation mode the
+placement of the roundings follows the reference text and is otherwise
+"parity unpinned"; its arithmetic is the same code the goldens pin in fp32.
+"""

@@ -1,0 +1,282 @@
+"""Oracle: checkpoint conversion and ``forward`` of the reference, in numpy.
+
+Test infrastructure only (see oracle/__init__.py).
+
+``OracleRWKV(checkpoint, strategy)`` restates ``RWKV.__init__`` (model.py:613-903:
+version detection, weight transforms, uint8 quantisation) and ``RWKV.forward``
+(model.py:1443-1677) for RWKV-4, 5.0, 5.1, 5.2 and 6.0.  Supported strategies are the
+single-segment ones:
+
+  'cpu fp32', 'cpu fp32i8'    the arithmetic the reference runs on CPU: fp32 everywhere,
+                              RESCALE_LAYER = 0 (model.py:634).  'cpu fp32i8' is the CPU
+                              baseline path: every matmul dequantises the whole matrix
+                              per call (model.py:91-97).
+  'cuda fp16', 'cuda fp16i8'  emulation of the GPU path: fp16 activations, fp32 WKV, fp32
+                              accumulation in every contraction, roundings where the
+                              reference's CUDA path rounds, RESCALE_LAYER = 6.
+
+Weights keep the reference's names (``blocks.0.att.key.weight`` and its ``_mx/_rx/_my/_ry``
+companions) so converted dicts can be compared key by key with the reference's.
+"""
+import os
+import re
+
+import numpy as np
+
+from . import ops, quant
+from .ops import Mat, f16, f32
+
+_STRATEGY = re.compile(r"^ *(cuda(?::0)?|cpu) (fp16|fp32)(i8)? *$")
+
+_MATRIX_KEYS = ('key.weight', 'value.weight', 'receptance.weight', 'gate.weight',
+                'output.weight', 'head.weight')
+
+
+def _np(t):
+    return t.detach().cpu().numpy() if hasattr(t, 'detach') else np.asarray(t)
+
+
+class OracleRWKV:
+    def __init__(self, checkpoint, strategy, rescale_layer=None, cache_dequant=None):
+        m = _STRATEGY.match(strategy)
+        if not m:
+            raise ValueError("oracle supports single-segment cpu/cuda fp32/fp16[i8] strategies")
+        self.device, at, i8 = m.group(1), m.group(2), m.group(3)
+        self.atype = f32 if at == 'fp32' else f16
+        self.wtype = np.uint8 if i8 else self.atype
+        # model.py:631-634
+        if rescale_layer is None:
+            env = os.environ.get("RWKV_RESCALE_LAYER")
+            rescale_layer = int(env) if env not in (None, '') else (6 if at == 'fp16' else 0)
+        self.rescale_layer = rescale_layer
+        # the CPU baseline path dequantises per call; the emulation may cache
+        self.cache = (self.device != 'cpu') if cache_dequant is None else cache_dequant
+        self._convert({k: _np(v) for k, v in checkpoint.items()})
+
+    # ------------------------------------------------------------------ conversion
+    def _convert(self, w):
+        # model.py:658-680
+        self.n_embd = w['emb.weight'].shape[1]
+        self.n_att = w['blocks.0.att.key.weight'].shape[0]
+        self.n_ffn = w['blocks.0.ffn.key.weight'].shape[0]
+        self.n_layer = 0
+        self.version = 4
+        self.n_head = 0
+        for x in w:
+            lid = int(x.split('.')[1]) if 'blocks.' in x else 0
+            self.n_layer = max(self.n_layer, lid + 1)
+            if 'ln_x' in x:
+                self.version = max(5, self.version)
+            if 'gate.weight' in x:
+                self.version = max(5.1, self.version)
+            if int(self.version) == 5 and 'att.time_decay' in x:
+                self.n_head = w[x].shape[0]
+                if w[x].ndim > 1 and w[x].shape[1] > 1:
+                    self.version = max(5.2, self.version)
+            if 'time_maa' in x:
+                self.version = max(6, self.version)
+            if int(self.version) == 6 and 'time_faaaa' in x:
+                self.n_head = w[x].shape[0]
+        A, R = self.atype, self.rescale_layer
+
+        # model.py:754-760: embedding absorbs ln0
+        w['emb.weight'] = ops.layer_norm(w['emb.weight'].astype(f32),
+                                         w['blocks.0.ln0.weight'], w['blocks.0.ln0.bias'])
+        del w['blocks.0.ln0.weight'], w['blocks.0.ln0.bias']
+        # model.py:764-771
+        real_time_first = any('.time_faaaa' in k for k in w)
+        w = {k.replace('.time_faaaa', '.time_first'): v for k, v in w.items()}
+
+        out = {}
+        for x, t in w.items():
+            lid = int(x.split('.')[1]) if 'blocks.' in x else 0
+            t = t.astype(f32)
+            if R > 0 and ('att.output.weight' in x or 'ffn.value.weight' in x):
+                t = t / f32(2 ** int(lid // R))                      # model.py:785-789
+            if '.time_' in x:
+                t = np.squeeze(t)                                    # model.py:791-792
+            if any(s in x for s in _MATRIX_KEYS):
+                t = t.T                                              # model.py:793-794 -> [in, out]
+            if '.time_decay' in x and '_w' not in x:                 # model.py:796-804
+                if self.version == 4:
+                    t = -np.exp(t)
+                elif int(self.version) == 5:
+                    t = np.exp(-np.exp(t)).reshape(-1, 1, 1)
+                    if self.version == 5.2:
+                        t = t.reshape(self.n_head, -1, 1)
+                else:
+                    t = t.reshape(self.n_head, -1, 1)
+                out[x] = t.astype(f32)
+            elif '.time_first' in x:                                 # model.py:805-814
+                if self.version != 4:
+                    t = (t if real_time_first else np.exp(t)).reshape(-1, 1, 1)
+                    if self.version in (5.2, 6):
+                        t = t.reshape(self.n_head, -1, 1)
+                out[x] = t.astype(f32)
+            elif '.ln_x' in x:                                       # model.py:815-816
+                out[x] = t.astype(f32)
+            elif t.ndim == 2 and 'emb' not in x and '_w1' not in x and '_w2' not in x:
+                if self.wtype != np.uint8:                           # model.py:819-820
+                    out[x] = np.ascontiguousarray(t).astype(self.wtype)
+                else:                                                # model.py:821-847
+                    q, mx, rx, my, ry = quant.quantize_u8(t, atype=A)
+                    out[x] = q
+                    out[x + '_mx'], out[x + '_rx'] = mx, rx
+                    out[x + '_my'], out[x + '_ry'] = my, ry
+            else:
+                out[x] = t.astype(A)                                 # model.py:849
+        self.w = out
+        self._mats = {}
+
+    def mat(self, name):
+        m = self._mats.get(name)
+        if m is None:
+            w = self.w
+            if w[name].dtype == np.uint8:
+                m = Mat(w[name], w[name + '_mx'], w[name + '_rx'], w[name + '_my'], w[name + '_ry'])
+            else:
+                m = Mat(w[name])
+            self._mats[name] = m
+        return m
+
+    def _mm(self, a, name, output_dtype=None):
+        return ops.matmul(a, self.mat(name), self.atype, output_dtype, cache=self.cache)
+
+    # ------------------------------------------------------------------ state
+    def init_state(self):
+        """model.py:1448-1471."""
+        L, C, A = self.n_layer, self.n_embd, self.atype
+        st = []
+        for i in range(L):
+            if self.version == 4:
+                st += [np.zeros(C, A), np.zeros(self.n_att, f32), np.zeros(self.n_att, f32),
+                       np.full(self.n_att, -1e30, f32), np.zeros(C, A)]
+            else:
+                N = self.n_att // self.n_head
+                st += [np.zeros(C, A), np.zeros((self.n_head, N, N), f32), np.zeros(C, A)]
+        return st
+
+    # ------------------------------------------------------------------ blocks
+    @staticmethod
+    def _shift(sx, xx):
+        """Token shift (model.py:997, 1060): row t sees the normalised activation of t-1."""
+        return np.concatenate([sx[None, :], xx[:-1]], axis=0)
+
+    def _ffn(self, x, sx, i):
+        """Channel mix.  v4/v5: model.py:984-1004; v6: model.py:1007-1029."""
+        w, p = self.w, f'blocks.{i}.'
+        one = self.atype(1)
+        xx = ops.layer_norm(x, w[p + 'ln2.weight'], w[p + 'ln2.bias'])
+        prev = self._shift(sx, xx)
+        if self.version >= 6:
+            d = prev - xx
+            kx = xx + d * w[p + 'ffn.time_maa_k']
+            rx = xx + d * w[p + 'ffn.time_maa_r']
+        else:
+            mk, mr = w[p + 'ffn.time_mix_k'], w[p + 'ffn.time_mix_r']
+            kx = xx * mk + prev * (one - mk)
+            rx = xx * mr + prev * (one - mr)
+        r = ops.sigmoid(self._mm(rx, p + 'ffn.receptance.weight'))
+        vx = ops.relu_sq(self._mm(kx, p + 'ffn.key.weight'))
+        out = r * self._mm(vx, p + 'ffn.value.weight')
+        return x + out, xx[-1]
+
+    def _att_v4(self, x, sx, aa, bb, pp, i):
+        """RWKV-4 time mix.  model.py:1034-1086 and 1346-1360."""
+        w, p = self.w, f'blocks.{i}.'
+        a = p + 'att.'
+        one = self.atype(1)
+        xx = ops.layer_norm(x, w[p + 'ln1.weight'], w[p + 'ln1.bias'])
+        prev = self._shift(sx, xx)
+        mk, mv, mr = w[a + 'time_mix_k'], w[a + 'time_mix_v'], w[a + 'time_mix_r']
+        kx = xx * mk + prev * (one - mk)
+        vx = xx * mv + prev * (one - mv)
+        rx = xx * mr + prev * (one - mr)
+        r = ops.sigmoid(self._mm(rx, a + 'receptance.weight'))
+        k = self._mm(kx, a + 'key.weight', output_dtype=f32)
+        v = self._mm(vx, a + 'value.weight', output_dtype=f32)
+        y, aa, bb, pp = ops.wkv4(k, v, w[a + 'time_first'], w[a + 'time_decay'], aa, bb, pp)
+        out = self._mm(r * y.astype(self.atype), a + 'output.weight')
+        return x + out, xx[-1], aa, bb, pp
+
+    def _att_v56(self, x, sx, S, i):
+        """RWKV-5.0 / 5.1 / 5.2 / 6.0 time mix.  model.py:1091-1340, 1363-1439."""
+        w, p = self.w, f'blocks.{i}.'
+        a = p + 'att.'
+        A = self.atype
+        one = A(1)
+        T = x.shape[0]
+        H = self.n_head
+        N = self.n_att // H
+        xx = ops.layer_norm(x, w[p + 'ln1.weight'], w[p + 'ln1.bias'])
+        prev = self._shift(sx, xx)
+        gated = self.version >= 5.1
+        if self.version >= 6:
+            d = prev - xx
+            xxx = xx + d * w[a + 'time_maa_x']
+            xxx = np.tanh(ops.small_matmul(xxx, w[a + 'time_maa_w1'], A).astype(f32)).astype(A)
+            xxx = xxx.reshape(T, 5, -1).transpose(1, 0, 2)                       # [5, T, 32]
+            mm = np.stack([ops.small_matmul(xxx[j], w[a + 'time_maa_w2'][j], A) for j in range(5)])
+            wx = xx + d * (w[a + 'time_maa_w'] + mm[0])
+            kx = xx + d * (w[a + 'time_maa_k'] + mm[1])
+            vx = xx + d * (w[a + 'time_maa_v'] + mm[2])
+            rx = xx + d * (w[a + 'time_maa_r'] + mm[3])
+            gx = xx + d * (w[a + 'time_maa_g'] + mm[4])
+        else:
+            mix = lambda name: xx * w[a + name] + prev * (one - w[a + name])
+            kx, vx, rx = mix('time_mix_k'), mix('time_mix_v'), mix('time_mix_r')
+            if gated:
+                gx = mix('time_mix_g')
+        r = self._mm(rx, a + 'receptance.weight', output_dtype=f32).reshape(T, H, N)
+        k = self._mm(kx, a + 'key.weight', output_dtype=f32).reshape(T, H, N)
+        v = self._mm(vx, a + 'value.weight', output_dtype=f32).reshape(T, H, N)
+        if gated:
+            g = ops.silu(self._mm(gx, a + 'gate.weight'))
+        if self.version >= 6:
+            # model.py:1286-1287, 1324-1325
+            lo = np.tanh(ops.small_matmul(wx, w[a + 'time_decay_w1'], A).astype(f32)).astype(A)
+            lo = ops.small_matmul(lo, w[a + 'time_decay_w2'], A).astype(f32)
+            dec = w[a + 'time_decay'].reshape(1, H, N) + lo.reshape(T, H, N)
+            dec = np.exp(-np.exp(dec.astype(f32))).astype(f32)
+        else:
+            dec = w[a + 'time_decay'].reshape(H, -1)
+        out, S = ops.wkv56(r, k, v, dec, w[a + 'time_first'].reshape(H, -1), S)
+        out = ops.group_norm(out.reshape(T, H * N), H, w[a + 'ln_x.weight'], w[a + 'ln_x.bias'])
+        out = out.astype(A)
+        if gated:
+            out = out * g
+        out = self._mm(out, a + 'output.weight')
+        return x + out, xx[-1], S
+
+    # ------------------------------------------------------------------ forward
+    def forward(self, tokens, state, full_output=False):
+        """model.py:1443-1677.  tokens: list of ints; returns (logits fp32, state list)."""
+        w, A = self.w, self.atype
+        if state is None:
+            state = self.init_state()
+        seq_mode = len(tokens) > 1
+        x = w['emb.weight'][np.asarray(tokens, dtype=np.int64)].astype(A)
+        for i in range(self.n_layer):
+            if self.version == 4:
+                o = 5 * i
+                x, state[o], state[o + 1], state[o + 2], state[o + 3] = self._att_v4(
+                    x, state[o], state[o + 1], state[o + 2], state[o + 3], i)
+                x, state[o + 4] = self._ffn(x, state[o + 4], i)
+            else:
+                o = 3 * i
+                x, state[o], state[o + 1] = self._att_v56(x, state[o], state[o + 1], i)
+                x, state[o + 2] = self._ffn(x, state[o + 2], i)
+            if self.rescale_layer > 0 and (i + 1) % self.rescale_layer == 0:
+                x = x / A(2)                                         # model.py:1660-1662
+        if seq_mode and not full_output:
+            x = x[-1:]
+        x = ops.layer_norm(x, w['ln_out.weight'], w['ln_out.bias'])
+        m = self.mat('head.weight')
+        if m.quantized:
+            x = ops.matmul(x, m, A, cache=self.cache)               # model.py:1672-1675
+        else:
+            x = ops.matmul(x, m, A, output_dtype=A, cache=self.cache)  # model.py:1670
+        x = x.astype(f32)
+        if not (seq_mode and full_output):
+            x = x[0]
+        return x, state

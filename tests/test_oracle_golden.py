@@ -1,0 +1,94 @@
+"""The oracle against the golden vectors written by the reference's own CPU path
+(tests/golden/make_goldens.py).  A wrong branch, sign, index or dropped term in the
+oracle fails here."""
+import os
+
+import numpy as np
+import pytest
+
+from chatrwkv_amd import synth
+from oracle.model import OracleRWKV
+
+from tests.golden.make_goldens import TINY, TINY8, PROMPT_SEED
+
+G = os.path.join(os.path.dirname(__file__), "golden")
+
+
+def _load(name):
+    return dict(np.load(os.path.join(G, name)))
+
+
+def test_quantizer_bit_exact_cpu_fp32i8():
+    """uint8 matrices and fp32 mx/rx/my/ry of every matrix equal the reference's, bit for bit
+    (both branches: ffn.key is N<M, ffn.value is N>M, att.* are square, head is N<M)."""
+    ref = _load("quant_v4_cpu_fp32i8.npz")
+    o = OracleRWKV(synth.make_checkpoint(version=4, seed=101, **TINY), "cpu fp32i8")
+    assert set(ref) == set(o.w)
+    n_u8 = 0
+    for k, v in ref.items():
+        mine = o.w[k]
+        assert mine.shape == v.shape, k
+        assert mine.dtype == v.dtype, k
+        if v.dtype == np.uint8:
+            n_u8 += 1
+            assert np.array_equal(mine, v), k
+        elif k.endswith(("_mx", "_rx", "_my", "_ry")):
+            assert np.array_equal(mine.view(np.uint32), v.view(np.uint32)), k
+        else:
+            np.testing.assert_allclose(mine, v, rtol=2e-6, atol=2e-6, err_msg=k)
+    assert n_u8 == 3 * 7 + 1
+
+
+def test_quantizer_bit_exact_cuda_fp16i8_convert():
+    """The dict the reference's convert_and_save_and_exit writes under 'cuda fp16i8':
+    fp16 scales, RESCALE_LAYER 6 applied to att.output / ffn.value of layers >= 6."""
+    ref = _load("quant_v4_cuda_fp16i8.npz")
+    assert str(ref.pop("meta_strategy")) == "cuda fp16i8"
+    assert int(ref.pop("meta_rescale_layer")) == 6
+    ref.pop("meta_version")
+    o = OracleRWKV(synth.make_checkpoint(version=4, seed=102, **TINY8), "cuda fp16i8")
+    assert o.rescale_layer == 6
+    assert set(ref) == set(o.w)
+    for k, v in ref.items():
+        mine = o.w[k]
+        assert mine.shape == v.shape and mine.dtype == v.dtype, k
+        if v.dtype == np.uint8:
+            assert np.array_equal(mine, v), k
+        elif k.endswith(("_mx", "_rx", "_my", "_ry")):
+            assert v.dtype == np.float16
+            assert np.array_equal(mine.view(np.uint16), v.view(np.uint16)), k
+        elif v.dtype == np.float16:
+            # emb (LayerNorm'ed), time_mix, ln weights: at most one fp16 ulp from the LN rounding
+            np.testing.assert_allclose(mine.astype(np.float32), v.astype(np.float32), rtol=2e-3, atol=1e-3, err_msg=k)
+        else:
+            np.testing.assert_allclose(mine, v, rtol=2e-6, atol=2e-6, err_msg=k)
+
+
+VERS = [(4, "v4"), (5, "v5_0"), (5.1, "v5_1"), (5.2, "v5_2"), (6, "v6_0")]
+
+
+@pytest.mark.parametrize("ver,tag", VERS)
+@pytest.mark.parametrize("strat", ["cpu fp32i8", "cpu fp32"])
+def test_forward_matches_reference_cpu(ver, tag, strat):
+    """Logits (full_output, chunked seq calls, one-token calls) and final state of tiny models
+    against the reference's CPU path."""
+    ref = _load(f"e2e_{tag}_{strat.replace(' ', '_')}.npz")
+    ck = synth.make_checkpoint(version=ver, seed=200 + int(ver * 10), **TINY)
+    o = OracleRWKV(ck, strat)
+    assert o.version == ver
+    toks = synth.random_tokens(9, TINY["vocab"], seed=PROMPT_SEED)
+    assert toks == list(ref["tokens"])
+    full, st_full = o.forward(toks, None, full_output=True)
+    assert full.dtype == np.float32 and full.shape == ref["full_logits"].shape
+    np.testing.assert_allclose(full, ref["full_logits"], rtol=2e-4, atol=2e-5)
+    st, outs = None, []
+    for a, b in ((0, 2), (2, 3), (3, 7), (7, 8), (8, 9)):
+        out, st = o.forward(toks[a:b], st)
+        assert out.shape == (TINY["vocab"],)
+        outs.append(out)
+    np.testing.assert_allclose(np.stack(outs), ref["chunk_logits"], rtol=2e-4, atol=2e-5)
+    for prefix, state in (("full_", st_full), ("chunk_", st)):
+        for i, s in enumerate(state):
+            r = ref[f"{prefix}state_{i}"]
+            assert s.shape == r.shape and s.dtype == r.dtype, (prefix, i)
+            np.testing.assert_allclose(s, r, rtol=2e-4, atol=2e-5, err_msg=f"{prefix}{i}")
