@@ -1,0 +1,75 @@
+// Shared device/host helpers for the gfx950 kernels.  Wave size is 64 everywhere.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stddef.h>
+#include "../../include/rwkv_hip.h"
+
+#define WAVE 64
+
+typedef _Float16 h16;
+typedef _Float16 h16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 h16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 h16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+#define DEV __device__ __forceinline__
+
+// ---- launch bookkeeping -------------------------------------------------------------------
+#define RWKV_LAUNCH_CHECK()                         \
+    do {                                            \
+        hipError_t e__ = hipGetLastError();         \
+        if (e__ != hipSuccess) return (int)e__;     \
+    } while (0)
+
+static inline bool aligned16(const void *p) { return (((uintptr_t)p) & 15) == 0; }
+
+// ---- fp16 <-> fp32 -----------------------------------------------------------------------
+DEV float h2f(rwkv_half v) { return (float)__builtin_bit_cast(h16, v); }
+DEV rwkv_half f2h(float v) { return __builtin_bit_cast(rwkv_half, (h16)v); }  // round-to-nearest-even
+DEV float round_h(float v) { return (float)(h16)v; }
+
+// ---- wave / block reductions ---------------------------------------------------------------
+DEV float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
+    return v;
+}
+DEV float wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, WAVE));
+    return v;
+}
+DEV float wave_min(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fminf(v, __shfl_xor(v, o, WAVE));
+    return v;
+}
+
+// Sum over the whole workgroup; every thread gets the result.  `red` is LDS scratch of at
+// least (blockDim.x / 64) floats; safe to call repeatedly with the same scratch.
+DEV float block_sum(float v, float *red) {
+    const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
+    v = wave_sum(v);
+    __syncthreads();
+    if (lane == 0) red[wid] = v;
+    __syncthreads();
+    float t = 0.f;
+    for (int i = 0; i < nw; ++i) t += red[i];
+    return t;
+}
+
+// ---- uint8 -> fp16 pairs -------------------------------------------------------------------
+// Bytes b0..b3 of `v` become the fp16 values (1024 + b): placing a byte under the exponent
+// byte 0x64 yields exactly 1024 + b.  lo = (b0, b1), hi = (b2, b3).
+DEV h16x2 u8pair_lo_1024(uint32_t v) {
+    return __builtin_bit_cast(h16x2, __builtin_amdgcn_perm(0x64646464u, v, 0x05010400u));
+}
+DEV h16x2 u8pair_hi_1024(uint32_t v) {
+    return __builtin_bit_cast(h16x2, __builtin_amdgcn_perm(0x64646464u, v, 0x07030602u));
+}
+
+DEV float sigmoidf_(float x) { return 1.f / (1.f + __expf(-x)); }

@@ -1,0 +1,294 @@
+// Prefill contraction y[T, M] = xs[T, N] @ W on fp16 MFMA (v_mfma_f32_32x32x16_f16).
+//
+// W is read in the input-contiguous layout (row m = N consecutive uint8 or fp16).  For
+// uint8 weights each 16-byte global load is widened in registers to the exact fp16 values
+// (b + 0.5) -- v_perm_b32 builds 1024 + b, one packed fp16 add removes 1023.5 -- and stored to
+// LDS, so the matrix cores see a plain fp16 x fp16 product with fp32 accumulation.  The
+// activation operand is the caller's x pre-multiplied by ry (mm8_prepare below), and the
+// rank-1 corrections enter in the epilogue:
+//     y[t, m] = rx[m] * acc[t, m] + mx[m] * S0[t] + S2[t],   S0 = sum_j x[t, j],  S2 = sum_j x[t, j] my[j].
+//
+// Tiling: BT x BM outputs per workgroup of 256 threads (2 x 2 waves), K step 64, LDS double
+// buffered; both LDS tiles are [row][64 halves] with the eight 16-byte chunks of a row XOR-
+// swizzled by (row & 7) so that the ds_read_b128 of 32 consecutive rows spreads over all banks.
+#include "common.h"
+
+namespace {
+
+constexpr int BK = 64;  // halves per LDS row
+
+enum { ACT_NONE = 0, ACT_SIGMOID = 1, ACT_RELU_SQ = 2, ACT_RESIDUAL = 3, ACT_GATED_RESIDUAL = 4 };
+
+struct GemmEpi {
+    const rwkv_half *mx, *rx;      // [M]; NULL for plain fp16 weights
+    const float *s0, *s2;          // [T]
+    int act;
+    const rwkv_half *res; int64_t ldres;   // residual input [T, M]
+    const rwkv_half *gate; int64_t ldgate; // gate [T, M]
+    float out_scale;               // applied to the final fp16 value (1 or 0.5)
+    int out_dtype;                 // RWKV_DT_F16 / RWKV_DT_F32 (F32 only with ACT_NONE: raw accumulator)
+};
+
+DEV int swz(int row, int chunk) { return row * BK + ((chunk ^ (row & 7)) << 3); }
+
+template <bool W_U8, int BT, int BM>
+__global__ __launch_bounds__(256) void gemm_kernel(int T, int N, int M, const h16 *__restrict__ A, int64_t lda,
+                                                   const void *__restrict__ Wv, int64_t ldw, void *__restrict__ Y,
+                                                   int64_t ldy, GemmEpi ep) {
+    static_assert(BT % 64 == 0 && BM % 64 == 0, "tile");
+    constexpr int MI = BT / 64, NI = BM / 64;  // 32x32 blocks per wave in each direction (2x2 waves)
+    extern __shared__ __align__(16) unsigned char smem[];
+    h16 *lA[2], *lB[2];
+    lA[0] = (h16 *)smem;
+    lB[0] = lA[0] + BT * BK;
+    lA[1] = lB[0] + BM * BK;
+    lB[1] = lA[1] + BT * BK;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wr = wave >> 1, wc = wave & 1;
+    // workgroup -> tile: consecutive workgroups walk the T direction first so that the
+    // workgroups sharing a weight tile run at the same time (the weight tile is then served
+    // from L2 for all but the first).
+    const int tiles_t = (T + BT - 1) / BT;
+    const int t0 = (blockIdx.x % tiles_t) * BT, m0 = (blockIdx.x / tiles_t) * BM;
+
+    constexpr int A_LD = BT / 32;                    // 16-byte loads per thread for the A tile
+    constexpr int B_LD = W_U8 ? BM / 64 : BM / 32;   // 16-byte loads per thread for the W tile
+    u32x4 ra[A_LD], rb[B_LD];
+
+    auto load_tiles = [&](int kt) {
+        const int k0 = kt * BK;
+#pragma unroll
+        for (int i = 0; i < A_LD; ++i) {
+            const int row = (tid >> 3) + 32 * i, ch = tid & 7;
+            const int t = min(t0 + row, T - 1);
+            ra[i] = *(const u32x4 *)(A + (size_t)t * lda + k0 + ch * 8);
+        }
+        if (W_U8) {
+#pragma unroll
+            for (int i = 0; i < B_LD; ++i) {
+                const int row = (tid >> 2) + 64 * i, ch = tid & 3;
+                const int m = min(m0 + row, M - 1);
+                rb[i] = __builtin_nontemporal_load((const u32x4 *)((const uint8_t *)Wv + (size_t)m * ldw + k0 + ch * 16));
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < B_LD; ++i) {
+                const int row = (tid >> 3) + 32 * i, ch = tid & 7;
+                const int m = min(m0 + row, M - 1);
+                rb[i] = *(const u32x4 *)((const h16 *)Wv + (size_t)m * ldw + k0 + ch * 8);
+            }
+        }
+    };
+    auto store_tiles = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < A_LD; ++i) {
+            const int row = (tid >> 3) + 32 * i, ch = tid & 7;
+            *(u32x4 *)(lA[buf] + swz(row, ch)) = ra[i];
+        }
+        if (W_U8) {
+            const h16x2 off = {(h16)1023.5f, (h16)1023.5f};
+#pragma unroll
+            for (int i = 0; i < B_LD; ++i) {
+                const int row = (tid >> 2) + 64 * i, ch = tid & 3;
+                u32x4 lo, hi;
+                const uint32_t d[4] = {rb[i].x, rb[i].y, rb[i].z, rb[i].w};
+                uint32_t o[8];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    o[2 * e] = __builtin_bit_cast(uint32_t, u8pair_lo_1024(d[e]) - off);
+                    o[2 * e + 1] = __builtin_bit_cast(uint32_t, u8pair_hi_1024(d[e]) - off);
+                }
+                lo.x = o[0]; lo.y = o[1]; lo.z = o[2]; lo.w = o[3];
+                hi.x = o[4]; hi.y = o[5]; hi.z = o[6]; hi.w = o[7];
+                *(u32x4 *)(lB[buf] + swz(row, 2 * ch)) = lo;
+                *(u32x4 *)(lB[buf] + swz(row, 2 * ch + 1)) = hi;
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < B_LD; ++i) {
+                const int row = (tid >> 3) + 32 * i, ch = tid & 7;
+                *(u32x4 *)(lB[buf] + swz(row, ch)) = rb[i];
+            }
+        }
+    };
+
+    f32x16 acc[MI][NI];
+#pragma unroll
+    for (int a = 0; a < MI; ++a)
+#pragma unroll
+        for (int b = 0; b < NI; ++b)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[a][b][e] = 0.f;
+
+    const int nk = N / BK;
+    load_tiles(0);
+    store_tiles(0);
+    __syncthreads();
+    for (int kt = 0; kt < nk; ++kt) {
+        const int buf = kt & 1;
+        if (kt + 1 < nk) load_tiles(kt + 1);
+#pragma unroll
+        for (int ks = 0; ks < BK / 16; ++ks) {
+            h16x8 fa[MI], fb[NI];
+            const int ch = 2 * ks + (lane >> 5);
+#pragma unroll
+            for (int a = 0; a < MI; ++a) {
+                const int row = wr * (BT / 2) + a * 32 + (lane & 31);
+                fa[a] = *(const h16x8 *)(lA[buf] + swz(row, ch));
+            }
+#pragma unroll
+            for (int b = 0; b < NI; ++b) {
+                const int row = wc * (BM / 2) + b * 32 + (lane & 31);
+                fb[b] = *(const h16x8 *)(lB[buf] + swz(row, ch));
+            }
+#pragma unroll
+            for (int a = 0; a < MI; ++a)
+#pragma unroll
+                for (int b = 0; b < NI; ++b)
+                    acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[a], fb[b], acc[a][b], 0, 0, 0);
+        }
+        if (kt + 1 < nk) store_tiles(buf ^ 1);
+        __syncthreads();
+    }
+
+    // epilogue: lane holds column m = .. + (lane & 31) and rows 8*(e/4) + 4*(lane>>5) + e%4
+#pragma unroll
+    for (int b = 0; b < NI; ++b) {
+        const int m = m0 + wc * (BM / 2) + b * 32 + (lane & 31);
+        if (m >= M) continue;
+        float rxm = 1.f, mxm = 0.f;
+        if (ep.rx) { rxm = h2f(ep.rx[m]); mxm = h2f(ep.mx[m]); }
+#pragma unroll
+        for (int a = 0; a < MI; ++a) {
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const int t = t0 + wr * (BT / 2) + a * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
+                if (t >= T) continue;
+                float v = acc[a][b][e];
+                if (ep.rx) v = rxm * v + mxm * ep.s0[t] + ep.s2[t];
+                if (ep.out_dtype == RWKV_DT_F32) {
+                    ((float *)Y)[(size_t)t * ldy + m] = v;
+                    continue;
+                }
+                float o = round_h(v);
+                switch (ep.act) {
+                    case ACT_SIGMOID: o = sigmoidf_(o); break;
+                    case ACT_RELU_SQ: o = fmaxf(o, 0.f); o = o * o; break;
+                    case ACT_RESIDUAL: o = h2f(ep.res[(size_t)t * ep.ldres + m]) + o; break;
+                    case ACT_GATED_RESIDUAL:
+                        o = round_h(h2f(ep.gate[(size_t)t * ep.ldgate + m]) * o);
+                        o = h2f(ep.res[(size_t)t * ep.ldres + m]) + o;
+                        break;
+                    default: break;
+                }
+                if (ep.out_scale != 1.f) o = round_h(o) * ep.out_scale;
+                ((rwkv_half *)Y)[(size_t)t * ldy + m] = f2h(o);
+            }
+        }
+    }
+}
+
+// xs[t, j] = fp16(x[t, j] * ry[j]);  s0[t] = sum_j x[t, j];  s2[t] = sum_j x[t, j] * my[j].  One wave per row.
+__global__ __launch_bounds__(256) void mm8_prepare_kernel(int T, int N, const rwkv_half *__restrict__ x, int64_t ldx,
+                                                          const rwkv_half *__restrict__ ry,
+                                                          const rwkv_half *__restrict__ my, rwkv_half *__restrict__ xs,
+                                                          float *__restrict__ s0, float *__restrict__ s2) {
+    const int t = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+    if (t >= T) return;
+    float a0 = 0.f, a2 = 0.f;
+    for (int j = lane * 8; j < N; j += 64 * 8) {
+        const u32x4 xv = *(const u32x4 *)(x + (size_t)t * ldx + j);
+        const u32x4 rv = *(const u32x4 *)(ry + j);
+        const u32x4 mv = *(const u32x4 *)(my + j);
+        const h16x8 xh = __builtin_bit_cast(h16x8, xv), rh = __builtin_bit_cast(h16x8, rv),
+                    mh = __builtin_bit_cast(h16x8, mv);
+        h16x8 o;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const float xf = (float)xh[e];
+            o[e] = (h16)(xf * (float)rh[e]);
+            a0 += xf;
+            a2 += xf * (float)mh[e];
+        }
+        *(u32x4 *)(xs + (size_t)t * N + j) = __builtin_bit_cast(u32x4, o);
+    }
+    a0 = wave_sum(a0);
+    a2 = wave_sum(a2);
+    if (lane == 0) { s0[t] = a0; s2[t] = a2; }
+}
+
+
+int gemm_launch(bool w_u8, int64_t T, int64_t N, int64_t M, const rwkv_half *A, int64_t lda, const void *W,
+                int64_t ldw, void *Y, int64_t ldy, const GemmEpi &ep, hipStream_t st) {
+    constexpr int BT = 128, BM = 128;
+    const size_t lds = 2 * (size_t)(BT + BM) * BK * sizeof(h16);
+    const int64_t tiles = ((T + BT - 1) / BT) * ((M + BM - 1) / BM);
+    if (w_u8)
+        hipLaunchKernelGGL((gemm_kernel<true, BT, BM>), dim3((unsigned)tiles), dim3(256), lds, st, (int)T, (int)N,
+                           (int)M, (const h16 *)A, lda, W, ldw, Y, ldy, ep);
+    else
+        hipLaunchKernelGGL((gemm_kernel<false, BT, BM>), dim3((unsigned)tiles), dim3(256), lds, st, (int)T, (int)N,
+                           (int)M, (const h16 *)A, lda, W, ldw, Y, ldy, ep);
+    RWKV_LAUNCH_CHECK();
+    return RWKV_OK;
+}
+
+int mm8_prepare_launch(int64_t T, int64_t N, const rwkv_half *x, int64_t ldx, const rwkv_half *ry,
+                       const rwkv_half *my, rwkv_half *xs, float *s0, float *s2, hipStream_t st) {
+    hipLaunchKernelGGL(mm8_prepare_kernel, dim3((unsigned)((T + 3) / 4)), dim3(256), 0, st, (int)T, (int)N, x, ldx, ry,
+                       my, xs, s0, s2);
+    RWKV_LAUNCH_CHECK();
+    return RWKV_OK;
+}
+
+}  // namespace
+
+int gemv_f16_launch(int64_t N, int64_t M, const rwkv_half *x, const rwkv_half *w, int64_t ldw, void *y,
+                    int y_dtype, hipStream_t st);
+
+extern "C" size_t rwkv_mm8_seq_workspace(int64_t B, int64_t N) {
+    if (B <= 0 || N <= 0) return 0;
+    return (size_t)B * N * 2 + 256 + (size_t)B * 8;
+}
+
+extern "C" int rwkv_mm8_seq_f16(int64_t B, int64_t N, int64_t M, const rwkv_half *x, int64_t x_stride,
+                                const uint8_t *w, int64_t w_stride_n, int64_t w_stride_m, const rwkv_half *mx,
+                                const rwkv_half *rx, const rwkv_half *my, const rwkv_half *ry, rwkv_half *y,
+                                int64_t y_stride, void *workspace, size_t workspace_bytes, void *stream) {
+    if (!x || !w || !mx || !rx || !my || !ry || !y || !workspace) return RWKV_E_NULL;
+    if (B <= 0 || N <= 0 || M <= 0 || (N % BK) != 0 || B > (1 << 24) || M > (1 << 24)) return RWKV_E_SHAPE;
+    if (w_stride_n != 1 || w_stride_m < N || (w_stride_m & 15) || !aligned16(w)) return RWKV_E_LAYOUT;
+    if (x_stride < N || (x_stride & 7) || !aligned16(x) || y_stride < M || !aligned16(my) || !aligned16(ry))
+        return RWKV_E_LAYOUT;
+    if (workspace_bytes < rwkv_mm8_seq_workspace(B, N) || !aligned16(workspace)) return RWKV_E_WORKSPACE;
+    hipStream_t st = (hipStream_t)stream;
+    rwkv_half *xs = (rwkv_half *)workspace;
+    const size_t xs_bytes = ((size_t)B * N * 2 + 255) & ~(size_t)255;
+    float *s0 = (float *)((unsigned char *)workspace + xs_bytes);
+    float *s2 = s0 + B;
+    int rc = mm8_prepare_launch(B, N, x, x_stride, ry, my, xs, s0, s2, st);
+    if (rc) return rc;
+    GemmEpi ep{};
+    ep.mx = mx; ep.rx = rx; ep.s0 = s0; ep.s2 = s2; ep.act = ACT_NONE; ep.out_scale = 1.f; ep.out_dtype = RWKV_DT_F16;
+    return gemm_launch(true, B, N, M, xs, N, w, w_stride_m, y, y_stride, ep, st);
+}
+
+extern "C" int rwkv_gemm_f16(int64_t B, int64_t N, int64_t M, const rwkv_half *a, int64_t a_stride,
+                             const rwkv_half *b, int64_t b_stride_n, int64_t b_stride_m, void *c, int64_t c_stride,
+                             int c_dtype, void *stream) {
+    if (!a || !b || !c) return RWKV_E_NULL;
+    if (B <= 0 || N <= 0 || M <= 0 || (N & 7) || B > (1 << 24) || M > (1 << 24)) return RWKV_E_SHAPE;
+    if (c_dtype != RWKV_DT_F16 && c_dtype != RWKV_DT_F32) return RWKV_E_DTYPE;
+    if (b_stride_n != 1 || b_stride_m < N || (b_stride_m & 7) || !aligned16(b)) return RWKV_E_LAYOUT;
+    if (a_stride < N || (a_stride & 7) || !aligned16(a) || c_stride < M) return RWKV_E_LAYOUT;
+    hipStream_t st = (hipStream_t)stream;
+    if (B == 1) {
+        if (N > 32768) return RWKV_E_SHAPE;
+        return gemv_f16_launch(N, M, a, b, b_stride_m, c, c_dtype, st);
+    }
+    if (N % BK) return RWKV_E_SHAPE;
+    GemmEpi ep{};
+    ep.act = ACT_NONE; ep.out_scale = 1.f; ep.out_dtype = c_dtype;
+    return gemm_launch(false, B, N, M, a, a_stride, b, b_stride_m, c, c_stride, ep, st);
+}

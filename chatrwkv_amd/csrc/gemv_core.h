@@ -1,0 +1,123 @@
+// Streaming GEMV building blocks for gfx950.
+//
+// Weight matrices are read in the input-contiguous layout: output row m is N consecutive
+// elements (uint8 or fp16).  One wave owns a few output rows; lane l reads the 16-byte
+// segments l, l+64, ... of each row (a wave reads 1 KiB contiguous per row per step), multiplies
+// with the activation vector held in LDS and reduces across the wave with shuffles.  Nothing
+// is shared between waves, so there are no atomics and results are deterministic.
+//
+// uint8 path: y[m] = rx[m] * sum_j xs[j] * (w[m][j] + 0.5) + mx[m] * S0 + S2 with
+//   xs[j] = fp16(x[j] * ry[j]),  S0 = sum x[j],  S2 = sum x[j] * my[j].
+// Bytes are widened two at a time to the fp16 values (1024 + b) with one v_perm_b32 and fed to
+// v_dot2_f32_f16 (fp32 accumulate); the 1024 offset is removed afterwards with S1 = sum xs[j]:
+//   sum xs[j] * (w + 0.5) = dot - 1023.5 * S1.
+#pragma once
+#include "common.h"
+
+// LDS layout of an activation vector of nseg = N/16 segments: the first 8 values of every
+// segment are stored as 16-byte items [0, nseg), the last 8 as items [nseg, 2*nseg), so that
+// the two ds_read_b128 of consecutive lanes hit consecutive 16-byte slots (conflict free).
+DEV int xs_slot(int j, int nseg) {
+    const int s = j >> 4, p = j & 15;
+    return ((p >> 3) * nseg + s) * 8 + (p & 7);
+}
+
+struct VecSums {
+    float s0, s1, s2;
+};
+
+// dot of 16 uint8 weights (as 1024 + b) with 16 fp16 activations.
+DEV float dot16_u8(u32x4 w, h16x8 x0, h16x8 x1, float acc) {
+    acc = __builtin_amdgcn_fdot2(u8pair_lo_1024(w.x), __builtin_shufflevector(x0, x0, 0, 1), acc, false);
+    acc = __builtin_amdgcn_fdot2(u8pair_hi_1024(w.x), __builtin_shufflevector(x0, x0, 2, 3), acc, false);
+    acc = __builtin_amdgcn_fdot2(u8pair_lo_1024(w.y), __builtin_shufflevector(x0, x0, 4, 5), acc, false);
+    acc = __builtin_amdgcn_fdot2(u8pair_hi_1024(w.y), __builtin_shufflevector(x0, x0, 6, 7), acc, false);
+    acc = __builtin_amdgcn_fdot2(u8pair_lo_1024(w.z), __builtin_shufflevector(x1, x1, 0, 1), acc, false);
+    acc = __builtin_amdgcn_fdot2(u8pair_hi_1024(w.z), __builtin_shufflevector(x1, x1, 2, 3), acc, false);
+    acc = __builtin_amdgcn_fdot2(u8pair_lo_1024(w.w), __builtin_shufflevector(x1, x1, 4, 5), acc, false);
+    acc = __builtin_amdgcn_fdot2(u8pair_hi_1024(w.w), __builtin_shufflevector(x1, x1, 6, 7), acc, false);
+    return acc;
+}
+
+// dot of 8 fp16 weights with 8 fp16 activations.
+DEV float dot8_f16(u32x4 w, h16x8 x, float acc) {
+    const h16x8 wh = __builtin_bit_cast(h16x8, w);
+    acc = __builtin_amdgcn_fdot2(__builtin_shufflevector(wh, wh, 0, 1), __builtin_shufflevector(x, x, 0, 1), acc, false);
+    acc = __builtin_amdgcn_fdot2(__builtin_shufflevector(wh, wh, 2, 3), __builtin_shufflevector(x, x, 2, 3), acc, false);
+    acc = __builtin_amdgcn_fdot2(__builtin_shufflevector(wh, wh, 4, 5), __builtin_shufflevector(x, x, 4, 5), acc, false);
+    acc = __builtin_amdgcn_fdot2(__builtin_shufflevector(wh, wh, 6, 7), __builtin_shufflevector(x, x, 6, 7), acc, false);
+    return acc;
+}
+
+// One wave: acc[r] += <row r, xs> for R rows, every lane ends with the full sums.
+// u8: rows are N bytes, xs in the split LDS layout above (nseg = N/16).
+// U = number of 16-byte segments per lane loaded before any is consumed (loads in flight = R*U).
+template <int R, int U>
+DEV void wave_rows_dot_u8(const uint8_t *const (&rows)[R], const h16 *xs, int nseg, float (&acc)[R]) {
+    const int lane = threadIdx.x & 63;
+    const h16x8 *xlo = (const h16x8 *)xs;
+    const h16x8 *xhi = xlo + nseg;
+    int s = lane;
+    // full batches: all 64 lanes have U segments
+    for (; s + 64 * (U - 1) < nseg; s += 64 * U) {
+        u32x4 wv[U][R];
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+                wv[u][r] = __builtin_nontemporal_load((const u32x4 *)(rows[r] + 16 * (size_t)(s + 64 * u)));
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const h16x8 x0 = xlo[s + 64 * u], x1 = xhi[s + 64 * u];
+#pragma unroll
+            for (int r = 0; r < R; ++r) acc[r] = dot16_u8(wv[u][r], x0, x1, acc[r]);
+        }
+    }
+    for (; s < nseg; s += 64) {
+        const h16x8 x0 = xlo[s], x1 = xhi[s];
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            u32x4 wv = __builtin_nontemporal_load((const u32x4 *)(rows[r] + 16 * (size_t)s));
+            acc[r] = dot16_u8(wv, x0, x1, acc[r]);
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) acc[r] = wave_sum(acc[r]);
+}
+
+// fp16 rows: N halves per row, xs stored linearly in LDS; segments are 8 values (16 bytes).
+template <int R, int U>
+DEV void wave_rows_dot_f16(const h16 *const (&rows)[R], const h16 *xs, int nseg8, float (&acc)[R]) {
+    const int lane = threadIdx.x & 63;
+    const h16x8 *xv = (const h16x8 *)xs;
+    int s = lane;
+    for (; s + 64 * (U - 1) < nseg8; s += 64 * U) {
+        u32x4 wv[U][R];
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+                wv[u][r] = __builtin_nontemporal_load((const u32x4 *)(rows[r] + 8 * (size_t)(s + 64 * u)));
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const h16x8 x = xv[s + 64 * u];
+#pragma unroll
+            for (int r = 0; r < R; ++r) acc[r] = dot8_f16(wv[u][r], x, acc[r]);
+        }
+    }
+    for (; s < nseg8; s += 64) {
+        const h16x8 x = xv[s];
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            u32x4 wv = __builtin_nontemporal_load((const u32x4 *)(rows[r] + 8 * (size_t)s));
+            acc[r] = dot8_f16(wv, x, acc[r]);
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) acc[r] = wave_sum(acc[r]);
+}
+
+// Final value of a uint8 row from its raw dot product.
+DEV float mm8_finish(float dot, const VecSums &S, float rx, float mx) {
+    return rx * (dot - 1023.5f * S.s1) + mx * S.s0 + S.s2;
+}

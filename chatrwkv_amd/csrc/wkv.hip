@@ -1,0 +1,210 @@
+// WKV recurrences: RWKV-4 (per channel, running-maximum form) and RWKV-5/6 (per-head 64x64 state).
+#include "common.h"
+
+namespace {
+
+// ---------------------------------------------------------------------------------------
+// RWKV-4.  One lane per channel, fp32 state in registers for the whole T loop; a wave reads
+// 64 consecutive channels of a token (coalesced).  k/v for the next UNR tokens are loaded
+// before the dependent chain of exp/div consumes them, so memory latency is off the
+// critical path.  One wave per workgroup spreads the C/64 waves over as many CUs as possible.
+//   MODE 0: k, v, y fp32 (operator-level interface)
+//   MODE 1: k, v fp16; y = fp16(r * fp16(wkv)) with r fp16 (already sigmoid'ed), fp16 out
+// ---------------------------------------------------------------------------------------
+template <int MODE> struct Wkv4IO;
+template <> struct Wkv4IO<0> {
+    const float *k, *v; float *y; const rwkv_half *r;
+    DEV float ldk(size_t i) const { return k[i]; }
+    DEV float ldv(size_t i) const { return v[i]; }
+    DEV float ldr(size_t) const { return 1.f; }
+    DEV void st(size_t i, float wkv, float) const { y[i] = wkv; }
+};
+template <> struct Wkv4IO<1> {
+    const rwkv_half *k, *v; rwkv_half *y; const rwkv_half *r;
+    DEV float ldk(size_t i) const { return h2f(k[i]); }
+    DEV float ldv(size_t i) const { return h2f(v[i]); }
+    DEV float ldr(size_t i) const { return h2f(r[i]); }
+    DEV void st(size_t i, float wkv, float rr) const { y[i] = f2h(rr * round_h(wkv)); }
+};
+
+DEV void wkv4_step(float kk, float vv, float u, float w, float &aa, float &bb, float &pp, float &out) {
+    float ww = u + kk;
+    float p = fmaxf(pp, ww);
+    float e1 = __expf(pp - p), e2 = __expf(ww - p);
+    out = (e1 * aa + e2 * vv) / (e1 * bb + e2);
+    ww = w + pp;
+    p = fmaxf(ww, kk);
+    e1 = __expf(ww - p);
+    e2 = __expf(kk - p);
+    aa = e1 * aa + e2 * vv;
+    bb = e1 * bb + e2;
+    pp = p;
+}
+
+template <int MODE>
+__global__ __launch_bounds__(64) void wkv4_kernel(int T, int C, const float *__restrict__ w_, const float *__restrict__ u_,
+                                                  Wkv4IO<MODE> io, float *__restrict__ aa_, float *__restrict__ bb_,
+                                                  float *__restrict__ pp_) {
+    constexpr int UNR = 8;
+    const int c = blockIdx.x * 64 + threadIdx.x;
+    const int b = blockIdx.y;
+    if (c >= C) return;
+    const size_t base = (size_t)b * T * C + c;
+    const int so = b * C + c;
+    const float u = u_[c], w = w_[c];
+    float aa = aa_[so], bb = bb_[so], pp = pp_[so];
+    int t = 0;
+    for (; t + UNR <= T; t += UNR) {
+        float kk[UNR], vv[UNR], rr[UNR];
+#pragma unroll
+        for (int i = 0; i < UNR; ++i) {
+            const size_t o = base + (size_t)(t + i) * C;
+            kk[i] = io.ldk(o); vv[i] = io.ldv(o); rr[i] = io.ldr(o);
+        }
+#pragma unroll
+        for (int i = 0; i < UNR; ++i) {
+            float out;
+            wkv4_step(kk[i], vv[i], u, w, aa, bb, pp, out);
+            io.st(base + (size_t)(t + i) * C, out, rr[i]);
+        }
+    }
+    for (; t < T; ++t) {
+        const size_t o = base + (size_t)t * C;
+        float out;
+        const float rr = io.ldr(o);
+        wkv4_step(io.ldk(o), io.ldv(o), u, w, aa, bb, pp, out);
+        io.st(o, out, rr);
+    }
+    aa_[so] = aa; bb_[so] = bb; pp_[so] = pp;
+}
+
+// ---------------------------------------------------------------------------------------
+// RWKV-5 / RWKV-6.  One workgroup of 256 threads per head (N = 64).  Thread (i, q), i = value
+// index 0..63, q = key quarter 0..3, keeps S[i][16q .. 16q+16) in registers for the whole call.
+// Tokens are processed in slabs of TS: r, k, v, w of the slab are staged in LDS once (one
+// barrier), every thread runs the TS steps on its slice reading r/k/w as wave-uniform LDS
+// broadcasts, writes its partial y to LDS, and after a second barrier the four quarters are
+// summed and stored coalesced.  PER_TOKEN_W: RWKV-6 (w[t][c]); otherwise RWKV-5 (w[c]).
+//   y_i = sum_j r_j (u_j k_j v_i + S_ij) ;  S_ij = S_ij w_j + k_j v_i
+// ---------------------------------------------------------------------------------------
+constexpr int HS = 64;   // head size
+constexpr int TS = 16;   // tokens per slab
+
+template <bool PER_TOKEN_W>
+__global__ __launch_bounds__(256) void wkv56_kernel(int T, int C, float *__restrict__ state, int state_layout,
+                                                    const float *__restrict__ r_, const float *__restrict__ k_,
+                                                    const float *__restrict__ v_, const float *__restrict__ w_,
+                                                    const float *__restrict__ u_, float *__restrict__ y_) {
+    __shared__ __align__(16) float sr[TS][HS], sk[TS][HS], sv[TS][HS], sw[TS][HS];
+    __shared__ __align__(16) float su[HS];
+    __shared__ float part[TS][4][HS];
+    const int h = blockIdx.x;
+    const int i = threadIdx.x & 63, q = threadIdx.x >> 6;
+    float *S = state + (size_t)h * HS * HS;
+    float s[16];
+#pragma unroll
+    for (int jj = 0; jj < 16; ++jj) {
+        const int j = 16 * q + jj;
+        s[jj] = state_layout == 0 ? S[i * HS + j] : S[j * HS + i];
+    }
+    if (threadIdx.x < HS) {
+        su[threadIdx.x] = u_[h * HS + threadIdx.x];
+        if (!PER_TOKEN_W) sw[0][threadIdx.x] = w_[h * HS + threadIdx.x];
+    }
+    for (int t0 = 0; t0 < T; t0 += TS) {
+        const int nt = min(TS, T - t0);
+        __syncthreads();  // previous slab fully consumed (and su / sw[0] visible)
+        for (int e = threadIdx.x; e < nt * HS; e += 256) {
+            const int tt = e >> 6, c = e & 63;
+            const size_t o = (size_t)(t0 + tt) * C + h * HS + c;
+            sr[tt][c] = r_[o]; sk[tt][c] = k_[o]; sv[tt][c] = v_[o];
+            if (PER_TOKEN_W) sw[tt][c] = w_[o];
+        }
+        __syncthreads();
+        for (int tt = 0; tt < nt; ++tt) {
+            const float vi = sv[tt][i];
+            const float *wrow = PER_TOKEN_W ? sw[tt] : sw[0];
+            float y = 0.f;
+#pragma unroll
+            for (int jj = 0; jj < 16; jj += 4) {
+                const int j = 16 * q + jj;
+                const f32x4 r4 = *(const f32x4 *)&sr[tt][j];
+                const f32x4 k4 = *(const f32x4 *)&sk[tt][j];
+                const f32x4 w4 = *(const f32x4 *)&wrow[j];
+                const f32x4 u4 = *(const f32x4 *)&su[j];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const float x = k4[e] * vi;
+                    y += r4[e] * (u4[e] * x + s[jj + e]);
+                    s[jj + e] = s[jj + e] * w4[e] + x;
+                }
+            }
+            part[tt][q][i] = y;
+        }
+        __syncthreads();
+        for (int e = threadIdx.x; e < nt * HS; e += 256) {
+            const int tt = e >> 6, c = e & 63;
+            y_[(size_t)(t0 + tt) * C + h * HS + c] = (part[tt][0][c] + part[tt][1][c]) + (part[tt][2][c] + part[tt][3][c]);
+        }
+    }
+#pragma unroll
+    for (int jj = 0; jj < 16; ++jj) {
+        const int j = 16 * q + jj;
+        if (state_layout == 0) S[i * HS + j] = s[jj]; else S[j * HS + i] = s[jj];
+    }
+}
+
+}  // namespace
+
+extern "C" int rwkv_wkv4_forward(int64_t B, int64_t T, int64_t C, const float *w, const float *u, const void *k,
+                                 const void *v, void *y, int kv_dtype, float *aa, float *bb, float *pp,
+                                 void *stream) {
+    if (!w || !u || !k || !v || !y || !aa || !bb || !pp) return RWKV_E_NULL;
+    if (B <= 0 || T <= 0 || C <= 0 || B > 65535 || B * T * C > ((int64_t)1 << 40)) return RWKV_E_SHAPE;
+    dim3 grid((unsigned)((C + 63) / 64), (unsigned)B);
+    if (kv_dtype == RWKV_DT_F32) {
+        Wkv4IO<0> io{(const float *)k, (const float *)v, (float *)y, nullptr};
+        hipLaunchKernelGGL(wkv4_kernel<0>, grid, dim3(64), 0, (hipStream_t)stream, (int)T, (int)C, w, u, io, aa, bb, pp);
+    } else {
+        return RWKV_E_DTYPE;
+    }
+    RWKV_LAUNCH_CHECK();
+    return RWKV_OK;
+}
+
+// fused variant used by the model path: fp16 k, v, r in; y = fp16(r * fp16(wkv)).
+int wkv4_fused_launch(int T, int C, const float *w, const float *u, const rwkv_half *k, const rwkv_half *v,
+                      const rwkv_half *r, rwkv_half *y, float *aa, float *bb, float *pp, hipStream_t st) {
+    Wkv4IO<1> io{k, v, y, r};
+    hipLaunchKernelGGL(wkv4_kernel<1>, dim3((unsigned)((C + 63) / 64), 1), dim3(64), 0, st, T, C, w, u, io, aa, bb, pp);
+    RWKV_LAUNCH_CHECK();
+    return RWKV_OK;
+}
+
+static int wkv56_launch(bool v6, int64_t B, int64_t T, int64_t C, int64_t H, float *state, int state_layout,
+                        const float *r, const float *k, const float *v, const float *w, const float *u, float *y,
+                        void *stream) {
+    if (!state || !r || !k || !v || !w || !u || !y) return RWKV_E_NULL;
+    if (B != 1 || T <= 0 || H <= 0 || C != H * HS) return RWKV_E_SHAPE;
+    if (state_layout != 0 && state_layout != 1) return RWKV_E_DTYPE;
+    if (v6)
+        hipLaunchKernelGGL(wkv56_kernel<true>, dim3((unsigned)H), dim3(256), 0, (hipStream_t)stream, (int)T, (int)C,
+                           state, state_layout, r, k, v, w, u, y);
+    else
+        hipLaunchKernelGGL(wkv56_kernel<false>, dim3((unsigned)H), dim3(256), 0, (hipStream_t)stream, (int)T, (int)C,
+                           state, state_layout, r, k, v, w, u, y);
+    RWKV_LAUNCH_CHECK();
+    return RWKV_OK;
+}
+
+extern "C" int rwkv_wkv5_forward(int64_t B, int64_t T, int64_t C, int64_t H, float *state, int state_layout,
+                                 const float *r, const float *k, const float *v, const float *w, const float *u,
+                                 float *y, void *stream) {
+    return wkv56_launch(false, B, T, C, H, state, state_layout, r, k, v, w, u, y, stream);
+}
+
+extern "C" int rwkv_wkv6_forward(int64_t B, int64_t T, int64_t C, int64_t H, float *state, int state_layout,
+                                 const float *r, const float *k, const float *v, const float *w, const float *u,
+                                 float *y, void *stream) {
+    return wkv56_launch(true, B, T, C, H, state, state_layout, r, k, v, w, u, y, stream);
+}

@@ -1,0 +1,70 @@
+"""ctypes binding of librwkv_hip.so (declared in include/rwkv_hip.h).
+
+The library is built in-tree by ``python -m chatrwkv_amd.build`` (hipcc, gfx950) and is the
+only compute path of this package: if it is missing, or a call is rejected, an exception is
+raised -- there is no fallback.
+"""
+import ctypes
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "librwkv_hip.so")
+
+RWKV_DT_F16, RWKV_DT_F32 = 0, 1
+
+_ERR = {
+    -1: "RWKV_E_SHAPE: size not supported by the kernel",
+    -2: "RWKV_E_LAYOUT: stride / alignment not supported",
+    -3: "RWKV_E_NULL: required pointer is NULL",
+    -4: "RWKV_E_WORKSPACE: workspace too small or misaligned",
+    -5: "RWKV_E_DTYPE: unknown dtype / mode code",
+}
+
+_i64, _int, _vp, _sz = ctypes.c_int64, ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t
+
+# name -> (restype, argtypes); mirrors include/rwkv_hip.h
+SIGNATURES = {
+    "rwkv_abi_version": (_int, []),
+    "rwkv_quantize_u8": (_int, [_i64, _i64, _vp, _i64, _i64, _vp, _i64, _i64, _vp, _vp, _vp, _vp, _int, _vp, _sz, _vp]),
+    "rwkv_repack_u8": (_int, [_i64, _i64, _vp, _i64, _i64, _vp, _i64, _i64, _vp]),
+    "rwkv_repack_f16": (_int, [_i64, _i64, _vp, _i64, _i64, _vp, _i64, _i64, _vp]),
+    "rwkv_mm8_one_f16": (_int, [_i64, _i64, _vp, _vp, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _int, _vp]),
+    "rwkv_mm8_seq_workspace": (_sz, [_i64, _i64]),
+    "rwkv_mm8_seq_f16": (_int, [_i64, _i64, _i64, _vp, _i64, _vp, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _i64, _vp, _sz, _vp]),
+    "rwkv_gemm_f16": (_int, [_i64, _i64, _i64, _vp, _i64, _vp, _i64, _i64, _vp, _i64, _int, _vp]),
+    "rwkv_wkv4_forward": (_int, [_i64, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _int, _vp, _vp, _vp, _vp]),
+    "rwkv_wkv5_forward": (_int, [_i64, _i64, _i64, _i64, _vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "rwkv_wkv6_forward": (_int, [_i64, _i64, _i64, _i64, _vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
+}
+
+_lib = None
+
+
+class RwkvHipError(RuntimeError):
+    pass
+
+
+def load():
+    """Load the shared library (once) and declare every entry point."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RwkvHipError(
+            f"{LIB_PATH} not found: build it with `python -m chatrwkv_amd.build` "
+            "(hipcc --offload-arch=gfx950). This package has no CPU or PyTorch fallback.")
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    _lib = lib
+    return lib
+
+
+def check(rc, what):
+    if rc == 0:
+        return
+    if rc < 0:
+        raise RwkvHipError(f"{what}: {_ERR.get(rc, rc)}")
+    raise RwkvHipError(f"{what}: HIP error {rc}")

@@ -1,0 +1,129 @@
+/*
+ * librwkv_hip.so -- C ABI of the MI355X (gfx950) kernels behind
+ * RWKV(model, 'cuda fp16i8' | 'cuda fp16').forward(tokens, state).
+ *
+ * Conventions
+ *   - Every pointer is a device pointer unless said otherwise; the library never
+ *     allocates or frees device memory: the caller owns inputs, outputs and workspaces.
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream).  Calls only
+ *     enqueue work; they never synchronise.
+ *   - Return value: 0 = enqueued; < 0 = rejected argument (RWKV_E_*); > 0 = hipError_t of
+ *     the failed launch.  Nothing is enqueued when the value is non-zero.
+ *   - fp16 values are IEEE binary16 passed as `rwkv_half` (uint16_t storage).
+ *   - A weight matrix is the reference's logical [N(in), M(out)] matrix
+ *     (rwkv_pip_package/src/rwkv/model.py:793-794) addressed as
+ *     w[n * w_stride_n + m * w_stride_m].  The fast layout is "input-contiguous":
+ *     w_stride_n == 1, w_stride_m >= N (the orientation checkpoints are stored in);
+ *     N % 16 == 0, w_stride_m % 16 == 0 and 16-byte aligned base pointers are required.
+ *     The reference's device layout (w_stride_m == 1) is accepted by
+ *     rwkv_repack_u8 / rwkv_repack_f16, which transpose it once at load time.
+ *   - mx, rx are per output column [M]; my, ry per input row [N]; rx and ry are the
+ *     stored ones (already divided by 16, model.py:845-847), so
+ *     W'[n,m] = (w[n,m] + 0.5) * ry[n] * rx[m] + my[n] + mx[m]   (model.py:93).
+ */
+#ifndef RWKV_HIP_H
+#define RWKV_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef uint16_t rwkv_half;
+
+#define RWKV_OK 0
+#define RWKV_E_SHAPE (-1)     /* size not supported (zero, negative, not a multiple the kernel needs) */
+#define RWKV_E_LAYOUT (-2)    /* stride / alignment not supported */
+#define RWKV_E_NULL (-3)      /* required pointer is NULL */
+#define RWKV_E_WORKSPACE (-4) /* workspace too small */
+#define RWKV_E_DTYPE (-5)     /* unknown dtype / mode code */
+
+#define RWKV_DT_F16 0
+#define RWKV_DT_F32 1
+
+/* Library / device identification.  Returns the ABI version (currently 1). */
+int rwkv_abi_version(void);
+
+/* ---------------------------------------------------------------------------------------
+ * uint8 quantizer.  Replaces the CPU routine in RWKV.__init__ (model.py:818-847); results
+ * are bit-identical to it.  `w` is the fp32 logical [N, M] matrix after transposition and
+ * rescale (model.py:785-794), addressed with the two strides (elements); it is not
+ * modified.  Outputs: q uint8 with strides (q_stride_n, q_stride_m); mx, rx [M] and my, ry
+ * [N] in `scale_dtype` (RWKV_DT_F16 / RWKV_DT_F32); rx, ry are stored divided by 16.
+ * Branch on N > M as model.py:824.  workspace: 4 * (N + M) floats.
+ */
+int rwkv_quantize_u8(int64_t N, int64_t M,
+                     const float *w, int64_t w_stride_n, int64_t w_stride_m,
+                     uint8_t *q, int64_t q_stride_n, int64_t q_stride_m,
+                     void *mx, void *rx, void *my, void *ry, int scale_dtype,
+                     float *workspace, size_t workspace_bytes, void *stream);
+
+/* Transposes between the reference's device layout and the input-contiguous layout:
+ * dst[n * dst_stride_n + m * dst_stride_m] = src[n * src_stride_n + m * src_stride_m]. */
+int rwkv_repack_u8(int64_t N, int64_t M, const uint8_t *src, int64_t src_stride_n, int64_t src_stride_m,
+                   uint8_t *dst, int64_t dst_stride_n, int64_t dst_stride_m, void *stream);
+int rwkv_repack_f16(int64_t N, int64_t M, const rwkv_half *src, int64_t src_stride_n, int64_t src_stride_m,
+                    rwkv_half *dst, int64_t dst_stride_n, int64_t dst_stride_m, void *stream);
+
+/* ---------------------------------------------------------------------------------------
+ * mm8_one: y[M] = x[N] @ W'.  Replaces torch.ops.rwkv.mm8_one (cuda/wrapper.cpp:84-117,
+ * cuda/operators.cu:207-246) and the Python wrapper cuda_mm8_one (model.py:75-86).
+ * fp32 accumulation.  y is written (not accumulated into: no pre-zeroing needed) as fp32
+ * (y_dtype RWKV_DT_F32, the kernel's raw sum) or rounded to fp16 (RWKV_DT_F16, what
+ * model.py:86 returns).  Deterministic: no atomics.
+ */
+int rwkv_mm8_one_f16(int64_t N, int64_t M, const rwkv_half *x,
+                     const uint8_t *w, int64_t w_stride_n, int64_t w_stride_m,
+                     const rwkv_half *mx, const rwkv_half *rx, const rwkv_half *my, const rwkv_half *ry,
+                     void *y, int y_dtype, void *stream);
+
+/* mm8_seq: y[B, M] = x[B, N] @ W', fp16 in, fp32 accumulation on MFMA, fp16 out.
+ * Replaces torch.ops.rwkv.mm8_seq (cuda/wrapper.cpp:50-83, cuda/operators.cu:116-154).
+ * x rows at x_stride elements, y rows at y_stride.  workspace: rwkv_mm8_seq_workspace(B, N)
+ * bytes (the ry-scaled copy of x and two per-row sums). */
+size_t rwkv_mm8_seq_workspace(int64_t B, int64_t N);
+int rwkv_mm8_seq_f16(int64_t B, int64_t N, int64_t M, const rwkv_half *x, int64_t x_stride,
+                     const uint8_t *w, int64_t w_stride_n, int64_t w_stride_m,
+                     const rwkv_half *mx, const rwkv_half *rx, const rwkv_half *my, const rwkv_half *ry,
+                     rwkv_half *y, int64_t y_stride, void *workspace, size_t workspace_bytes, void *stream);
+
+/* gemm_fp16: c[B, M] = a[B, N] @ b[N, M], fp16 operands, fp32 accumulation, c written
+ * directly as fp16 or fp32 (c_dtype) with no intermediate fp16 rounding.  Replaces
+ * torch.ops.rwkv.gemm_fp16_cublas (cuda/gemm_fp16_cublas.cpp:28-75) for 2-D operands;
+ * B == 1 takes the streaming GEMV path. */
+int rwkv_gemm_f16(int64_t B, int64_t N, int64_t M, const rwkv_half *a, int64_t a_stride,
+                  const rwkv_half *b, int64_t b_stride_n, int64_t b_stride_m,
+                  void *c, int64_t c_stride, int c_dtype, void *stream);
+
+/* ---------------------------------------------------------------------------------------
+ * wkv_forward: RWKV-4 WKV recurrence over T tokens with running-maximum tracking.
+ * Replaces torch.ops.rwkv.wkv_forward (cuda/wrapper.cpp:27-48, cuda/operators.cu:11-58).
+ * w = time_decay (-exp(raw)), u = time_first, fp32 [C]; k, v, y [B*T, C] in `kv_dtype`
+ * (fp32 is what model.py:1355-1357 passes); aa, bb, pp fp32 [B*C] updated in place.
+ */
+int rwkv_wkv4_forward(int64_t B, int64_t T, int64_t C, const float *w, const float *u,
+                      const void *k, const void *v, void *y, int kv_dtype,
+                      float *aa, float *bb, float *pp, void *stream);
+
+/* RWKV-5 (constant per-channel decay) and RWKV-6 (per-token decay) recurrences on the
+ * per-head N x N state, fp32.  Replace rwkv5.forward_fp32 / rwkv6.forward_fp32
+ * (cuda/rwkv5_op.cpp:20-23 + cuda/rwkv5.cu:8-88; cuda/rwkv6_op.cpp:20-23 +
+ * cuda/rwkv6.cu:8-87).  r, k, v, y: [T, C]; u: [C]; head size N = C / H must be 64.
+ * w: v5 [C] (decay in (0,1)); v6 [T, C] *after* exp(-exp(.)) (model.py:959).
+ * state_layout 0: [H][value i][key j] (what the reference kernels take, model.py:1376, 1429);
+ * state_layout 1: [H][key j][value i] (the layout of the state list, model.py:1470).
+ * state is updated in place.  B must be 1 (cuda/rwkv6.cu:17).
+ */
+int rwkv_wkv5_forward(int64_t B, int64_t T, int64_t C, int64_t H, float *state, int state_layout,
+                      const float *r, const float *k, const float *v, const float *w, const float *u,
+                      float *y, void *stream);
+int rwkv_wkv6_forward(int64_t B, int64_t T, int64_t C, int64_t H, float *state, int state_layout,
+                      const float *r, const float *k, const float *v, const float *w, const float *u,
+                      float *y, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* RWKV_HIP_H */
