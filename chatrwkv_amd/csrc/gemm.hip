@@ -11,23 +11,11 @@
 // Tiling: BT x BM outputs per workgroup of 256 threads (2 x 2 waves), K step 64, LDS double
 // buffered; both LDS tiles are [row][64 halves] with the eight 16-byte chunks of a row XOR-
 // swizzled by (row & 7) so that the ds_read_b128 of 32 consecutive rows spreads over all banks.
-#include "common.h"
+#include "kernels.h"
 
 namespace {
 
 constexpr int BK = 64;  // halves per LDS row
-
-enum { ACT_NONE = 0, ACT_SIGMOID = 1, ACT_RELU_SQ = 2, ACT_RESIDUAL = 3, ACT_GATED_RESIDUAL = 4 };
-
-struct GemmEpi {
-    const rwkv_half *mx, *rx;      // [M]; NULL for plain fp16 weights
-    const float *s0, *s2;          // [T]
-    int act;
-    const rwkv_half *res; int64_t ldres;   // residual input [T, M]
-    const rwkv_half *gate; int64_t ldgate; // gate [T, M]
-    float out_scale;               // applied to the final fp16 value (1 or 0.5)
-    int out_dtype;                 // RWKV_DT_F16 / RWKV_DT_F32 (F32 only with ACT_NONE: raw accumulator)
-};
 
 DEV int swz(int row, int chunk) { return row * BK + ((chunk ^ (row & 7)) << 3); }
 
@@ -167,7 +155,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(int T, int N, int M, const h1
                 if (t >= T) continue;
                 float v = acc[a][b][e];
                 if (ep.rx) v = rxm * v + mxm * ep.s0[t] + ep.s2[t];
-                if (ep.out_dtype == RWKV_DT_F32) {
+                if (ep.raw_f32) {
                     ((float *)Y)[(size_t)t * ldy + m] = v;
                     continue;
                 }
@@ -183,7 +171,10 @@ __global__ __launch_bounds__(256) void gemm_kernel(int T, int N, int M, const h1
                     default: break;
                 }
                 if (ep.out_scale != 1.f) o = round_h(o) * ep.out_scale;
-                ((rwkv_half *)Y)[(size_t)t * ldy + m] = f2h(o);
+                if (ep.out_dtype == RWKV_DT_F32)
+                    ((float *)Y)[(size_t)t * ldy + m] = round_h(o);
+                else
+                    ((rwkv_half *)Y)[(size_t)t * ldy + m] = f2h(o);
             }
         }
     }
@@ -219,6 +210,8 @@ __global__ __launch_bounds__(256) void mm8_prepare_kernel(int T, int N, const rw
 }
 
 
+}  // namespace
+
 int gemm_launch(bool w_u8, int64_t T, int64_t N, int64_t M, const rwkv_half *A, int64_t lda, const void *W,
                 int64_t ldw, void *Y, int64_t ldy, const GemmEpi &ep, hipStream_t st) {
     constexpr int BT = 128, BM = 128;
@@ -242,10 +235,6 @@ int mm8_prepare_launch(int64_t T, int64_t N, const rwkv_half *x, int64_t ldx, co
     return RWKV_OK;
 }
 
-}  // namespace
-
-int gemv_f16_launch(int64_t N, int64_t M, const rwkv_half *x, const rwkv_half *w, int64_t ldw, void *y,
-                    int y_dtype, hipStream_t st);
 
 extern "C" size_t rwkv_mm8_seq_workspace(int64_t B, int64_t N) {
     if (B <= 0 || N <= 0) return 0;
@@ -289,6 +278,6 @@ extern "C" int rwkv_gemm_f16(int64_t B, int64_t N, int64_t M, const rwkv_half *a
     }
     if (N % BK) return RWKV_E_SHAPE;
     GemmEpi ep{};
-    ep.act = ACT_NONE; ep.out_scale = 1.f; ep.out_dtype = c_dtype;
+    ep.act = ACT_NONE; ep.out_scale = 1.f; ep.out_dtype = c_dtype; ep.raw_f32 = (c_dtype == RWKV_DT_F32);
     return gemm_launch(false, B, N, M, a, a_stride, b, b_stride_m, c, c_stride, ep, st);
 }

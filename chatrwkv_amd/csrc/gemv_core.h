@@ -49,14 +49,13 @@ DEV float dot8_f16(u32x4 w, h16x8 x, float acc) {
     return acc;
 }
 
-// One wave: acc[r] += <row r, xs> for R rows, every lane ends with the full sums.
-// u8: rows are N bytes, xs in the split LDS layout above (nseg = N/16).
+// One wave: acc[r] += <row r, xs[r]> for R rows, every lane ends with the full sums.
+// u8: rows are N bytes, xs[r] in the split LDS layout above (nseg = N/16); rows may share one
+// activation vector (pass the same pointer: the LDS reads are then common) or have one each.
 // U = number of 16-byte segments per lane loaded before any is consumed (loads in flight = R*U).
 template <int R, int U>
-DEV void wave_rows_dot_u8(const uint8_t *const (&rows)[R], const h16 *xs, int nseg, float (&acc)[R]) {
+DEV void wave_rows_dot_u8(const uint8_t *const (&rows)[R], const h16 *const (&xs)[R], int nseg, float (&acc)[R]) {
     const int lane = threadIdx.x & 63;
-    const h16x8 *xlo = (const h16x8 *)xs;
-    const h16x8 *xhi = xlo + nseg;
     int s = lane;
     // full batches: all 64 lanes have U segments
     for (; s + 64 * (U - 1) < nseg; s += 64 * U) {
@@ -68,15 +67,19 @@ DEV void wave_rows_dot_u8(const uint8_t *const (&rows)[R], const h16 *xs, int ns
                 wv[u][r] = __builtin_nontemporal_load((const u32x4 *)(rows[r] + 16 * (size_t)(s + 64 * u)));
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            const h16x8 x0 = xlo[s + 64 * u], x1 = xhi[s + 64 * u];
 #pragma unroll
-            for (int r = 0; r < R; ++r) acc[r] = dot16_u8(wv[u][r], x0, x1, acc[r]);
+            for (int r = 0; r < R; ++r) {
+                const h16x8 *xlo = (const h16x8 *)xs[r];
+                const h16x8 x0 = xlo[s + 64 * u], x1 = xlo[nseg + s + 64 * u];
+                acc[r] = dot16_u8(wv[u][r], x0, x1, acc[r]);
+            }
         }
     }
     for (; s < nseg; s += 64) {
-        const h16x8 x0 = xlo[s], x1 = xhi[s];
 #pragma unroll
         for (int r = 0; r < R; ++r) {
+            const h16x8 *xlo = (const h16x8 *)xs[r];
+            const h16x8 x0 = xlo[s], x1 = xlo[nseg + s];
             u32x4 wv = __builtin_nontemporal_load((const u32x4 *)(rows[r] + 16 * (size_t)s));
             acc[r] = dot16_u8(wv, x0, x1, acc[r]);
         }
@@ -85,11 +88,10 @@ DEV void wave_rows_dot_u8(const uint8_t *const (&rows)[R], const h16 *xs, int ns
     for (int r = 0; r < R; ++r) acc[r] = wave_sum(acc[r]);
 }
 
-// fp16 rows: N halves per row, xs stored linearly in LDS; segments are 8 values (16 bytes).
+// fp16 rows: N halves per row, xs[r] stored linearly in LDS; segments are 8 values (16 bytes).
 template <int R, int U>
-DEV void wave_rows_dot_f16(const h16 *const (&rows)[R], const h16 *xs, int nseg8, float (&acc)[R]) {
+DEV void wave_rows_dot_f16(const h16 *const (&rows)[R], const h16 *const (&xs)[R], int nseg8, float (&acc)[R]) {
     const int lane = threadIdx.x & 63;
-    const h16x8 *xv = (const h16x8 *)xs;
     int s = lane;
     for (; s + 64 * (U - 1) < nseg8; s += 64 * U) {
         u32x4 wv[U][R];
@@ -100,21 +102,43 @@ DEV void wave_rows_dot_f16(const h16 *const (&rows)[R], const h16 *xs, int nseg8
                 wv[u][r] = __builtin_nontemporal_load((const u32x4 *)(rows[r] + 8 * (size_t)(s + 64 * u)));
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            const h16x8 x = xv[s + 64 * u];
 #pragma unroll
-            for (int r = 0; r < R; ++r) acc[r] = dot8_f16(wv[u][r], x, acc[r]);
+            for (int r = 0; r < R; ++r) {
+                const h16x8 x = ((const h16x8 *)xs[r])[s + 64 * u];
+                acc[r] = dot8_f16(wv[u][r], x, acc[r]);
+            }
         }
     }
     for (; s < nseg8; s += 64) {
-        const h16x8 x = xv[s];
 #pragma unroll
         for (int r = 0; r < R; ++r) {
+            const h16x8 x = ((const h16x8 *)xs[r])[s];
             u32x4 wv = __builtin_nontemporal_load((const u32x4 *)(rows[r] + 8 * (size_t)s));
             acc[r] = dot8_f16(wv, x, acc[r]);
         }
     }
 #pragma unroll
     for (int r = 0; r < R; ++r) acc[r] = wave_sum(acc[r]);
+}
+
+// Sum K values over the workgroup at once; every thread gets all K totals.
+// `red` is LDS scratch of at least K * (blockDim.x / 64) floats.
+template <int K>
+DEV void block_sum_n(float (&v)[K], float *red) {
+    const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
+#pragma unroll
+    for (int k = 0; k < K; ++k) v[k] = wave_sum(v[k]);
+    __syncthreads();
+    if (lane == 0)
+#pragma unroll
+        for (int k = 0; k < K; ++k) red[k * nw + wid] = v[k];
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+        float t = 0.f;
+        for (int i = 0; i < nw; ++i) t += red[k * nw + i];
+        v[k] = t;
+    }
 }
 
 // Final value of a uint8 row from its raw dot product.

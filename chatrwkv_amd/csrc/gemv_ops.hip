@@ -1,5 +1,6 @@
 // Operator-level GEMV entry points: rwkv_mm8_one_f16 and the B == 1 path of rwkv_gemm_f16.
 #include "gemv_core.h"
+#include "kernels.h"
 
 namespace {
 
@@ -36,14 +37,16 @@ __global__ __launch_bounds__(GEMV_THREADS) void mm8_one_kernel(
     const int ngroups = (M + R - 1) / R;
     for (int g = blockIdx.x * (GEMV_THREADS / 64) + wave; g < ngroups; g += nwaves) {
         const uint8_t *rows[R];
+        const h16 *xv[R];
         float acc[R];
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             const int m = min(g * R + r, M - 1);
             rows[r] = w + (size_t)m * ldw;
+            xv[r] = xs;
             acc[r] = 0.f;
         }
-        wave_rows_dot_u8<R, U>(rows, xs, nseg, acc);
+        wave_rows_dot_u8<R, U>(rows, xv, nseg, acc);
         if (lane < R) {
             float a = acc[0];
 #pragma unroll
@@ -73,14 +76,16 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_f16_kernel(
     const int ngroups = (M + R - 1) / R;
     for (int g = blockIdx.x * (GEMV_THREADS / 64) + wave; g < ngroups; g += nwaves) {
         const h16 *rows[R];
+        const h16 *xv[R];
         float acc[R];
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             const int m = min(g * R + r, M - 1);
             rows[r] = w + (size_t)m * ldw;
+            xv[r] = xs;
             acc[r] = 0.f;
         }
-        wave_rows_dot_f16<R, U>(rows, xs, N >> 3, acc);
+        wave_rows_dot_f16<R, U>(rows, xv, N >> 3, acc);
         if (lane < R) {
             float a = acc[0];
 #pragma unroll

@@ -1,0 +1,30 @@
+// Launchers shared between translation units of librwkv_hip.so (internal, not part of the C ABI).
+#pragma once
+#include "common.h"
+
+enum { ACT_NONE = 0, ACT_SIGMOID = 1, ACT_RELU_SQ = 2, ACT_RESIDUAL = 3, ACT_GATED_RESIDUAL = 4 };
+
+// Epilogue of the MFMA contraction (gemm.hip).
+struct GemmEpi {
+    const rwkv_half *mx, *rx;      // [M]; NULL for plain fp16 weights
+    const float *s0, *s2;          // [T] row sums of the unscaled activation (uint8 weights)
+    int act;
+    const rwkv_half *res; int64_t ldres;    // residual input [T, M]
+    const rwkv_half *gate; int64_t ldgate;  // gate [T, M]
+    float out_scale;               // applied to the final fp16 value (1 or 0.5)
+    int out_dtype;                 // RWKV_DT_F16 / RWKV_DT_F32 (the fp16-rounded value widened)
+    int raw_f32;                   // 1: store the fp32 accumulator unrounded (out_dtype must be F32)
+};
+
+int gemm_launch(bool w_u8, int64_t T, int64_t N, int64_t M, const rwkv_half *A, int64_t lda, const void *W,
+                int64_t ldw, void *Y, int64_t ldy, const GemmEpi &ep, hipStream_t st);
+int mm8_prepare_launch(int64_t T, int64_t N, const rwkv_half *x, int64_t ldx, const rwkv_half *ry,
+                       const rwkv_half *my, rwkv_half *xs, float *s0, float *s2, hipStream_t st);
+int gemv_f16_launch(int64_t N, int64_t M, const rwkv_half *x, const rwkv_half *w, int64_t ldw, void *y,
+                    int y_dtype, hipStream_t st);
+// kv_f32: k, v are fp32 (fp16-weight strategy) instead of fp16.
+int wkv4_fused_launch(int T, int C, const float *w, const float *u, const void *k, const void *v, int kv_f32,
+                      const rwkv_half *r, rwkv_half *y, float *aa, float *bb, float *pp, hipStream_t st);
+int v4_model_check(const rwkv_v4_model *m);
+int v4_head_launch(const rwkv_v4_model *m, const rwkv_half *x, float *logits, hipStream_t st);
+int num_cu();

@@ -1,0 +1,303 @@
+// RWKV-4 sequence mode (len(tokens) > 1): per layer
+//   lnmix_seq (LN1, token shift, k/v/r mixes, ry scaling, row sums) -> 3 MFMA GEMMs (sigmoid fused for r)
+//   -> WKV-4 over T (r gating fused) -> prepare -> GEMM Wo (+ residual)
+//   lnmix_seq (LN2, ...) -> GEMM Wr (sigmoid), GEMM Wk (relu^2) -> prepare -> GEMM Wv (gate, residual, /2)
+// and LN_out + head on the last row (GEMV) or on every row (GEMM) for full_output.
+#include "kernels.h"
+
+namespace {
+
+constexpr float LN_EPS = 1e-5f;
+
+__global__ __launch_bounds__(256) void gather_emb_kernel(int T, int C, const int32_t *__restrict__ tokens,
+                                                         const rwkv_half *__restrict__ emb,
+                                                         rwkv_half *__restrict__ x) {
+    const int t = blockIdx.x;
+    const u32x4 *src = (const u32x4 *)(emb + (size_t)tokens[t] * C);
+    u32x4 *dst = (u32x4 *)(x + (size_t)t * C);
+    for (int i = threadIdx.x; i < (C >> 3); i += blockDim.x) dst[i] = src[i];
+}
+
+__global__ __launch_bounds__(256) void copy16_kernel(int n16, const u32x4 *__restrict__ src, u32x4 *__restrict__ dst) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n16) dst[i] = src[i];
+}
+
+DEV void row_stats(const rwkv_half *x, int C, float *red, float &mean, float &rstd) {
+    float s = 0.f;
+    for (int j8 = threadIdx.x; j8 < (C >> 3); j8 += blockDim.x) {
+        const h16x8 v = *(const h16x8 *)(x + 8 * j8);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) s += (float)v[e];
+    }
+    mean = block_sum(s, red) / C;
+    float q = 0.f;
+    for (int j8 = threadIdx.x; j8 < (C >> 3); j8 += blockDim.x) {
+        const h16x8 v = *(const h16x8 *)(x + 8 * j8);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const float d = (float)v[e] - mean;
+            q += d * d;
+        }
+    }
+    rstd = rsqrtf(block_sum(q, red) / C + LN_EPS);
+}
+
+struct SeqMixArgs {
+    int T, C;
+    const rwkv_half *x;        // [T, C]
+    const rwkv_half *ln_w, *ln_b;
+    const rwkv_half *sx;       // state (previous token's normalised activation), NULL = no token shift
+    rwkv_half *xx_last;        // scratch [C]: normalised activation of the last row (new state)
+    const rwkv_half *mix[3];   // NULL entry = consumer sees LN(x)
+    const rwkv_half *ry[3], *my[3];  // NULL ry = no scaling / sums (fp16 weights)
+    rwkv_half *xs[3];          // [T, C] outputs
+    float *s0[3], *s2[3];      // [T] outputs
+};
+
+// One workgroup per token row.  Row t needs LN(x[t-1]) for the token shift: it is recomputed here
+// from x[t-1] (same code, same data => same bits as row t-1 computes for itself), which keeps all
+// rows independent.
+template <int NJ>
+__global__ __launch_bounds__(256) void lnmix_seq_kernel(SeqMixArgs a) {
+    __shared__ float red[2 * 3 * 4 + 4];
+    const int t = blockIdx.x, C = a.C;
+    const rwkv_half *x = a.x + (size_t)t * C;
+    float mean, rstd, pmean = 0.f, prstd = 0.f;
+    row_stats(x, C, red, mean, rstd);
+    const bool shift = a.sx != nullptr;
+    const rwkv_half *xp = x - C;
+    if (shift && t > 0) row_stats(xp, C, red, pmean, prstd);
+    float acc[2 * NJ];
+#pragma unroll
+    for (int i = 0; i < 2 * NJ; ++i) acc[i] = 0.f;
+    for (int j8 = threadIdx.x; j8 < (C >> 3); j8 += blockDim.x) {
+        const h16x8 xv = *(const h16x8 *)(x + 8 * j8);
+        const h16x8 wv = *(const h16x8 *)(a.ln_w + 8 * j8);
+        const h16x8 bv = *(const h16x8 *)(a.ln_b + 8 * j8);
+        h16x8 xx, pv;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) xx[e] = (h16)(((float)xv[e] - mean) * rstd * (float)wv[e] + (float)bv[e]);
+        pv = xx;
+        if (shift) {
+            if (t > 0) {
+                const h16x8 pxv = *(const h16x8 *)(xp + 8 * j8);
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    pv[e] = (h16)(((float)pxv[e] - pmean) * prstd * (float)wv[e] + (float)bv[e]);
+            } else {
+                pv = *(const h16x8 *)(a.sx + 8 * j8);
+            }
+        }
+        if (a.xx_last && t == a.T - 1) *(h16x8 *)(a.xx_last + 8 * j8) = xx;
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+            h16x8 kx = xx;
+            if (a.mix[j]) {
+                const h16x8 mv = *(const h16x8 *)(a.mix[j] + 8 * j8);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const float m = (float)mv[e];
+                    kx[e] = (h16)((float)xx[e] * m + (float)pv[e] * (1.f - m));
+                }
+            }
+            h16x8 o = kx;
+            if (a.ry[j]) {
+                const h16x8 rv = *(const h16x8 *)(a.ry[j] + 8 * j8);
+                const h16x8 yv = *(const h16x8 *)(a.my[j] + 8 * j8);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const float k = (float)kx[e];
+                    o[e] = (h16)(k * (float)rv[e]);
+                    acc[2 * j] += k;
+                    acc[2 * j + 1] += k * (float)yv[e];
+                }
+            }
+            *(h16x8 *)(a.xs[j] + (size_t)t * C + 8 * j8) = o;
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+        if (!a.ry[j]) continue;
+        const float v0 = block_sum(acc[2 * j], red), v2 = block_sum(acc[2 * j + 1], red);
+        if (threadIdx.x == 0) { a.s0[j][t] = v0; a.s2[j][t] = v2; }
+    }
+}
+
+__global__ __launch_bounds__(256) void ln_f32_f16_kernel(int C, const float *__restrict__ x_, const float *__restrict__ w,
+                                                         const float *__restrict__ b, rwkv_half *__restrict__ y_) {
+    __shared__ float red[4];
+    const float *x = x_ + (size_t)blockIdx.x * C;
+    rwkv_half *y = y_ + (size_t)blockIdx.x * C;
+    float s = 0.f;
+    for (int j = threadIdx.x; j < C; j += blockDim.x) s += x[j];
+    const float mean = block_sum(s, red) / C;
+    float q = 0.f;
+    for (int j = threadIdx.x; j < C; j += blockDim.x) { const float d = x[j] - mean; q += d * d; }
+    const float rstd = rsqrtf(block_sum(q, red) / C + LN_EPS);
+    for (int j = threadIdx.x; j < C; j += blockDim.x) y[j] = f2h((x[j] - mean) * rstd * w[j] + b[j]);
+}
+
+size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
+
+struct SeqWs {
+    rwkv_half *x, *xs[3], *r, *rwkv, *vx, *xsv, *xx_att, *xx_ffn;
+    void *k, *v;       // fp16 (uint8 weights) or fp32 (fp16 weights)
+    float *sums;       // 8 * T floats
+    size_t total;
+};
+
+SeqWs carve(void *base, int64_t T, int64_t C, int64_t F) {
+    SeqWs w;
+    unsigned char *p = (unsigned char *)base;
+    auto take = [&](size_t bytes) { void *q = p; p += align256(bytes); return q; };
+    const size_t tc = (size_t)T * C * 2, tf = (size_t)T * F * 2;
+    w.x = (rwkv_half *)take(tc);
+    for (int j = 0; j < 3; ++j) w.xs[j] = (rwkv_half *)take(tc);
+    w.r = (rwkv_half *)take(tc);
+    w.rwkv = (rwkv_half *)take(tc);
+    w.k = take(2 * tc);
+    w.v = take(2 * tc);
+    w.vx = (rwkv_half *)take(tf);
+    w.xsv = (rwkv_half *)take(tf);
+    w.xx_att = (rwkv_half *)take((size_t)C * 2);
+    w.xx_ffn = (rwkv_half *)take((size_t)C * 2);
+    w.sums = (float *)take((size_t)T * 8 * sizeof(float));
+    w.total = (size_t)(p - (unsigned char *)base);
+    return w;
+}
+
+int run_gemm(const rwkv_mat &m, bool u8, int64_t T, const rwkv_half *A, const float *s0, const float *s2, void *Y,
+             int64_t ldy, GemmEpi ep, hipStream_t st) {
+    ep.mx = u8 ? m.mx : nullptr;
+    ep.rx = u8 ? m.rx : nullptr;
+    ep.s0 = s0;
+    ep.s2 = s2;
+    return gemm_launch(u8, T, m.N, m.M, A, m.N, m.w, m.ld, Y, ldy, ep, st);
+}
+
+}  // namespace
+
+extern "C" int rwkv_layernorm_f32_f16(int64_t T, int64_t C, const float *x, const float *w, const float *b,
+                                      rwkv_half *y, void *stream) {
+    if (!x || !w || !b || !y) return RWKV_E_NULL;
+    if (T <= 0 || C <= 0 || T > 0x7fffffff) return RWKV_E_SHAPE;
+    hipLaunchKernelGGL(ln_f32_f16_kernel, dim3((unsigned)T), dim3(256), 0, (hipStream_t)stream, (int)C, x, w, b, y);
+    RWKV_LAUNCH_CHECK();
+    return RWKV_OK;
+}
+
+extern "C" size_t rwkv_v4_seq_workspace(const rwkv_v4_model *m, int64_t T, int full_output) {
+    if (!m || T <= 0) return 0;
+    (void)full_output;
+    return carve((void *)256, T, m->n_embd, m->n_ffn).total;
+}
+
+extern "C" int rwkv_v4_forward_seq(const rwkv_v4_model *m, const rwkv_v4_layer_state *states, const int32_t *tokens,
+                                   int64_t T, int full_output, float *logits, void *workspace,
+                                   size_t workspace_bytes, void *stream) {
+    int rc = v4_model_check(m);
+    if (rc) return rc;
+    if (!states || !tokens || !logits || !workspace) return RWKV_E_NULL;
+    if (T <= 0 || T > (1 << 20)) return RWKV_E_SHAPE;
+    if (workspace_bytes < rwkv_v4_seq_workspace(m, T, full_output) || (((uintptr_t)workspace) & 255))
+        return RWKV_E_WORKSPACE;
+    for (int i = 0; i < m->n_layer; ++i) {
+        const rwkv_v4_layer_state &s = states[i];
+        if (!s.att_xx || !s.aa || !s.bb || !s.pp || !s.ffn_xx) return RWKV_E_NULL;
+        if (!aligned16(s.att_xx) || !aligned16(s.ffn_xx)) return RWKV_E_LAYOUT;
+    }
+    hipStream_t st = (hipStream_t)stream;
+    const int C = m->n_embd, F = m->n_ffn;
+    const bool u8 = m->weights_u8 != 0;
+    SeqWs ws = carve(workspace, T, C, F);
+    float *s0[3] = {ws.sums, ws.sums + 2 * T, ws.sums + 4 * T};
+    float *s2[3] = {ws.sums + T, ws.sums + 3 * T, ws.sums + 5 * T};
+    float *s0v = ws.sums + 6 * T, *s2v = ws.sums + 7 * T;
+    const int n16 = C >> 3;
+
+    hipLaunchKernelGGL(gather_emb_kernel, dim3((unsigned)T), dim3(256), 0, st, (int)T, C, tokens, m->emb, ws.x);
+
+    for (int i = 0; i < m->n_layer; ++i) {
+        const rwkv_v4_layer &l = m->layers[i];
+        const rwkv_v4_layer_state &s = states[i];
+        // ---- time mix
+        {
+            SeqMixArgs a{};
+            a.T = (int)T; a.C = C; a.x = ws.x; a.ln_w = l.ln1_w; a.ln_b = l.ln1_b; a.sx = s.att_xx;
+            a.xx_last = ws.xx_att;
+            const rwkv_half *mix[3] = {l.att_mix_k, l.att_mix_v, l.att_mix_r};
+            const rwkv_mat *mt[3] = {&l.att_key, &l.att_value, &l.att_receptance};
+            for (int j = 0; j < 3; ++j) {
+                a.mix[j] = mix[j]; a.ry[j] = u8 ? mt[j]->ry : nullptr; a.my[j] = u8 ? mt[j]->my : nullptr;
+                a.xs[j] = ws.xs[j]; a.s0[j] = s0[j]; a.s2[j] = s2[j];
+            }
+            hipLaunchKernelGGL(lnmix_seq_kernel<3>, dim3((unsigned)T), dim3(256), 0, st, a);
+        }
+        hipLaunchKernelGGL(copy16_kernel, dim3((n16 + 255) / 256), dim3(256), 0, st, n16, (const u32x4 *)ws.xx_att,
+                           (u32x4 *)s.att_xx);
+        GemmEpi e{};
+        e.out_scale = 1.f;
+        // k, v: uint8 weights return fp16 (widened by the consumer); fp16 weights return fp32 directly
+        e.act = ACT_NONE; e.out_dtype = u8 ? RWKV_DT_F16 : RWKV_DT_F32; e.raw_f32 = u8 ? 0 : 1;
+        if ((rc = run_gemm(l.att_key, u8, T, ws.xs[0], s0[0], s2[0], ws.k, C, e, st))) return rc;
+        if ((rc = run_gemm(l.att_value, u8, T, ws.xs[1], s0[1], s2[1], ws.v, C, e, st))) return rc;
+        e.act = ACT_SIGMOID; e.out_dtype = RWKV_DT_F16; e.raw_f32 = 0;
+        if ((rc = run_gemm(l.att_receptance, u8, T, ws.xs[2], s0[2], s2[2], ws.r, C, e, st))) return rc;
+        if ((rc = wkv4_fused_launch((int)T, C, l.time_decay, l.time_first, ws.k, ws.v, u8 ? 0 : 1, ws.r, ws.rwkv, s.aa,
+                                    s.bb, s.pp, st)))
+            return rc;
+        const rwkv_half *a_out = ws.rwkv;
+        if (u8) {
+            if ((rc = mm8_prepare_launch(T, C, ws.rwkv, C, l.att_output.ry, l.att_output.my, ws.xs[0], s0[0], s2[0], st)))
+                return rc;
+            a_out = ws.xs[0];
+        }
+        e.act = ACT_RESIDUAL; e.res = ws.x; e.ldres = C;
+        if ((rc = run_gemm(l.att_output, u8, T, a_out, s0[0], s2[0], ws.x, C, e, st))) return rc;
+        // ---- channel mix
+        {
+            SeqMixArgs a{};
+            a.T = (int)T; a.C = C; a.x = ws.x; a.ln_w = l.ln2_w; a.ln_b = l.ln2_b; a.sx = s.ffn_xx;
+            a.xx_last = ws.xx_ffn;
+            const rwkv_half *mix[2] = {l.ffn_mix_r, l.ffn_mix_k};
+            const rwkv_mat *mt[2] = {&l.ffn_receptance, &l.ffn_key};
+            for (int j = 0; j < 2; ++j) {
+                a.mix[j] = mix[j]; a.ry[j] = u8 ? mt[j]->ry : nullptr; a.my[j] = u8 ? mt[j]->my : nullptr;
+                a.xs[j] = ws.xs[j]; a.s0[j] = s0[j]; a.s2[j] = s2[j];
+            }
+            hipLaunchKernelGGL(lnmix_seq_kernel<2>, dim3((unsigned)T), dim3(256), 0, st, a);
+        }
+        hipLaunchKernelGGL(copy16_kernel, dim3((n16 + 255) / 256), dim3(256), 0, st, n16, (const u32x4 *)ws.xx_ffn,
+                           (u32x4 *)s.ffn_xx);
+        e = GemmEpi{};
+        e.out_scale = 1.f; e.out_dtype = RWKV_DT_F16;
+        e.act = ACT_SIGMOID;
+        if ((rc = run_gemm(l.ffn_receptance, u8, T, ws.xs[0], s0[0], s2[0], ws.r, C, e, st))) return rc;
+        e.act = ACT_RELU_SQ;
+        if ((rc = run_gemm(l.ffn_key, u8, T, ws.xs[1], s0[1], s2[1], ws.vx, F, e, st))) return rc;
+        const rwkv_half *a_v = ws.vx;
+        if (u8) {
+            if ((rc = mm8_prepare_launch(T, F, ws.vx, F, l.ffn_value.ry, l.ffn_value.my, ws.xsv, s0v, s2v, st))) return rc;
+            a_v = ws.xsv;
+        }
+        e.act = ACT_GATED_RESIDUAL; e.gate = ws.r; e.ldgate = C; e.res = ws.x; e.ldres = C;
+        e.out_scale = (m->rescale_layer > 0 && (i + 1) % m->rescale_layer == 0) ? 0.5f : 1.f;
+        if ((rc = run_gemm(l.ffn_value, u8, T, a_v, s0v, s2v, ws.x, C, e, st))) return rc;
+        RWKV_LAUNCH_CHECK();
+    }
+    if (!full_output) return v4_head_launch(m, ws.x + (size_t)(T - 1) * C, logits, st);
+    {
+        SeqMixArgs a{};
+        a.T = (int)T; a.C = C; a.x = ws.x; a.ln_w = m->ln_out_w; a.ln_b = m->ln_out_b; a.sx = nullptr;
+        a.xx_last = nullptr; a.mix[0] = nullptr;
+        a.ry[0] = u8 ? m->head.ry : nullptr; a.my[0] = u8 ? m->head.my : nullptr;
+        a.xs[0] = ws.xs[0]; a.s0[0] = s0[0]; a.s2[0] = s2[0];
+        hipLaunchKernelGGL(lnmix_seq_kernel<1>, dim3((unsigned)T), dim3(256), 0, st, a);
+    }
+    GemmEpi e{};
+    e.out_scale = 1.f; e.act = ACT_NONE; e.out_dtype = RWKV_DT_F32;
+    if ((rc = run_gemm(m->head, u8, T, ws.xs[0], s0[0], s2[0], logits, m->vocab, e, st))) return rc;
+    RWKV_LAUNCH_CHECK();
+    return RWKV_OK;
+}

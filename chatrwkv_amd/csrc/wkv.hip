@@ -1,5 +1,5 @@
 // WKV recurrences: RWKV-4 (per channel, running-maximum form) and RWKV-5/6 (per-head 64x64 state).
-#include "common.h"
+#include "kernels.h"
 
 namespace {
 
@@ -10,6 +10,7 @@ namespace {
 // critical path.  One wave per workgroup spreads the C/64 waves over as many CUs as possible.
 //   MODE 0: k, v, y fp32 (operator-level interface)
 //   MODE 1: k, v fp16; y = fp16(r * fp16(wkv)) with r fp16 (already sigmoid'ed), fp16 out
+//   MODE 2: as MODE 1 with k, v fp32
 // ---------------------------------------------------------------------------------------
 template <int MODE> struct Wkv4IO;
 template <> struct Wkv4IO<0> {
@@ -23,6 +24,13 @@ template <> struct Wkv4IO<1> {
     const rwkv_half *k, *v; rwkv_half *y; const rwkv_half *r;
     DEV float ldk(size_t i) const { return h2f(k[i]); }
     DEV float ldv(size_t i) const { return h2f(v[i]); }
+    DEV float ldr(size_t i) const { return h2f(r[i]); }
+    DEV void st(size_t i, float wkv, float rr) const { y[i] = f2h(rr * round_h(wkv)); }
+};
+template <> struct Wkv4IO<2> {
+    const float *k, *v; rwkv_half *y; const rwkv_half *r;
+    DEV float ldk(size_t i) const { return k[i]; }
+    DEV float ldv(size_t i) const { return v[i]; }
     DEV float ldr(size_t i) const { return h2f(r[i]); }
     DEV void st(size_t i, float wkv, float rr) const { y[i] = f2h(rr * round_h(wkv)); }
 };
@@ -172,11 +180,17 @@ extern "C" int rwkv_wkv4_forward(int64_t B, int64_t T, int64_t C, const float *w
     return RWKV_OK;
 }
 
-// fused variant used by the model path: fp16 k, v, r in; y = fp16(r * fp16(wkv)).
-int wkv4_fused_launch(int T, int C, const float *w, const float *u, const rwkv_half *k, const rwkv_half *v,
+// fused variant used by the model path: k, v (fp16 or fp32) and fp16 r in; y = fp16(r * fp16(wkv)).
+int wkv4_fused_launch(int T, int C, const float *w, const float *u, const void *k, const void *v, int kv_f32,
                       const rwkv_half *r, rwkv_half *y, float *aa, float *bb, float *pp, hipStream_t st) {
-    Wkv4IO<1> io{k, v, y, r};
-    hipLaunchKernelGGL(wkv4_kernel<1>, dim3((unsigned)((C + 63) / 64), 1), dim3(64), 0, st, T, C, w, u, io, aa, bb, pp);
+    const dim3 grid((unsigned)((C + 63) / 64), 1);
+    if (kv_f32) {
+        Wkv4IO<2> io{(const float *)k, (const float *)v, y, r};
+        hipLaunchKernelGGL(wkv4_kernel<2>, grid, dim3(64), 0, st, T, C, w, u, io, aa, bb, pp);
+    } else {
+        Wkv4IO<1> io{(const rwkv_half *)k, (const rwkv_half *)v, y, r};
+        hipLaunchKernelGGL(wkv4_kernel<1>, grid, dim3(64), 0, st, T, C, w, u, io, aa, bb, pp);
+    }
     RWKV_LAUNCH_CHECK();
     return RWKV_OK;
 }

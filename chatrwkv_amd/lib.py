@@ -37,6 +37,40 @@ SIGNATURES = {
     "rwkv_wkv6_forward": (_int, [_i64, _i64, _i64, _i64, _vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
 }
 
+
+
+class RwkvMat(ctypes.Structure):
+    _fields_ = [("w", _vp), ("ld", _i64), ("mx", _vp), ("rx", _vp), ("my", _vp), ("ry", _vp), ("N", _i64), ("M", _i64)]
+
+
+class RwkvV4Layer(ctypes.Structure):
+    _fields_ = [("ln1_w", _vp), ("ln1_b", _vp), ("ln2_w", _vp), ("ln2_b", _vp),
+                ("att_mix_k", _vp), ("att_mix_v", _vp), ("att_mix_r", _vp),
+                ("time_decay", _vp), ("time_first", _vp),
+                ("att_key", RwkvMat), ("att_value", RwkvMat), ("att_receptance", RwkvMat), ("att_output", RwkvMat),
+                ("ffn_mix_k", _vp), ("ffn_mix_r", _vp),
+                ("ffn_key", RwkvMat), ("ffn_receptance", RwkvMat), ("ffn_value", RwkvMat)]
+
+
+class RwkvV4LayerState(ctypes.Structure):
+    _fields_ = [("att_xx", _vp), ("aa", _vp), ("bb", _vp), ("pp", _vp), ("ffn_xx", _vp)]
+
+
+class RwkvV4Model(ctypes.Structure):
+    _fields_ = [("n_layer", ctypes.c_int32), ("n_embd", ctypes.c_int32), ("n_ffn", ctypes.c_int32),
+                ("vocab", ctypes.c_int32), ("rescale_layer", ctypes.c_int32), ("weights_u8", ctypes.c_int32),
+                ("emb", _vp), ("ln_out_w", _vp), ("ln_out_b", _vp), ("head", RwkvMat),
+                ("layers", ctypes.POINTER(RwkvV4Layer))]
+
+
+SIGNATURES.update({
+    "rwkv_layernorm_f32_f16": (_int, [_i64, _i64, _vp, _vp, _vp, _vp, _vp]),
+    "rwkv_v4_one_workspace": (_sz, [ctypes.POINTER(RwkvV4Model)]),
+    "rwkv_v4_forward_one": (_int, [ctypes.POINTER(RwkvV4Model), ctypes.POINTER(RwkvV4LayerState), _vp, _vp, _vp, _sz, _vp]),
+    "rwkv_v4_seq_workspace": (_sz, [ctypes.POINTER(RwkvV4Model), _i64, _int]),
+    "rwkv_v4_forward_seq": (_int, [ctypes.POINTER(RwkvV4Model), ctypes.POINTER(RwkvV4LayerState), _vp, _i64, _int, _vp, _vp, _sz, _vp]),
+})
+
 _lib = None
 
 

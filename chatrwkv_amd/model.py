@@ -1,0 +1,363 @@
+"""``RWKV(model, strategy)`` / ``model.forward(tokens, state)`` on one MI355X.
+
+Drop-in for the class of the same name in rwkv_pip_package/src/rwkv/model.py:612-1677 for
+the strategies 'cuda fp16i8' and 'cuda fp16': same constructor and forward signatures, same
+state-list layout, dtypes and initial values (model.py:1448-1471), same chunked-prefill
+behaviour (len(tokens) == 1 -> one-token mode, > 1 -> sequence mode, state carried
+between calls).  Everything numeric runs in librwkv_hip.so; PyTorch provides device
+memory, streams and graph capture only.
+
+Differences a caller can observe, all deliberate:
+  * the embedding table lives on the GPU (the reference keeps it on the CPU and copies one
+    row per token, model.py:852-853, 1475);
+  * weight matrices keep the reference's shape [in, out] but are stored input-contiguous
+    (strides (1, in)), the orientation the kernels stream;
+  * every state tensor is updated in place (the reference's CUDA sequence path already does
+    this for aa, bb, pp); ``copy.deepcopy(state)`` snapshots a state as in v2/chat.py:166-179;
+  * ``model`` may also be an in-memory ``{name: tensor}`` dict (tensors on CPU or GPU), and
+    ``tokens`` of a one-token call may be a 1-element integer tensor on the GPU, which keeps a
+    greedy decode loop free of host synchronisation.
+"""
+import collections
+import ctypes
+import gc
+import os
+import types
+
+import torch
+
+from . import lib as _lib
+from . import ops as _ops
+from . import strategy as _strategy
+
+_MATRIX_KEYS = ('key.weight', 'value.weight', 'receptance.weight', 'gate.weight', 'output.weight', 'head.weight')
+
+
+class StateList(list):
+    """The state list returned by forward(): a plain list of tensors (model.py:1448-1471) that
+    also remembers the flat buffers its entries are views of, so that a one-token step on the
+    same state can replay a captured HIP graph."""
+    flat = None      # tuple of backing tensors
+    views = None     # the tensors as handed out, to detect replaced entries
+
+    def intact(self):
+        v = self.views
+        return v is not None and len(v) == len(self) and all(a is b for a, b in zip(self, v))
+
+
+def _ptr(t):
+    return ctypes.c_void_p(t.data_ptr())
+
+
+class RWKV:
+    def __init__(self, model, strategy, verbose=True, convert_and_save_and_exit=None):
+        prxxx = (lambda *a, **k: print(*a, **k)) if verbose else (lambda *a, **k: None)
+        self.args = types.SimpleNamespace()
+        args = self.args
+        args.strategy_string = _strategy.normalize(strategy)          # ValueError on a bad string
+        try:                                                          # model.py:631-634
+            self.RESCALE_LAYER = int(os.environ["RWKV_RESCALE_LAYER"])
+        except (KeyError, ValueError):
+            self.RESCALE_LAYER = 6 if 'fp16' in args.strategy_string else 0
+
+        if isinstance(model, dict):
+            args.MODEL_NAME = '<dict>'
+            w = dict(model)
+        else:
+            args.MODEL_NAME = model.strip()
+            if not args.MODEL_NAME.endswith('.pth'):
+                args.MODEL_NAME += '.pth'
+            prxxx(f'Loading {args.MODEL_NAME} ...')
+            w = torch.load(args.MODEL_NAME, map_location='cpu')
+
+        converted = '_strategy' in w                                  # model.py:646-656
+        if converted:
+            assert convert_and_save_and_exit is None
+            assert w['_strategy'] == args.strategy_string
+            assert float(w['_version']) >= 0.7
+            assert w['_rescale_layer'] == self.RESCALE_LAYER
+            for k in ('_strategy', '_version', '_rescale_layer'):
+                del w[k]
+
+        # shape / version detection (model.py:658-680)
+        args.n_embd = w['emb.weight'].shape[1]
+        args.n_att = w['blocks.0.att.key.weight'].shape[1 if converted else 0]
+        args.n_ffn = w['blocks.0.ffn.key.weight'].shape[1 if converted else 0]
+        args.n_layer = 0
+        args.n_head = 0
+        self.version = 4
+        for x in list(w.keys()):
+            layer_id = int(x.split('.')[1]) if ('blocks.' in x) else 0
+            args.n_layer = max(args.n_layer, layer_id + 1)
+            if 'ln_x' in x:
+                self.version = max(5, self.version)
+            if 'gate.weight' in x:
+                self.version = max(5.1, self.version)
+            if int(self.version) == 5 and 'att.time_decay' in x:
+                args.n_head = w[x].shape[0]
+                if len(w[x].shape) > 1 and w[x].shape[1] > 1:
+                    self.version = max(5.2, self.version)
+            if 'time_maa' in x:
+                self.version = max(6, self.version)
+            if int(self.version) == 6 and 'time_faaaa' in x:
+                args.n_head = w[x].shape[0]
+        prxxx(f'Model detected: v{self.version:.1f}')
+
+        self.strategy = _strategy.plan(args.strategy_string, args.n_layer)
+        for n, s in enumerate(self.strategy):
+            prxxx(f"{n}-{s.device}-{str(s.atype).replace('torch.', '')}-{str(s.wtype).replace('torch.', '')}"
+                  f"{'-stream' if s.stream else ''}", end=' ')
+        prxxx()
+        self._wkind = _strategy.require_single_gpu(self.strategy)    # NotImplementedError otherwise
+        if self.version != 4:
+            raise NotImplementedError(f"RWKV v{self.version} is not wired into chatrwkv_amd.RWKV yet "
+                                      "(the v5/v6 operators are in chatrwkv_amd.ops)")
+        if args.n_att != args.n_embd:
+            raise NotImplementedError("n_att != n_embd")
+        _lib.load()                                                   # fail early and loudly
+        if not torch.cuda.is_available():
+            raise _lib.RwkvHipError("no ROCm GPU visible: chatrwkv_amd has no CPU path")
+        self.device = torch.device('cuda:0')
+        torch.cuda.set_device(self.device)
+
+        with torch.no_grad():
+            self.w = self._convert(w, converted, prxxx)
+            if convert_and_save_and_exit:
+                self._save_converted(convert_and_save_and_exit, prxxx)
+                raise SystemExit(0)                                   # model.py:903
+            self._build_descriptors()
+        self._graphs = collections.OrderedDict()
+        self._seq_ws = None
+        gc.collect()
+        torch.cuda.empty_cache()
+
+    # ------------------------------------------------------------------ weights
+    def _convert(self, w, converted, prxxx):
+        """Weight transforms of model.py:754-849, executed on the GPU: LayerNorm of the embedding,
+        rescale, quantisation.  The small time_* vectors follow the reference on the CPU."""
+        args, dev, R = self.args, self.device, self.RESCALE_LAYER
+        L = _lib.load()
+        st = torch.cuda.current_stream().cuda_stream
+        u8 = self._wkind == 'u8'
+        out = {}
+        if not converted:
+            emb = w['emb.weight'].to(device=dev, dtype=torch.float32).contiguous()
+            ln_w = w['blocks.0.ln0.weight'].to(device=dev, dtype=torch.float32).contiguous()
+            ln_b = w['blocks.0.ln0.bias'].to(device=dev, dtype=torch.float32).contiguous()
+            emb16 = torch.empty(emb.shape, dtype=torch.float16, device=dev)
+            _lib.check(L.rwkv_layernorm_f32_f16(emb.shape[0], emb.shape[1], emb.data_ptr(), ln_w.data_ptr(),
+                                                ln_b.data_ptr(), emb16.data_ptr(), st), "rwkv_layernorm_f32_f16")
+            out['emb.weight'] = emb16
+            del emb
+        for x in list(w.keys()):
+            if x in ('blocks.0.ln0.weight', 'blocks.0.ln0.bias') and not converted:
+                continue
+            if x == 'emb.weight' and not converted:
+                continue
+            t = w[x]
+            layer_id = int(x.split('.')[1]) if ('blocks.' in x) else 0
+            is_matrix = any(s in x for s in _MATRIX_KEYS) and not x.endswith(('_mx', '_rx', '_my', '_ry'))
+            if converted:
+                if is_matrix:
+                    # reference device layout [in, out] with out contiguous -> input-contiguous
+                    out[x] = _ops.to_input_contiguous(t.to(dev))
+                elif x.endswith(('_mx', '_rx', '_my', '_ry')) or 'emb.' in x:
+                    out[x] = t.to(dev).contiguous()
+                else:
+                    out[x] = t.to(dev).contiguous()
+                continue
+            if is_matrix:
+                t = t.to(device=dev, dtype=torch.float32)
+                if R > 0 and ('att.output.weight' in x or 'ffn.value.weight' in x):
+                    t = t / (2 ** int(layer_id // R))                 # model.py:785-789 (exact scaling)
+                # checkpoint orientation [out, in] row-major == logical [in, out] input-contiguous
+                t = t.contiguous()
+                if u8:
+                    q, mx, rx, my, ry = _ops.quantize_u8(t.t(), scale_dtype=torch.float16, input_contiguous=True)
+                    out[x], out[x + '_mx'], out[x + '_rx'], out[x + '_my'], out[x + '_ry'] = q, mx, rx, my, ry
+                else:
+                    out[x] = t.to(torch.float16).t()
+                del t
+                continue
+            t = t.detach().to('cpu')
+            if '.time_' in x:
+                t = t.squeeze()
+            if '.time_decay' in x and '_w' not in x:
+                t = -torch.exp(t.float())                             # model.py:797-798
+            elif '.time_first' in x:
+                t = t.float()                                         # model.py:806-807
+            else:
+                t = t.to(torch.float16)                               # model.py:849
+            out[x] = t.contiguous().to(dev)
+        torch.cuda.synchronize()
+        return out
+
+    def _save_converted(self, path, prxxx):
+        """model.py:894-903: the converted dict in the reference's own layout ([in, out] matrices
+        with the output index contiguous) so that either implementation can load the file."""
+        if not path.endswith('.pth'):
+            path += '.pth'
+        sd = {}
+        for k, v in self.w.items():
+            v = v.detach()
+            is_matrix = any(s in k for s in _MATRIX_KEYS) and not k.endswith(('_mx', '_rx', '_my', '_ry'))
+            sd[k] = (v.contiguous() if is_matrix else v).cpu()
+        sd['_strategy'] = self.args.strategy_string
+        sd['_rescale_layer'] = self.RESCALE_LAYER
+        sd['_version'] = '0.7'
+        prxxx(f'Saving to {path}...')
+        torch.save(sd, path)
+        prxxx('Converted and saved. Now this will exit.')
+
+    def _mat(self, name):
+        w = self.w
+        t = w[name]
+        N, M = t.shape
+        assert t.stride(0) == 1, name
+        m = _lib.RwkvMat()
+        m.w, m.ld, m.N, m.M = t.data_ptr(), t.stride(1), N, M
+        if t.dtype == torch.uint8:
+            m.mx, m.rx = w[name + '_mx'].data_ptr(), w[name + '_rx'].data_ptr()
+            m.my, m.ry = w[name + '_my'].data_ptr(), w[name + '_ry'].data_ptr()
+        return m
+
+    def _build_descriptors(self):
+        a, w = self.args, self.w
+        layers = (_lib.RwkvV4Layer * a.n_layer)()
+        for i in range(a.n_layer):
+            b, at, ff = f'blocks.{i}.', f'blocks.{i}.att.', f'blocks.{i}.ffn.'
+            l = layers[i]
+            l.ln1_w, l.ln1_b = w[b + 'ln1.weight'].data_ptr(), w[b + 'ln1.bias'].data_ptr()
+            l.ln2_w, l.ln2_b = w[b + 'ln2.weight'].data_ptr(), w[b + 'ln2.bias'].data_ptr()
+            l.att_mix_k, l.att_mix_v, l.att_mix_r = (w[at + 'time_mix_' + c].data_ptr() for c in 'kvr')
+            l.time_decay, l.time_first = w[at + 'time_decay'].data_ptr(), w[at + 'time_first'].data_ptr()
+            l.att_key, l.att_value = self._mat(at + 'key.weight'), self._mat(at + 'value.weight')
+            l.att_receptance, l.att_output = self._mat(at + 'receptance.weight'), self._mat(at + 'output.weight')
+            l.ffn_mix_k, l.ffn_mix_r = w[ff + 'time_mix_k'].data_ptr(), w[ff + 'time_mix_r'].data_ptr()
+            l.ffn_key, l.ffn_receptance = self._mat(ff + 'key.weight'), self._mat(ff + 'receptance.weight')
+            l.ffn_value = self._mat(ff + 'value.weight')
+        m = _lib.RwkvV4Model()
+        m.n_layer, m.n_embd, m.n_ffn = a.n_layer, a.n_embd, a.n_ffn
+        m.vocab = w['emb.weight'].shape[0]
+        m.rescale_layer = self.RESCALE_LAYER
+        m.weights_u8 = 1 if self._wkind == 'u8' else 0
+        m.emb = w['emb.weight'].data_ptr()
+        m.ln_out_w, m.ln_out_b = w['ln_out.weight'].data_ptr(), w['ln_out.bias'].data_ptr()
+        m.head = self._mat('head.weight')
+        m.layers = layers
+        self._layers, self._model = layers, m
+        L = _lib.load()
+        nbytes = L.rwkv_v4_one_workspace(ctypes.byref(m))
+        self._one_ws = torch.empty(nbytes, dtype=torch.uint8, device=self.device)
+        self._token_dev = torch.zeros(1, dtype=torch.int32, device=self.device)
+        self._logits = torch.empty(m.vocab, dtype=torch.float32, device=self.device)
+
+    # ------------------------------------------------------------------ state
+    def _new_state(self):
+        """model.py:1448-1459: per layer [xx fp16 (C), aa, bb fp32 (C), pp fp32 = -1e30, ffn_xx fp16 (C)],
+        carved from two flat buffers."""
+        a, dev = self.args, self.device
+        C, L = a.n_embd, a.n_layer
+        f16 = torch.zeros(L * 2 * C, dtype=torch.float16, device=dev)
+        f32 = torch.zeros(L * 3 * C, dtype=torch.float32, device=dev)
+        st = StateList()
+        for i in range(L):
+            st.append(f16[(2 * i) * C:(2 * i + 1) * C])
+            st.append(f32[(3 * i) * C:(3 * i + 1) * C])
+            st.append(f32[(3 * i + 1) * C:(3 * i + 2) * C])
+            pp = f32[(3 * i + 2) * C:(3 * i + 3) * C]
+            pp.fill_(-1e30)
+            st.append(pp)
+            st.append(f16[(2 * i + 1) * C:(2 * i + 2) * C])
+        st.flat = (f16, f32)
+        st.views = list(st)
+        return st
+
+    def _state_desc(self, state):
+        a = self.args
+        if len(state) != 5 * a.n_layer:
+            raise ValueError(f"state must hold {5 * a.n_layer} tensors")
+        arr = (_lib.RwkvV4LayerState * a.n_layer)()
+        for i in range(a.n_layer):
+            xx, aa, bb, pp, fx = state[5 * i:5 * i + 5]
+            for t, dt in ((xx, torch.float16), (aa, torch.float32), (bb, torch.float32), (pp, torch.float32),
+                          (fx, torch.float16)):
+                if not (t.is_cuda and t.dtype == dt and t.is_contiguous() and t.numel() == a.n_embd):
+                    raise ValueError("state tensors must be contiguous GPU tensors with the layout of model.py:1448-1459")
+            s = arr[i]
+            s.att_xx, s.aa, s.bb, s.pp, s.ffn_xx = (t.data_ptr() for t in (xx, aa, bb, pp, fx))
+        return arr
+
+    # ------------------------------------------------------------------ forward
+    def _launch_one(self, sdesc):
+        L = _lib.load()
+        rc = L.rwkv_v4_forward_one(ctypes.byref(self._model), sdesc, self._token_dev.data_ptr(),
+                                   self._logits.data_ptr(), self._one_ws.data_ptr(), self._one_ws.numel(),
+                                   torch.cuda.current_stream().cuda_stream)
+        _lib.check(rc, "rwkv_v4_forward_one")
+
+    def _forward_one(self, token, state):
+        if isinstance(token, torch.Tensor):
+            self._token_dev.copy_(token.reshape(1), non_blocking=True)
+        else:
+            # the id travels as a kernel argument of the fill: no host buffer that a later call
+            # could overwrite while this one is still queued
+            self._token_dev.fill_(int(token))
+        use_graph = os.environ.get("RWKV_HIP_GRAPH", "1") != "0"
+        key = None
+        if use_graph and isinstance(state, StateList) and state.intact():
+            key = tuple(t.data_ptr() for t in state.flat)
+        if key is None:
+            self._launch_one(self._state_desc(state))
+            return self._logits.clone(), state
+        entry = self._graphs.get(key)
+        if entry is None:
+            sdesc = self._state_desc(state)
+            # warm-up outside capture must not advance the state: run it on a scratch copy
+            scratch = self._new_state()
+            self._launch_one(self._state_desc(scratch))
+            torch.cuda.synchronize()
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                self._launch_one(sdesc)
+            entry = (g, sdesc, state.flat)
+            self._graphs[key] = entry
+            while len(self._graphs) > 8:
+                self._graphs.popitem(last=False)
+        else:
+            self._graphs.move_to_end(key)
+        entry[0].replay()
+        return self._logits.clone(), state
+
+    def _forward_seq(self, tokens, state, full_output):
+        L = _lib.load()
+        T = len(tokens)
+        tok = torch.tensor(tokens, dtype=torch.int32).to(self.device)
+        nbytes = L.rwkv_v4_seq_workspace(ctypes.byref(self._model), T, int(full_output))
+        if self._seq_ws is None or self._seq_ws.numel() < nbytes:
+            self._seq_ws = None
+            self._seq_ws = torch.empty(nbytes, dtype=torch.uint8, device=self.device)
+        V = self._model.vocab
+        logits = torch.empty((T, V) if full_output else (V,), dtype=torch.float32, device=self.device)
+        rc = L.rwkv_v4_forward_seq(ctypes.byref(self._model), self._state_desc(state), tok.data_ptr(), T,
+                                   int(full_output), logits.data_ptr(), self._seq_ws.data_ptr(),
+                                   self._seq_ws.numel(), torch.cuda.current_stream().cuda_stream)
+        _lib.check(rc, "rwkv_v4_forward_seq")
+        return logits, state
+
+    def forward(self, tokens, state, full_output=False):
+        """model.py:1443-1677.  Returns (logits fp32 [vocab] or [T, vocab], state)."""
+        with torch.no_grad():
+            if state is None:
+                state = self._new_state()
+            if isinstance(tokens, torch.Tensor):
+                if tokens.numel() == 1:
+                    return self._forward_one(tokens if tokens.is_cuda else int(tokens), state)
+                tokens = tokens.tolist()
+            tokens = [int(t) for t in tokens]
+            V = self._model.vocab
+            if any(t < 0 or t >= V for t in tokens):
+                raise IndexError("token id out of range")
+            if len(tokens) == 1:
+                return self._forward_one(tokens[0], state)
+            return self._forward_seq(tokens, state, full_output)

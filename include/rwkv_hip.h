@@ -123,6 +123,69 @@ int rwkv_wkv6_forward(int64_t B, int64_t T, int64_t C, int64_t H, float *state, 
                       const float *r, const float *k, const float *v, const float *w, const float *u,
                       float *y, void *stream);
 
+/* Row-wise LayerNorm of an fp32 [T, C] matrix with fp32 affine, fp16 output (eps 1e-5).
+ * Used once at load time for emb <- LayerNorm(emb; ln0) (model.py:756), which the reference
+ * computes with F.layer_norm on the CPU. */
+int rwkv_layernorm_f32_f16(int64_t T, int64_t C, const float *x, const float *w, const float *b,
+                           rwkv_half *y, void *stream);
+
+/* =======================================================================================
+ * Model-level entry points: one call runs RWKV.forward (model.py:1443-1677) for RWKV-4 on
+ * one GPU, with the elementwise chains of att_one / ffn_one / cuda_att_seq / ffn_seq
+ * (model.py:984-1004, 1034-1055, 1346-1360) folded into the GEMV / GEMM prologues and
+ * epilogues.  The structs below are plain host memory filled by the caller; every pointer
+ * inside them is a device pointer.  Matrices are input-contiguous (see the top of this file):
+ * uint8 with fp16 mx/rx/my/ry under 'cuda fp16i8', fp16 with NULL scales under 'cuda fp16'.
+ */
+typedef struct {
+    const void *w;       /* uint8 or fp16, row m = N consecutive elements at w + m * ld */
+    int64_t ld;          /* elements between consecutive output rows */
+    const rwkv_half *mx, *rx, *my, *ry; /* NULL for fp16 weights */
+    int64_t N, M;
+} rwkv_mat;
+
+typedef struct {
+    const rwkv_half *ln1_w, *ln1_b, *ln2_w, *ln2_b;               /* [C] */
+    const rwkv_half *att_mix_k, *att_mix_v, *att_mix_r;           /* [C] */
+    const float *time_decay, *time_first;                         /* [C] fp32; decay = -exp(raw) */
+    rwkv_mat att_key, att_value, att_receptance, att_output;      /* [C -> C] */
+    const rwkv_half *ffn_mix_k, *ffn_mix_r;                       /* [C] */
+    rwkv_mat ffn_key, ffn_receptance, ffn_value;                  /* [C -> F], [C -> C], [F -> C] */
+} rwkv_v4_layer;
+
+typedef struct {
+    rwkv_half *att_xx;      /* [C] fp16 */
+    float *aa, *bb, *pp;    /* [C] fp32 */
+    rwkv_half *ffn_xx;      /* [C] fp16 */
+} rwkv_v4_layer_state;
+
+typedef struct {
+    int32_t n_layer, n_embd, n_ffn, vocab;
+    int32_t rescale_layer;  /* x /= 2 after every rescale_layer-th layer; 0 = never (model.py:1660-1662) */
+    int32_t weights_u8;     /* 1: uint8 matrices ('cuda fp16i8'); 0: fp16 matrices ('cuda fp16') */
+    const rwkv_half *emb;   /* [vocab, C] fp16, ln0 already applied (model.py:756) */
+    const rwkv_half *ln_out_w, *ln_out_b;
+    rwkv_mat head;          /* [C -> vocab] */
+    const rwkv_v4_layer *layers; /* host array [n_layer] */
+} rwkv_v4_model;
+
+/* One-token step (len(tokens) == 1).  `token` is a device int32: the kernels read the id from
+ * device memory so that a captured graph can be replayed with a new token.  `states` is a host
+ * array [n_layer]; all state tensors are updated in place.  logits: fp32 [vocab] (values are
+ * fp16-rounded as in model.py:86, 1675-1677).  workspace: rwkv_v4_one_workspace() bytes.
+ * Only launches kernels (no memset / memcpy nodes): safe to capture into a HIP graph. */
+size_t rwkv_v4_one_workspace(const rwkv_v4_model *m);
+int rwkv_v4_forward_one(const rwkv_v4_model *m, const rwkv_v4_layer_state *states, const int32_t *token,
+                        float *logits, void *workspace, size_t workspace_bytes, void *stream);
+
+/* Sequence mode (len(tokens) > 1): tokens is a device int32 [T].  logits: fp32 [vocab] for the
+ * last token, or [T, vocab] when full_output != 0.  workspace: rwkv_v4_seq_workspace(m, T,
+ * full_output) bytes. */
+size_t rwkv_v4_seq_workspace(const rwkv_v4_model *m, int64_t T, int full_output);
+int rwkv_v4_forward_seq(const rwkv_v4_model *m, const rwkv_v4_layer_state *states, const int32_t *tokens,
+                        int64_t T, int full_output, float *logits, void *workspace, size_t workspace_bytes,
+                        void *stream);
+
 #ifdef __cplusplus
 }
 #endif

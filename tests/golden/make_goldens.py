@@ -14,6 +14,7 @@ RWKV_CUDA_ON=0 (no native build), feeds it synthetic checkpoints from
   e2e_<ver>_<strategy>.npz  logits (full_output over a 9-token prompt, then chunked calls
                             and one-token calls) and the final state, tiny models of
                             RWKV-4 / 5.0 / 5.1 / 5.2 / 6.0 under 'cpu fp32i8' and 'cpu fp32'
+  planner.json              the per-slot plan the reference prints for a list of strategy strings
   e2e_v4_169m_cpu_fp32i8.npz  the 169M-shape model: 128-token prefill + 32 greedy steps;
                             argmax per position, 256 fixed logits per position, state sums
 Only outputs and seeds are stored; no reference source is copied.
@@ -155,10 +156,46 @@ def e2e_169m(tmp):
     print("wrote e2e_v4_169m_cpu_fp32i8.npz")
 
 
+PLAN_STRATEGIES = [
+    "cuda fp16i8", "cuda fp16", "cpu fp32i8", "cpu fp32", "cuda:0 fp16i8", "cuda fp16i8 *10 -> cuda fp16",
+    "cuda fp16 *10+", "cuda:0 fp16 *20 -> cuda:1 fp16", "cuda fp16i8 *1 -> cuda fp16", "cuda fp16i8 -> cpu fp32 *1",
+    "cuda fp16 *0+ -> cpu fp32 *1", "cuda fp16i8 *4 -> cuda fp16 *3 -> cpu fp32", "cuda fp16 *6+",
+    "cuda fp16i8 *2 -> cuda fp16 *2+ -> cpu fp32 *1", "cuda fp16 -> cuda:1 fp16", "cpu bf16", "cuda fp16i8 *100",
+    "cuda fp16 *3 -> cuda:1 fp16 *3 -> cpu fp32",
+]
+
+
+def planner(tmp):
+    """The per-slot plan the reference prints (model.py:726-750) for a list of strategy strings,
+    on an 8-layer model.  The loader later fails where it moves tensors to a GPU that is not there;
+    the plan is printed before that."""
+    ck = synth.make_checkpoint(version=4, seed=102, **TINY8)
+    p = os.path.join(tmp, "tiny8p.pth")
+    _save_ckpt(ck, p)
+    out = {}
+    for strat in PLAN_STRATEGIES:
+        code = (
+            "import os, sys\n"
+            "os.environ['RWKV_CUDA_ON']='0'\n"
+            f"sys.path.insert(0, {REF_SRC!r})\n"
+            "from rwkv.model import RWKV\n"
+            f"RWKV({p!r}, {strat!r}, verbose=True)\n"
+        )
+        r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True)
+        line = [l for l in r.stdout.splitlines() if l.startswith("0-")]
+        out[strat] = line[0].strip() if line else "ERROR"
+    import json
+    with open(os.path.join(HERE, "planner.json"), "w") as f:
+        json.dump({"n_layer": TINY8["n_layer"], "plans": out}, f, indent=1)
+    print("wrote planner.json")
+
+
 if __name__ == "__main__":
     torch.manual_seed(0)
     with tempfile.TemporaryDirectory() as tmp:
-        which = sys.argv[1:] or ["quant_cpu", "quant_cuda", "tiny", "169m"]
+        which = sys.argv[1:] or ["quant_cpu", "quant_cuda", "tiny", "169m", "planner"]
+        if "planner" in which:
+            planner(tmp)
         if "quant_cpu" in which:
             quant_cpu(tmp)
         if "quant_cuda" in which:
