@@ -1,0 +1,208 @@
+"""Headline benchmark: RWKV-4 7B-shape 'cuda fp16i8', batch 1, on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--shape v4-7b] [--no-cpu]
+
+Workload (BASELINE.json configs[2]): random-init 32-layer / n_embd 4096 / ffn 16384 / vocab
+50277 model, prefill of 1024 uniform-random tokens in one call, then greedy decode.  A "step"
+is one decoded token (one pass of forward([token], state)); W untimed steps, then exactly K
+timed steps with the next token taken on the device (argmax) so the loop has no host
+synchronisation; the same K steps are also timed with a host sync per token.
+
+One JSON line is printed:
+  value / ms_per_step   decode tokens/s (device-token loop) and ms per token
+  roofline              the dominant decode kernel (channel-mix receptance+key GEMV): algorithmic
+                        bytes per launch / mean launch duration from HIP events around every launch
+                        (rwkv_v4_profile_one), against the 8 TB/s HBM peak
+  decode_hbm            whole-step figure: uint8 weight bytes per token x tokens/s / 8 TB/s
+  prefill               prefill tokens/s and the MFMA fraction of the whole prefill
+  cpu_baseline          the oracle's 'cpu fp32i8' path (numpy port of the reference's CPU arithmetic)
+                        timed on this host: a bounded sample at the 7B shape, extrapolated per token
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK = 8.0e12      # bytes/s, MI355X HBM3E
+MFMA_F16_PEAK = 2.5e15  # flop/s dense fp16
+
+
+def u8_weight_bytes(L, C, F, V):
+    return L * (5 * C * C + 2 * C * F) + C * V
+
+
+def cpu_baseline(shape, budget_s=25.0):
+    """Oracle 'cpu fp32i8' (dequantise the whole matrix per call, fp32 matvec: the reference's
+    CPU path) on a bounded sample: ONE layer of the named shape plus the head, a few tokens;
+    per-token time of the full model = n_layer * t_layer + t_head."""
+    import numpy as np
+    from chatrwkv_amd import synth
+    from oracle import ops as oops
+    from oracle.model import OracleRWKV
+    try:
+        from threadpoolctl import threadpool_info
+        threads = max([p.get("num_threads", 1) for p in threadpool_info()] + [1])
+    except Exception:
+        threads = os.cpu_count() or 1
+    version, L, C, F, V = synth.SHAPES[shape]
+    t0 = time.perf_counter()
+    # converted weights filled with random bytes/scales: the CPU path's speed does not depend on values
+    o = OracleRWKV.random_converted_v4(1, C, F, V, seed=0)
+    setup = time.perf_counter() - t0
+    st = o.init_state()
+    x = o.w["emb.weight"][[1]].astype(np.float32)
+    # warm-up token, then timed tokens through the single layer and through the head
+    tl, th = [], []
+    deadline = time.perf_counter() + budget_s
+    for it in range(5):
+        a = time.perf_counter()
+        y, st[0], st[1], st[2], st[3] = o._att_v4(x, st[0], st[1], st[2], st[3], 0)
+        y, st[4] = o._ffn(y, st[4], 0)
+        b = time.perf_counter()
+        z = oops.layer_norm(y, o.w["ln_out.weight"], o.w["ln_out.bias"])
+        z = oops.matmul(z, o.mat("head.weight"), o.atype, cache=False)
+        c = time.perf_counter()
+        if it > 0:
+            tl.append(b - a)
+            th.append(c - b)
+        if time.perf_counter() > deadline and len(tl) >= 2:
+            break
+    t_layer, t_head = float(np.median(tl)), float(np.median(th))
+    per_token = L * t_layer + t_head
+    return {
+        "value": 1.0 / per_token, "unit": "tok/s", "cores": int(threads), "kind": "port",
+        "sample": (f"{shape}: {len(tl)} tokens through 1 of {L} layers + head, numpy oracle 'cpu fp32i8' "
+                   f"(whole-matrix dequantisation per call, single-threaded elementwise + {threads}-thread BLAS); "
+                   f"t_layer {t_layer * 1e3:.0f} ms, t_head {t_head * 1e3:.0f} ms, "
+                   f"per token = {L} x t_layer + t_head = {per_token:.2f} s; setup {setup:.0f} s"),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=256)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--shape", default="v4-7b")
+    ap.add_argument("--strategy", default="cuda fp16i8")
+    ap.add_argument("--prefill", type=int, default=1024)
+    ap.add_argument("--layers", type=int, default=None, help="debug: fewer layers (result is then not the headline)")
+    ap.add_argument("--no-cpu", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs on ONE GPU; the path has no multi-GPU mode (--gpus must be 1)",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+    from chatrwkv_amd import synth
+    from chatrwkv_amd.model import RWKV
+
+    version, L, C, F, V = synth.SHAPES[args.shape]
+    if args.layers:
+        L = args.layers
+    dev = "cuda:0"
+    torch.cuda.set_device(0)
+    ck = synth.make_checkpoint(version=version, n_layer=L, n_embd=C, n_ffn=F, vocab=V, seed=2, device=dev)
+    model = RWKV(ck, args.strategy, verbose=False)
+    del ck
+    torch.cuda.empty_cache()
+    u8 = args.strategy.endswith("i8")
+    wbytes = u8_weight_bytes(L, C, F, V) * (1 if u8 else 2)
+
+    # ---- prefill: one call over `prefill` tokens (median of 3, after one warm-up call)
+    ptoks = synth.random_tokens(args.prefill, V, seed=2)
+    model.forward(ptoks, None)
+    torch.cuda.synchronize()
+    pt = []
+    for _ in range(3):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        out, state = model.forward(ptoks, None)
+        e1.record()
+        torch.cuda.synchronize()
+        pt.append(e0.elapsed_time(e1) * 1e-3)
+    t_prefill = float(np.median(pt))
+    prefill_flops = 2.0 * args.prefill * (wbytes / (1 if u8 else 2) - C * V) + 2.0 * C * V
+
+    # ---- decode: W warm-up + K timed greedy steps, token stays on the device
+    tok = out.argmax().reshape(1).to(torch.int32)
+    for _ in range(args.warmup):
+        out, state = model.forward(tok, state)
+        tok = out.argmax().reshape(1).to(torch.int32)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        out, state = model.forward(tok, state)
+        tok = out.argmax().reshape(1).to(torch.int32)
+    torch.cuda.synchronize()
+    t_dev = time.perf_counter() - t0
+
+    # the same K steps with the token fetched to the host every step (what a sampling caller does)
+    t0 = time.perf_counter()
+    nxt = int(tok)
+    for _ in range(args.steps):
+        out, state = model.forward([nxt], state)
+        nxt = int(out.argmax())
+    torch.cuda.synchronize()
+    t_host = time.perf_counter() - t0
+
+    # ---- per-kernel durations from HIP events around every launch (not under graph replay)
+    per = []
+    for _ in range(8):
+        out, state, ms = model.profile_one(nxt, state)
+        nxt = int(out.argmax())
+        per.append(ms)
+    per = np.array(per[2:])  # drop two warm-up steps
+    names = ["att_kvr_wkv", "att_output", "ffn_rk", "ffn_value"]
+    scale = 1 if u8 else 2
+    kbytes = {"att_kvr_wkv": 3 * C * C * scale, "att_output": C * C * scale, "ffn_rk": (C * C + C * F) * scale,
+              "ffn_value": C * F * scale, "head": C * V * scale}
+    kms = {n: float(per[:, j:4 * L:4].mean()) for j, n in enumerate(names)}
+    kms["head"] = float(per[:, -1].mean())
+    ktot = {n: kms[n] * (L if n != "head" else 1) for n in kms}
+    dom = max(ktot, key=ktot.get)
+    kernels = {n: {"ms": round(kms[n], 5), "bytes": kbytes[n], "GBps": round(kbytes[n] / (kms[n] * 1e-3) / 1e9, 1)}
+               for n in kms}
+
+    tok_s = args.steps / t_dev
+    res = {
+        "metric": "7B fp16i8 decode tok/s (% HBM peak) + prefill tok/s, 1 MI355X",
+        "value": tok_s, "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": 1e3 * t_dev / args.steps, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "u8 weights, fp16 activations, fp32 accumulate" if u8 else "fp16",
+        "data": "synthetic (random-init weights, random tokens)",
+        "config": {"workload": f"RWKV-4 {args.shape} ({L} layers, n_embd {C}, ffn {F}, vocab {V}) '{args.strategy}', "
+                               f"batch 1: prefill {args.prefill} tokens in one call, then greedy decode "
+                               f"(BASELINE.json configs[2])",
+                   "strategy": args.strategy, "prefill_tokens": args.prefill},
+        "roofline": {
+            "bound": "hbm", "kernel": {"att_kvr_wkv": "att_kernel", "att_output": "vec_kernel", "ffn_rk": "lnmix_kernel",
+                                        "ffn_value": "vec_kernel", "head": "lnmix_kernel"}[dom] + f" ({dom})",
+            "achieved": kbytes[dom] / (kms[dom] * 1e-3) / 1e9, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+            "frac": kbytes[dom] / (kms[dom] * 1e-3) / HBM_PEAK, "traffic": None,
+            "bytes_per_launch": kbytes[dom], "ms_per_launch": kms[dom],
+        },
+        "decode_hbm": {"weight_bytes_per_token": wbytes, "achieved_GBps": wbytes * tok_s / 1e9,
+                       "frac_of_peak": wbytes * tok_s / HBM_PEAK},
+        "decode_tok_s_host_sync": args.steps / t_host,
+        "decode_kernels": kernels,
+        "prefill": {"tokens": args.prefill, "tok_s": args.prefill / t_prefill, "ms": 1e3 * t_prefill,
+                    "flops": prefill_flops, "TFLOPs": prefill_flops / t_prefill / 1e12,
+                    "frac_of_mfma_peak": prefill_flops / t_prefill / MFMA_F16_PEAK},
+    }
+    if not args.no_cpu:
+        res["cpu_baseline"] = cpu_baseline(args.shape)
+    else:
+        res["cpu_baseline"] = None
+    print(json.dumps(res))
+
+
+if __name__ == "__main__":
+    main()

@@ -411,8 +411,10 @@ int v4_head_launch(const rwkv_v4_model *m, const rwkv_half *x, float *logits, hi
     return RWKV_OK;
 }
 
-extern "C" int rwkv_v4_forward_one(const rwkv_v4_model *m, const rwkv_v4_layer_state *states, const int32_t *token,
-                                   float *logits, void *workspace, size_t workspace_bytes, void *stream) {
+// `ev` (optional): 4 * n_layer + 2 events; ev[0] is recorded before the first launch and
+// ev[i + 1] after the i-th launch.
+static int v4_one_impl(const rwkv_v4_model *m, const rwkv_v4_layer_state *states, const int32_t *token,
+                       float *logits, void *workspace, size_t workspace_bytes, void *stream, hipEvent_t *ev) {
     int rc = v4_model_check(m);
     if (rc) return rc;
     if (!states || !token || !logits || !workspace) return RWKV_E_NULL;
@@ -435,6 +437,9 @@ extern "C" int rwkv_v4_forward_one(const rwkv_v4_model *m, const rwkv_v4_layer_s
     ws.xx_ffn = (rwkv_half *)p; p += cb;
     ws.vx = (rwkv_half *)p;
     const int grid = num_cu();
+    int nev = 0;
+    auto mark = [&]() { if (ev) (void)hipEventRecord(ev[nev++], st); };
+    mark();
 
     for (int i = 0; i < m->n_layer; ++i) {
         const rwkv_v4_layer &l = m->layers[i];
@@ -451,6 +456,7 @@ extern "C" int rwkv_v4_forward_one(const rwkv_v4_model *m, const rwkv_v4_layer_s
             const size_t lds = 3 * (size_t)C * 2;
             if (u8) hipLaunchKernelGGL(att_kernel<true>, dim3(grid), dim3(DTHREADS), lds, st, a);
             else hipLaunchKernelGGL(att_kernel<false>, dim3(grid), dim3(DTHREADS), lds, st, a);
+            mark();
         }
         {
             VecArgs a{};
@@ -460,6 +466,7 @@ extern "C" int rwkv_v4_forward_one(const rwkv_v4_model *m, const rwkv_v4_layer_s
             const size_t lds = (size_t)C * 2;
             if (u8) hipLaunchKernelGGL((vec_kernel<true, 4>), dim3(grid), dim3(DTHREADS), lds, st, a);
             else hipLaunchKernelGGL((vec_kernel<false, 4>), dim3(grid), dim3(DTHREADS), lds, st, a);
+            mark();
         }
         {
             LnMixArgs a{};
@@ -471,6 +478,7 @@ extern "C" int rwkv_v4_forward_one(const rwkv_v4_model *m, const rwkv_v4_layer_s
             const size_t lds = 2 * (size_t)C * 2;
             if (u8) hipLaunchKernelGGL((lnmix_kernel<true, 2, 2>), dim3(grid), dim3(DTHREADS), lds, st, a);
             else hipLaunchKernelGGL((lnmix_kernel<false, 2, 2>), dim3(grid), dim3(DTHREADS), lds, st, a);
+            mark();
         }
         {
             VecArgs a{};
@@ -481,8 +489,38 @@ extern "C" int rwkv_v4_forward_one(const rwkv_v4_model *m, const rwkv_v4_layer_s
             const size_t lds = (size_t)F * 2;
             if (u8) hipLaunchKernelGGL((vec_kernel<true, 4>), dim3(grid), dim3(DTHREADS), lds, st, a);
             else hipLaunchKernelGGL((vec_kernel<false, 4>), dim3(grid), dim3(DTHREADS), lds, st, a);
+            mark();
         }
         RWKV_LAUNCH_CHECK();
     }
-    return v4_head_launch(m, ws.x, logits, st);
+    rc = v4_head_launch(m, ws.x, logits, st);
+    mark();
+    return rc;
+}
+
+extern "C" int rwkv_v4_forward_one(const rwkv_v4_model *m, const rwkv_v4_layer_state *states, const int32_t *token,
+                                   float *logits, void *workspace, size_t workspace_bytes, void *stream) {
+    return v4_one_impl(m, states, token, logits, workspace, workspace_bytes, stream, nullptr);
+}
+
+extern "C" int rwkv_v4_profile_one(const rwkv_v4_model *m, const rwkv_v4_layer_state *states, const int32_t *token,
+                                   float *logits, void *workspace, size_t workspace_bytes, void *stream,
+                                   float *ms, int64_t n_ms) {
+    if (!m || !ms) return RWKV_E_NULL;
+    const int n = 4 * m->n_layer + 1;
+    if (n_ms < n) return RWKV_E_SHAPE;
+    hipEvent_t *ev = new hipEvent_t[n + 1];
+    int made = 0, rc = RWKV_OK;
+    for (; made < n + 1; ++made)
+        if (hipEventCreate(&ev[made]) != hipSuccess) { rc = (int)hipErrorOutOfMemory; break; }
+    if (rc == RWKV_OK) rc = v4_one_impl(m, states, token, logits, workspace, workspace_bytes, stream, ev);
+    if (rc == RWKV_OK) {
+        hipError_t e = hipEventSynchronize(ev[n]);
+        if (e != hipSuccess) rc = (int)e;
+        for (int i = 0; i < n && rc == RWKV_OK; ++i)
+            if (hipEventElapsedTime(&ms[i], ev[i], ev[i + 1]) != hipSuccess) rc = (int)hipErrorInvalidValue;
+    }
+    for (int i = 0; i < made; ++i) (void)hipEventDestroy(ev[i]);
+    delete[] ev;
+    return rc;
 }

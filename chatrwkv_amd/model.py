@@ -329,6 +329,22 @@ class RWKV:
         entry[0].replay()
         return self._logits.clone(), state
 
+    def profile_one(self, token, state):
+        """One-token step with a HIP event around every kernel launch (rwkv_v4_profile_one).
+        Returns (logits, state, ms) with ms[4 * i + j] the j-th launch of layer i and ms[-1] the head."""
+        with torch.no_grad():
+            if state is None:
+                state = self._new_state()
+            self._token_dev.fill_(int(token))
+            n = 4 * self.args.n_layer + 1
+            ms = (ctypes.c_float * n)()
+            rc = _lib.load().rwkv_v4_profile_one(ctypes.byref(self._model), self._state_desc(state),
+                                                 self._token_dev.data_ptr(), self._logits.data_ptr(),
+                                                 self._one_ws.data_ptr(), self._one_ws.numel(),
+                                                 torch.cuda.current_stream().cuda_stream, ms, n)
+            _lib.check(rc, "rwkv_v4_profile_one")
+            return self._logits.clone(), state, list(ms)
+
     def _forward_seq(self, tokens, state, full_output):
         L = _lib.load()
         T = len(tokens)

@@ -178,6 +178,15 @@ size_t rwkv_v4_one_workspace(const rwkv_v4_model *m);
 int rwkv_v4_forward_one(const rwkv_v4_model *m, const rwkv_v4_layer_state *states, const int32_t *token,
                         float *logits, void *workspace, size_t workspace_bytes, void *stream);
 
+/* Measurement aid: the same step as rwkv_v4_forward_one with a HIP event recorded on `stream`
+ * around every kernel launch.  Blocks until the step has finished and writes the elapsed
+ * milliseconds of the 4 * n_layer + 1 launches to ms[] in launch order: per layer (time-mix
+ * k/v/r + WKV, time-mix output, channel-mix r/k, channel-mix value), then the head.
+ * Not capturable (it synchronises). */
+int rwkv_v4_profile_one(const rwkv_v4_model *m, const rwkv_v4_layer_state *states, const int32_t *token,
+                        float *logits, void *workspace, size_t workspace_bytes, void *stream,
+                        float *ms, int64_t n_ms);
+
 /* Sequence mode (len(tokens) > 1): tokens is a device int32 [T].  logits: fp32 [vocab] for the
  * last token, or [T, vocab] when full_output != 0.  workspace: rwkv_v4_seq_workspace(m, T,
  * full_output) bytes. */

@@ -53,6 +53,47 @@ class OracleRWKV:
         self.cache = (self.device != 'cpu') if cache_dequant is None else cache_dequant
         self._convert({k: _np(v) for k, v in checkpoint.items()})
 
+    @classmethod
+    def random_converted_v4(cls, n_layer, n_embd, n_ffn, vocab, seed=0):
+        """A 'cpu fp32i8' RWKV-4 oracle whose *converted* weights are filled directly with uniform
+        random bytes and plausible scales, skipping the (slow, CPU) quantizer.  For timing the CPU
+        path only: its speed does not depend on the weight values."""
+        self = object.__new__(cls)
+        self.device, self.atype, self.wtype = 'cpu', f32, np.uint8
+        self.rescale_layer, self.cache = 0, False
+        self.n_embd = self.n_att = n_embd
+        self.n_ffn, self.n_layer, self.version, self.n_head = n_ffn, n_layer, 4, 0
+        rng = np.random.Generator(np.random.PCG64(seed))
+        C, F, V = n_embd, n_ffn, vocab
+        w = {'emb.weight': rng.standard_normal((16, C), dtype=f32)}
+
+        def qmat(name, N, M):
+            w[name] = rng.integers(0, 256, size=(N, M), dtype=np.uint8)
+            w[name + '_mx'] = (rng.standard_normal(M, dtype=f32) * f32(0.01))
+            w[name + '_rx'] = (rng.random(M, dtype=f32) * f32(0.01) + f32(0.005))
+            w[name + '_my'] = (rng.standard_normal((N, 1), dtype=f32) * f32(0.01))
+            w[name + '_ry'] = (rng.random((N, 1), dtype=f32) * f32(0.03) + f32(0.03))
+
+        for i in range(n_layer):
+            p = f'blocks.{i}.'
+            for ln in ('ln1', 'ln2'):
+                w[p + ln + '.weight'], w[p + ln + '.bias'] = np.ones(C, f32), np.zeros(C, f32)
+            w[p + 'att.time_decay'] = -np.exp(rng.uniform(-6, -1, C)).astype(f32)
+            w[p + 'att.time_first'] = rng.uniform(-1, 1, C).astype(f32)
+            for m in 'kvr':
+                w[p + 'att.time_mix_' + m] = rng.random(C, dtype=f32)
+            for m in 'kr':
+                w[p + 'ffn.time_mix_' + m] = rng.random(C, dtype=f32)
+            for name in ('key', 'value', 'receptance', 'output'):
+                qmat(p + f'att.{name}.weight', C, C)
+            qmat(p + 'ffn.key.weight', C, F)
+            qmat(p + 'ffn.receptance.weight', C, C)
+            qmat(p + 'ffn.value.weight', F, C)
+        w['ln_out.weight'], w['ln_out.bias'] = np.ones(C, f32), np.zeros(C, f32)
+        qmat('head.weight', C, V)
+        self.w, self._mats = w, {}
+        return self
+
     # ------------------------------------------------------------------ conversion
     def _convert(self, w):
         # model.py:658-680
