@@ -33,10 +33,28 @@ DEV rwkv_half f2h(float v) { return __builtin_bit_cast(rwkv_half, (h16)v); }  //
 DEV float round_h(float v) { return (float)(h16)v; }
 
 // ---- wave / block reductions ---------------------------------------------------------------
-DEV float wave_sum(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
+// Sums use DPP lane permutes (one VALU issue each, no LDS traffic): a butterfly inside each row
+// of 16 lanes (xor 1, xor 2, half-mirror, mirror), then the four row totals are combined
+// through v_readlane.  Every lane gets the result.
+template <int CTRL>
+DEV float dpp_mov(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+DEV float row16_sum(float v) {
+    v += dpp_mov<0xB1>(v);   // quad_perm [1,0,3,2]
+    v += dpp_mov<0x4E>(v);   // quad_perm [2,3,0,1]
+    v += dpp_mov<0x141>(v);  // row_half_mirror
+    v += dpp_mov<0x140>(v);  // row_mirror
     return v;
+}
+DEV float wave_sum(float v) {
+    v = row16_sum(v);
+    const int b = __builtin_bit_cast(int, v);
+    const float r0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 0));
+    const float r1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 16));
+    const float r2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 32));
+    const float r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 48));
+    return (r0 + r1) + (r2 + r3);
 }
 DEV float wave_max(float v) {
 #pragma unroll

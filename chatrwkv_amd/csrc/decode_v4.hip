@@ -8,12 +8,15 @@
 //   vec_kernel    vx * ry                                    -> rows of Wv -> x += r * out  (and x /= 2)
 //   lnmix_kernel  LN_out                                     -> rows of head -> logits
 //
-// Weight loads do not depend on activations, so every wave issues its first batch of row
-// loads, and only then are they consumed against the activation vector that the workgroup
-// has meanwhile built in LDS (each workgroup redoes the O(C) prologue: a few thousand
-// elements served from L2, against hundreds of KiB of weights streamed from HBM).
-// The token-shift state xx is read by every workgroup, so its new value goes to a scratch
-// vector and is committed to the state by workgroup 0 of the *next* launch.
+// A launch is short (3-15 us of streaming), so what matters is the chain of dependent memory
+// round trips, each ~2 us while HBM is saturated.  Every kernel therefore issues ALL its
+// independent loads in its first instructions -- the prologue operands (x, LayerNorm and mix
+// vectors, scales), the epilogue operands of its first rows (rx, mx, state) and the first tile
+// of weights -- and only then starts the reductions: one round trip instead of four.
+// Each workgroup redoes the O(C) prologue (a few thousand elements served from L2) against
+// hundreds of KiB of weights streamed from HBM.  The token-shift state xx is read by every
+// workgroup, so its new value goes to a scratch vector and is committed to the state by
+// workgroup 0 of the *next* launch.
 #include "gemv_core.h"
 #include "kernels.h"
 
@@ -22,31 +25,11 @@ namespace {
 constexpr int DTHREADS = 1024;
 constexpr int DWAVES = DTHREADS / 64;
 constexpr float LN_EPS = 1e-5f;
+constexpr int VP = 4;  // 8-element groups per thread the vector prologue keeps in registers (N <= 32768)
 
 // x for this step: the embedding row of the token (first layer) or the running activation.
 DEV const rwkv_half *resolve_x(const rwkv_half *x, const rwkv_half *emb, const int32_t *token, int C) {
     return token ? emb + (size_t)(*token) * C : x;
-}
-
-// mean / rstd of x[0..C) (fp16), fp32 two-pass; C % 8 == 0.
-DEV void ln_stats(const rwkv_half *x, int C, float *red, float &mean, float &rstd) {
-    float s = 0.f;
-    for (int j8 = threadIdx.x; j8 < (C >> 3); j8 += blockDim.x) {
-        const h16x8 v = *(const h16x8 *)(x + 8 * j8);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) s += (float)v[e];
-    }
-    mean = block_sum(s, red) / C;
-    float q = 0.f;
-    for (int j8 = threadIdx.x; j8 < (C >> 3); j8 += blockDim.x) {
-        const h16x8 v = *(const h16x8 *)(x + 8 * j8);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            const float d = (float)v[e] - mean;
-            q += d * d;
-        }
-    }
-    rstd = rsqrtf(block_sum(q, red) / C + LN_EPS);
 }
 
 // LDS item (16 bytes = 8 halves) index of the 8-element group j8 of an activation vector.
@@ -59,86 +42,196 @@ struct MatDev {
     const rwkv_half *mx, *rx, *my, *ry;
 };
 
-// LN + (optional) token-shift mixes for NJ consumers; fills xs[j] (LDS) and the per-consumer
-// sums.  mix[j] == nullptr means "no mixing" (the consumer sees LN(x) itself).
+// Workgroup sums of K values with ONE barrier: `red` (K * DWAVES floats) must not be in use by
+// an earlier reduction that other waves may still be reading (callers pass disjoint regions).
+// Stage 2 reads one wave's partial per lane (lane l takes wave l % 16: DWAVES == 16 == one DPP
+// row) and finishes with a 16-lane row sum.
+template <int K>
+DEV void block_sum_1b(float (&v)[K], float *red) {
+    static_assert(DWAVES == 16, "stage 2 assumes 16 waves");
+    const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
+#pragma unroll
+    for (int k = 0; k < K; ++k) v[k] = wave_sum(v[k]);
+    if (lane == 0)
+#pragma unroll
+        for (int k = 0; k < K; ++k) red[k * DWAVES + wid] = v[k];
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < K; ++k) v[k] = row16_sum(red[k * DWAVES + (lane & 15)]);
+}
+
+// LayerNorm + token-shift mixes for NJ consumers, operands staged in registers.
+// Requires C / 8 <= DTHREADS (C <= 8192): thread t owns elements [8t, 8t + 8).
 template <bool U8, int NJ>
-DEV void ln_mix_prologue(const rwkv_half *x, int C, const rwkv_half *ln_w, const rwkv_half *ln_b,
-                         const rwkv_half *sx, const rwkv_half *const (&mix)[NJ], const MatDev (&mat)[NJ],
-                         h16 *const (&xs)[NJ], VecSums (&S)[NJ], rwkv_half *xx_out, float *red) {
-    float mean, rstd;
-    ln_stats(x, C, red, mean, rstd);
-    const int nseg = C >> 4;
-    float acc[3 * NJ];
-#pragma unroll
-    for (int i = 0; i < 3 * NJ; ++i) acc[i] = 0.f;
-    for (int j8 = threadIdx.x; j8 < (C >> 3); j8 += blockDim.x) {
-        const h16x8 xv = *(const h16x8 *)(x + 8 * j8);
-        const h16x8 wv = *(const h16x8 *)(ln_w + 8 * j8);
-        const h16x8 bv = *(const h16x8 *)(ln_b + 8 * j8);
-        h16x8 xx;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) xx[e] = (h16)(((float)xv[e] - mean) * rstd * (float)wv[e] + (float)bv[e]);
-        if (xx_out && blockIdx.x == 0) *(h16x8 *)(xx_out + 8 * j8) = xx;
-        h16x8 pv = xx;
-        if (sx) pv = *(const h16x8 *)(sx + 8 * j8);
+struct LnMixPro {
+    h16x8 x, lw, lb, sx, mix[NJ], ry[NJ], my[NJ];
+    bool own;
+
+    DEV void load(const rwkv_half *xp, int C, const rwkv_half *ln_w, const rwkv_half *ln_b, const rwkv_half *sxp,
+                  const rwkv_half *const (&mixp)[NJ], const MatDev (&mat)[NJ]) {
+        const int j8 = threadIdx.x;
+        own = j8 < (C >> 3);
+        if (!own) return;
+        x = *(const h16x8 *)(xp + 8 * j8);
+        lw = *(const h16x8 *)(ln_w + 8 * j8);
+        lb = *(const h16x8 *)(ln_b + 8 * j8);
+        if (sxp) sx = *(const h16x8 *)(sxp + 8 * j8);
 #pragma unroll
         for (int j = 0; j < NJ; ++j) {
-            h16x8 kx = xx;
-            if (mix[j]) {
-                const h16x8 mv = *(const h16x8 *)(mix[j] + 8 * j8);
-#pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    const float m = (float)mv[e];
-                    kx[e] = (h16)((float)xx[e] * m + (float)pv[e] * (1.f - m));
-                }
-            }
-            h16x8 o = kx;
+            if (mixp[j]) mix[j] = *(const h16x8 *)(mixp[j] + 8 * j8);
             if (U8) {
-                const h16x8 rv = *(const h16x8 *)(mat[j].ry + 8 * j8);
-                const h16x8 yv = *(const h16x8 *)(mat[j].my + 8 * j8);
-#pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    const float k = (float)kx[e];
-                    o[e] = (h16)(k * (float)rv[e]);
-                    acc[3 * j] += k;
-                    acc[3 * j + 1] += (float)o[e];
-                    acc[3 * j + 2] += k * (float)yv[e];
-                }
+                ry[j] = *(const h16x8 *)(mat[j].ry + 8 * j8);
+                my[j] = *(const h16x8 *)(mat[j].my + 8 * j8);
             }
-            ((h16x8 *)xs[j])[xs_item<U8>(j8, nseg)] = o;
         }
     }
-    if (U8) {
-        block_sum_n<3 * NJ>(acc, red);
-#pragma unroll
-        for (int j = 0; j < NJ; ++j) { S[j].s0 = acc[3 * j]; S[j].s1 = acc[3 * j + 1]; S[j].s2 = acc[3 * j + 2]; }
-    }
-    __syncthreads();
-}
 
-template <bool U8, int R, int U>
-DEV void rows_dot(const void *const (&rows)[R], const h16 *const (&xs)[R], int N, float (&acc)[R]) {
-    if constexpr (U8) {
-        const uint8_t *rr[R];
+    // red: 2 * DWAVES + 3 * NJ * DWAVES floats
+    DEV void compute(int C, bool has_sx, const rwkv_half *const (&mixp)[NJ], h16 *const (&xs)[NJ], VecSums (&S)[NJ],
+                     rwkv_half *xx_out, float *red) {
+        float m[2] = {0.f, 0.f};
+        if (own)
 #pragma unroll
-        for (int r = 0; r < R; ++r) rr[r] = (const uint8_t *)rows[r];
-        wave_rows_dot_u8<R, U>(rr, xs, N >> 4, acc);
-    } else {
-        const h16 *rr[R];
+            for (int e = 0; e < 8; ++e) {
+                const float f = (float)x[e];
+                m[0] += f;
+                m[1] += f * f;
+            }
+        block_sum_1b<2>(m, red);
+        const float mean = m[0] / C;
+        const float rstd = rsqrtf(fmaxf(m[1] / C - mean * mean, 0.f) + LN_EPS);
+        const int nseg = C >> 4, j8 = threadIdx.x;
+        float acc[3 * NJ];
 #pragma unroll
-        for (int r = 0; r < R; ++r) rr[r] = (const h16 *)rows[r];
-        wave_rows_dot_f16<R, U>(rr, xs, N >> 3, acc);
+        for (int i = 0; i < 3 * NJ; ++i) acc[i] = 0.f;
+        if (own) {
+            h16x8 xx;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) xx[e] = (h16)(((float)x[e] - mean) * rstd * (float)lw[e] + (float)lb[e]);
+            if (xx_out && blockIdx.x == 0) *(h16x8 *)(xx_out + 8 * j8) = xx;
+            const h16x8 pv = has_sx ? sx : xx;
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) {
+                h16x8 kx = xx;
+                if (mixp[j]) {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        const float mm = (float)mix[j][e];
+                        kx[e] = (h16)((float)xx[e] * mm + (float)pv[e] * (1.f - mm));
+                    }
+                }
+                h16x8 o = kx;
+                if (U8) {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        const float k = (float)kx[e];
+                        o[e] = (h16)(k * (float)ry[j][e]);
+                        acc[3 * j] += k;
+                        acc[3 * j + 1] += (float)o[e];
+                        acc[3 * j + 2] += k * (float)my[j][e];
+                    }
+                }
+                ((h16x8 *)xs[j])[xs_item<U8>(j8, nseg)] = o;
+            }
+        }
+        // one barrier publishes both the LDS activation vectors and the partial sums
+        block_sum_1b<3 * NJ>(acc, red + 2 * DWAVES);
+        if (U8)
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) { S[j].s0 = acc[3 * j]; S[j].s1 = acc[3 * j + 1]; S[j].s2 = acc[3 * j + 2]; }
     }
+};
+
+template <bool U8>
+DEV const uint8_t *row_ptr(const MatDev &m, int64_t row) {
+    return (const uint8_t *)m.w + row * m.ld * (U8 ? 1 : 2);
 }
 
 template <bool U8>
-DEV const void *row_ptr(const MatDev &m, int64_t row) {
-    return U8 ? (const void *)((const uint8_t *)m.w + row * m.ld) : (const void *)((const h16 *)m.w + row * m.ld);
+DEV float finish(float dot, const VecSums &S, float rx, float mx) {
+    return U8 ? mm8_finish(dot, S, rx, mx) : dot;
 }
 
-template <bool U8>
-DEV float finish(float dot, const VecSums &S, const MatDev &m, int row) {
-    return U8 ? mm8_finish(dot, S, h2f(m.rx[row]), h2f(m.mx[row])) : dot;
+// Streaming body shared by the three kernels.  The row space is `ngroups` groups of K rows
+// (K = 3 for the time-mix kernel: the key, value and receptance row of one channel; K = 1
+// otherwise).  Every wave owns a contiguous range of groups and walks it as a flat sequence of
+// batches (G groups x U segments per lane), ping-ponging between two register tiles: the loads
+// of batch q+1 are in flight while batch q is multiplied.
+//   pro_load():           issue the loads of the prologue operands (called first)
+//   pro_compute():        build the LDS activation vectors (contains the workgroup barriers)
+//   rowf(g, k, row, xs):  weight row pointer and LDS activation vector of row k of group g
+//   epi_load(g) -> E:     loads of the operands the epilogue of group g needs (no dependence on
+//                         the dot products: issued together with the group's first weight tile)
+//   epi(g, dots, E):      called by one lane per group with the K reduced dot products
+template <bool U8, int G, int K, int U, class E, class ProLoad, class ProCompute, class RowFn, class EpiLoad, class EpiFn>
+DEV void stream_rows(int ngroups, int nseg, ProLoad pro_load, ProCompute pro_compute, RowFn rowf, EpiLoad epi_load,
+                     EpiFn epi) {
+    constexpr int R = G * K;
+    const int lane = threadIdx.x & 63;
+    const int wave = blockIdx.x * DWAVES + (threadIdx.x >> 6), nwaves = gridDim.x * DWAVES;
+    const int per = (ngroups + nwaves - 1) / nwaves;
+    const int g0 = min(wave * per, ngroups), g1 = min(g0 + per, ngroups);
+    const int nsb = (nseg + 64 * U - 1) / (64 * U);             // segment batches per group batch
+    const int nb = ((g1 - g0 + G - 1) / G) * nsb;               // batches of this wave
+    RowTile<U8, R, U> t0, t1;
+    E e0{}, e1{};
+    // epilogue operands live in slot (group batch index & 1): they are loaded with the first
+    // tile of a group batch and used after its last one, by when at most the next group batch
+    // has started loading
+    auto load = [&](RowTile<U8, R, U> &t, int q) {
+        const int gbi = q / nsb, gb = g0 + gbi * G, sb = q % nsb;
+        const uint8_t *rows[R];
+        const h16 *xs_unused;
+#pragma unroll
+        for (int i = 0; i < G; ++i)
+#pragma unroll
+            for (int k = 0; k < K; ++k) rowf(min(gb + i, g1 - 1), k, rows[i * K + k], xs_unused);
+        if (sb == 0 && lane < G && gb + lane < g1) {
+            const E e = epi_load(gb + lane);
+            if (gbi & 1) e1 = e; else e0 = e;
+        }
+        t.load(rows, sb * 64 * U, nseg);
+    };
+    float acc[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) acc[r] = 0.f;
+    auto process = [&](const RowTile<U8, R, U> &t, int q) {
+        const int gbi = q / nsb, sb = q % nsb, gb = g0 + gbi * G;
+        const uint8_t *row_unused;
+        const h16 *xs[R];
+#pragma unroll
+        for (int i = 0; i < G; ++i)
+#pragma unroll
+            for (int k = 0; k < K; ++k) rowf(min(gb + i, g1 - 1), k, row_unused, xs[i * K + k]);
+        t.consume(xs, sb * 64 * U, nseg, acc);
+        if (sb == nsb - 1) {
+#pragma unroll
+            for (int r = 0; r < R; ++r) acc[r] = wave_sum(acc[r]);
+            if (lane < G && gb + lane < g1) {
+                float d[K];
+#pragma unroll
+                for (int k = 0; k < K; ++k) {
+                    d[k] = acc[k];
+#pragma unroll
+                    for (int i = 1; i < G; ++i) d[k] = (lane == i) ? acc[i * K + k] : d[k];
+                }
+                epi(gb + lane, d, (gbi & 1) ? e1 : e0);
+            }
+#pragma unroll
+            for (int r = 0; r < R; ++r) acc[r] = 0.f;
+        }
+    };
+    pro_load();
+    if (nb > 0) load(t0, 0);
+    pro_compute();
+    for (int q = 0; q < nb; q += 2) {
+        if (q + 1 < nb) load(t1, q + 1);
+        process(t0, q);
+        if (q + 1 < nb) {
+            if (q + 2 < nb) load(t0, q + 2);
+            process(t1, q + 1);
+        }
+    }
 }
 
 // ------------------------------------------------------------------------------------------
@@ -155,45 +248,57 @@ struct AttArgs {
     rwkv_half *rwkv;          // out: r * wkv, fp16 [C]
 };
 
-template <bool U8>
+struct AttEpi {
+    float rx[3], mx[3], u, w, aa, bb, pp;
+};
+
+template <bool U8, int G>
 __global__ __launch_bounds__(DTHREADS) void att_kernel(AttArgs a) {
     extern __shared__ __align__(16) unsigned char smem[];
-    __shared__ float red[9 * DWAVES];
+    __shared__ float red[(2 + 9) * DWAVES];
     const int C = a.C;
     h16 *xs[3] = {(h16 *)smem, (h16 *)smem + C, (h16 *)smem + 2 * C};
     VecSums S[3];
-    const rwkv_half *x = resolve_x(a.x, a.emb, a.token, C);
-    ln_mix_prologue<U8, 3>(x, C, a.ln_w, a.ln_b, a.sx, a.mix, a.mat, xs, S, a.xx_tmp, red);
-
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const int nwaves = gridDim.x * DWAVES;
-    for (int c = blockIdx.x * DWAVES + wave; c < C; c += nwaves) {
-        const void *rows[3] = {row_ptr<U8>(a.mat[0], c), row_ptr<U8>(a.mat[1], c), row_ptr<U8>(a.mat[2], c)};
-        const h16 *xv[3] = {xs[0], xs[1], xs[2]};
-        float acc[3] = {0.f, 0.f, 0.f};
-        rows_dot<U8, 3, 4>(rows, xv, C, acc);
-        if (lane == 0) {
-            float k = finish<U8>(acc[0], S[0], a.mat[0], c);
-            float v = finish<U8>(acc[1], S[1], a.mat[1], c);
-            float r = finish<U8>(acc[2], S[2], a.mat[2], c);
-            if (U8) { k = round_h(k); v = round_h(v); }  // uint8 path returns fp16, widened again
-            r = round_h(sigmoidf_(round_h(r)));
-            const float u = a.first[c], w = a.decay[c];
-            float aa = a.aa[c], bb = a.bb[c], pp = a.pp[c];
-            float ww = u + k;
-            float p = fmaxf(pp, ww);
-            float e1 = __expf(pp - p), e2 = __expf(ww - p);
-            const float wkv = (e1 * aa + e2 * v) / (e1 * bb + e2);
-            ww = w + pp;
-            p = fmaxf(ww, k);
-            e1 = __expf(ww - p);
-            e2 = __expf(k - p);
-            a.aa[c] = e1 * aa + e2 * v;
-            a.bb[c] = e1 * bb + e2;
-            a.pp[c] = p;
-            a.rwkv[c] = f2h(r * round_h(wkv));
+    LnMixPro<U8, 3> pro;
+    auto pro_load = [&]() {
+        pro.load(resolve_x(a.x, a.emb, a.token, C), C, a.ln_w, a.ln_b, a.sx, a.mix, a.mat);
+    };
+    auto pro_compute = [&]() { pro.compute(C, a.sx != nullptr, a.mix, xs, S, a.xx_tmp, red); };
+    auto rowf = [&](int c, int k, const uint8_t *&row, const h16 *&xv) {
+        row = row_ptr<U8>(a.mat[k], c);
+        xv = xs[k];
+    };
+    auto epi_load = [&](int c) {
+        AttEpi e;
+#pragma unroll
+        for (int k = 0; k < 3; ++k) {
+            e.rx[k] = U8 ? h2f(a.mat[k].rx[c]) : 1.f;
+            e.mx[k] = U8 ? h2f(a.mat[k].mx[c]) : 0.f;
         }
-    }
+        e.u = a.first[c]; e.w = a.decay[c];
+        e.aa = a.aa[c]; e.bb = a.bb[c]; e.pp = a.pp[c];
+        return e;
+    };
+    auto epi = [&](int c, const float (&d)[3], const AttEpi &e) {
+        float k = finish<U8>(d[0], S[0], e.rx[0], e.mx[0]);
+        float v = finish<U8>(d[1], S[1], e.rx[1], e.mx[1]);
+        float r = finish<U8>(d[2], S[2], e.rx[2], e.mx[2]);
+        if (U8) { k = round_h(k); v = round_h(v); }  // uint8 path returns fp16, widened again
+        r = round_h(sigmoidf_(round_h(r)));
+        float ww = e.u + k;
+        float p = fmaxf(e.pp, ww);
+        float e1 = __expf(e.pp - p), e2 = __expf(ww - p);
+        const float wkv = (e1 * e.aa + e2 * v) / (e1 * e.bb + e2);
+        ww = e.w + e.pp;
+        p = fmaxf(ww, k);
+        e1 = __expf(ww - p);
+        e2 = __expf(k - p);
+        a.aa[c] = e1 * e.aa + e2 * v;
+        a.bb[c] = e1 * e.bb + e2;
+        a.pp[c] = p;
+        a.rwkv[c] = f2h(r * round_h(wkv));
+    };
+    stream_rows<U8, G, 3, 2, AttEpi>(C, (C * (U8 ? 1 : 2)) >> 4, pro_load, pro_compute, rowf, epi_load, epi);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -211,10 +316,14 @@ struct LnMixArgs {
     void *out[2];
 };
 
-template <bool U8, int NJ, int R>
+struct ScaleEpi {
+    float rx, mx;
+};
+
+template <bool U8, int NJ, int G>
 __global__ __launch_bounds__(DTHREADS) void lnmix_kernel(LnMixArgs a) {
     extern __shared__ __align__(16) unsigned char smem[];
-    __shared__ float red[3 * NJ * DWAVES];
+    __shared__ float red[(2 + 3 * NJ) * DWAVES];
     const int C = a.C;
     h16 *xs[NJ];
     const rwkv_half *mix[NJ];
@@ -222,45 +331,39 @@ __global__ __launch_bounds__(DTHREADS) void lnmix_kernel(LnMixArgs a) {
 #pragma unroll
     for (int j = 0; j < NJ; ++j) { xs[j] = (h16 *)smem + j * C; mix[j] = a.mix[j]; mat[j] = a.mat[j]; }
     VecSums S[NJ];
-    ln_mix_prologue<U8, NJ>(a.x, C, a.ln_w, a.ln_b, a.sx, mix, mat, xs, S, a.xx_tmp, red);
-
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const int nwaves = gridDim.x * DWAVES;
-    const int g0 = (a.M[0] + R - 1) / R;
-    const int gtot = g0 + (NJ > 1 ? (a.M[1] + R - 1) / R : 0);
-    for (int g = blockIdx.x * DWAVES + wave; g < gtot; g += nwaves) {
-        const int j = (NJ > 1 && g >= g0) ? 1 : 0;
-        const int row0 = (j ? g - g0 : g) * R;
-        const int M = a.M[j];
-        const void *rows[R];
-        const h16 *xv[R];
-        float acc[R];
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-            rows[r] = row_ptr<U8>(mat[j], min(row0 + r, M - 1));
-            xv[r] = xs[j];
-            acc[r] = 0.f;
+    const int M0 = a.M[0];
+    LnMixPro<U8, NJ> pro;
+    auto pro_load = [&]() { pro.load(a.x, C, a.ln_w, a.ln_b, a.sx, mix, mat); };
+    auto pro_compute = [&]() { pro.compute(C, a.sx != nullptr, mix, xs, S, a.xx_tmp, red); };
+    auto rowf = [&](int g, int, const uint8_t *&row, const h16 *&xv) {
+        const int j = (NJ > 1 && g >= M0) ? 1 : 0;
+        row = row_ptr<U8>(mat[j], j ? g - M0 : g);
+        xv = xs[j];
+    };
+    auto epi_load = [&](int g) {
+        const int j = (NJ > 1 && g >= M0) ? 1 : 0;
+        const int m = j ? g - M0 : g;
+        ScaleEpi e;
+        e.rx = U8 ? h2f(mat[j].rx[m]) : 1.f;
+        e.mx = U8 ? h2f(mat[j].mx[m]) : 0.f;
+        return e;
+    };
+    auto epi = [&](int g, const float (&d)[1], const ScaleEpi &e) {
+        const int j = (NJ > 1 && g >= M0) ? 1 : 0;
+        const int m = j ? g - M0 : g;
+        const float v = round_h(finish<U8>(d[0], S[j], e.rx, e.mx));
+        const int kind = a.epi[j];
+        if (kind == EPI_LOGITS) {
+            ((float *)a.out[j])[m] = v;
+        } else if (kind == EPI_SIGMOID) {
+            ((rwkv_half *)a.out[j])[m] = f2h(sigmoidf_(v));
+        } else {
+            const float t = fmaxf(v, 0.f);
+            ((rwkv_half *)a.out[j])[m] = f2h(t * t);
         }
-        rows_dot<U8, R, (R >= 4 ? 2 : 4)>(rows, xv, C, acc);
-        if (lane < R) {
-            float d = acc[0];
-#pragma unroll
-            for (int r = 1; r < R; ++r) d = (lane == r) ? acc[r] : d;
-            const int m = row0 + lane;
-            if (m < M) {
-                const float v = round_h(finish<U8>(d, S[j], mat[j], m));
-                const int epi = a.epi[j];
-                if (epi == EPI_LOGITS) {
-                    ((float *)a.out[j])[m] = v;
-                } else if (epi == EPI_SIGMOID) {
-                    ((rwkv_half *)a.out[j])[m] = f2h(sigmoidf_(v));
-                } else {
-                    const float t = fmaxf(v, 0.f);
-                    ((rwkv_half *)a.out[j])[m] = f2h(t * t);
-                }
-            }
-        }
-    }
+    };
+    stream_rows<U8, G, 1, (G >= 4 ? 1 : 2), ScaleEpi>(M0 + (NJ > 1 ? a.M[1] : 0), (C * (U8 ? 1 : 2)) >> 4, pro_load,
+                                                      pro_compute, rowf, epi_load, epi);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -278,57 +381,77 @@ struct VecArgs {
     rwkv_half *commit_dst;
 };
 
+struct VecEpi {
+    float rx, mx, xin, gate;
+};
+
 template <bool U8, int U>
 __global__ __launch_bounds__(DTHREADS) void vec_kernel(VecArgs a) {
     extern __shared__ __align__(16) unsigned char smem[];
     __shared__ float red[3 * DWAVES];
     const int N = a.N;
     h16 *xs = (h16 *)smem;
-    if (blockIdx.x == 0 && a.commit_dst)
-        for (int j8 = threadIdx.x; j8 < (a.C >> 3); j8 += blockDim.x)
-            *(u32x4 *)(a.commit_dst + 8 * j8) = *(const u32x4 *)(a.commit_src + 8 * j8);
     VecSums S;
-    {
-        const int nseg = N >> 4;
-        float acc[3] = {0.f, 0.f, 0.f};
-        for (int j8 = threadIdx.x; j8 < (N >> 3); j8 += blockDim.x) {
-            const h16x8 xv = *(const h16x8 *)(a.vin + 8 * j8);
-            h16x8 o = xv;
-            if (U8) {
-                const h16x8 rv = *(const h16x8 *)(a.mat.ry + 8 * j8);
-                const h16x8 yv = *(const h16x8 *)(a.mat.my + 8 * j8);
+    h16x8 pv[VP], pr[VP], pm[VP];
+    auto pro_load = [&]() {
 #pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    const float k = (float)xv[e];
-                    o[e] = (h16)(k * (float)rv[e]);
-                    acc[0] += k;
-                    acc[1] += (float)o[e];
-                    acc[2] += k * (float)yv[e];
+        for (int i = 0; i < VP; ++i) {
+            const int j8 = threadIdx.x + i * DTHREADS;
+            if (j8 < (N >> 3)) {
+                pv[i] = *(const h16x8 *)(a.vin + 8 * j8);
+                if (U8) {
+                    pr[i] = *(const h16x8 *)(a.mat.ry + 8 * j8);
+                    pm[i] = *(const h16x8 *)(a.mat.my + 8 * j8);
                 }
             }
-            ((h16x8 *)xs)[xs_item<U8>(j8, nseg)] = o;
         }
-        if (U8) {
-            block_sum_n<3>(acc, red);
-            S.s0 = acc[0]; S.s1 = acc[1]; S.s2 = acc[2];
+    };
+    auto pro_compute = [&]() {
+        if (blockIdx.x == 0 && a.commit_dst)
+            for (int j8 = threadIdx.x; j8 < (a.C >> 3); j8 += blockDim.x)
+                *(u32x4 *)(a.commit_dst + 8 * j8) = *(const u32x4 *)(a.commit_src + 8 * j8);
+        const int nseg = N >> 4;
+        float acc[3] = {0.f, 0.f, 0.f};
+#pragma unroll
+        for (int i = 0; i < VP; ++i) {
+            const int j8 = threadIdx.x + i * DTHREADS;
+            if (j8 < (N >> 3)) {
+                h16x8 o = pv[i];
+                if (U8) {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        const float k = (float)pv[i][e];
+                        o[e] = (h16)(k * (float)pr[i][e]);
+                        acc[0] += k;
+                        acc[1] += (float)o[e];
+                        acc[2] += k * (float)pm[i][e];
+                    }
+                }
+                ((h16x8 *)xs)[xs_item<U8>(j8, nseg)] = o;
+            }
         }
-        __syncthreads();
-    }
-    const rwkv_half *xin = resolve_x(a.x_in, a.emb, a.token, a.C);
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const int nwaves = gridDim.x * DWAVES;
-    for (int m = blockIdx.x * DWAVES + wave; m < a.M; m += nwaves) {
-        const void *rows[1] = {row_ptr<U8>(a.mat, m)};
-        const h16 *xv[1] = {xs};
-        float acc[1] = {0.f};
-        rows_dot<U8, 1, U>(rows, xv, N, acc);
-        if (lane == 0) {
-            float o = round_h(finish<U8>(acc[0], S, a.mat, m));
-            if (a.gate) o = round_h(h2f(a.gate[m]) * o);
-            o = round_h(h2f(xin[m]) + o);
-            a.x_out[m] = f2h(o * a.out_scale);
-        }
-    }
+        block_sum_1b<3>(acc, red);  // the barrier also publishes xs
+        if (U8) { S.s0 = acc[0]; S.s1 = acc[1]; S.s2 = acc[2]; }
+    };
+    auto rowf = [&](int m, int, const uint8_t *&row, const h16 *&xv) {
+        row = row_ptr<U8>(a.mat, m);
+        xv = xs;
+    };
+    auto epi_load = [&](int m) {
+        VecEpi e;
+        e.rx = U8 ? h2f(a.mat.rx[m]) : 1.f;
+        e.mx = U8 ? h2f(a.mat.mx[m]) : 0.f;
+        e.xin = h2f(resolve_x(a.x_in, a.emb, a.token, a.C)[m]);
+        e.gate = a.gate ? h2f(a.gate[m]) : 1.f;
+        return e;
+    };
+    auto epi = [&](int m, const float (&d)[1], const VecEpi &e) {
+        float o = round_h(finish<U8>(d[0], S, e.rx, e.mx));
+        if (a.gate) o = round_h(e.gate * o);
+        o = round_h(e.xin + o);
+        a.x_out[m] = f2h(o * a.out_scale);
+    };
+    stream_rows<U8, 1, 1, U, VecEpi>(a.M, (N * (U8 ? 1 : 2)) >> 4, pro_load, pro_compute, rowf, epi_load, epi);
 }
 
 int g_num_cu = 0;
@@ -372,7 +495,7 @@ size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 int v4_model_check(const rwkv_v4_model *m) {
     if (!m || !m->layers || !m->emb || !m->ln_out_w || !m->ln_out_b) return RWKV_E_NULL;
     const int64_t C = m->n_embd, F = m->n_ffn, V = m->vocab;
-    if (m->n_layer <= 0 || C <= 0 || F <= 0 || V <= 0 || (C & 63) || (F & 63) || C > 10240 || F > 32768)
+    if (m->n_layer <= 0 || C <= 0 || F <= 0 || V <= 0 || (C & 63) || (F & 63) || C > 8 * DTHREADS || F > 8 * VP * DTHREADS)
         return RWKV_E_SHAPE;
     const bool u8 = m->weights_u8 != 0;
     for (int i = 0; i < m->n_layer; ++i) {
@@ -454,8 +577,8 @@ static int v4_one_impl(const rwkv_v4_model *m, const rwkv_v4_layer_state *states
             a.decay = l.time_decay; a.first = l.time_first; a.aa = s.aa; a.bb = s.bb; a.pp = s.pp;
             a.rwkv = ws.rwkv;
             const size_t lds = 3 * (size_t)C * 2;
-            if (u8) hipLaunchKernelGGL(att_kernel<true>, dim3(grid), dim3(DTHREADS), lds, st, a);
-            else hipLaunchKernelGGL(att_kernel<false>, dim3(grid), dim3(DTHREADS), lds, st, a);
+            if (u8) hipLaunchKernelGGL((att_kernel<true, 1>), dim3(grid), dim3(DTHREADS), lds, st, a);
+            else hipLaunchKernelGGL((att_kernel<false, 1>), dim3(grid), dim3(DTHREADS), lds, st, a);
             mark();
         }
         {
@@ -476,8 +599,17 @@ static int v4_one_impl(const rwkv_v4_model *m, const rwkv_v4_layer_state *states
             a.mix[1] = l.ffn_mix_k; a.mat[1] = to_dev(l.ffn_key); a.M[1] = F; a.epi[1] = EPI_RELU_SQ;
             a.out[1] = ws.vx;
             const size_t lds = 2 * (size_t)C * 2;
-            if (u8) hipLaunchKernelGGL((lnmix_kernel<true, 2, 2>), dim3(grid), dim3(DTHREADS), lds, st, a);
-            else hipLaunchKernelGGL((lnmix_kernel<false, 2, 2>), dim3(grid), dim3(DTHREADS), lds, st, a);
+            const int per = (C + F + grid * DWAVES - 1) / (grid * DWAVES);
+            if (per % 5 == 0) {
+                if (u8) hipLaunchKernelGGL((lnmix_kernel<true, 2, 5>), dim3(grid), dim3(DTHREADS), lds, st, a);
+                else hipLaunchKernelGGL((lnmix_kernel<false, 2, 5>), dim3(grid), dim3(DTHREADS), lds, st, a);
+            } else if (per >= 4) {
+                if (u8) hipLaunchKernelGGL((lnmix_kernel<true, 2, 4>), dim3(grid), dim3(DTHREADS), lds, st, a);
+                else hipLaunchKernelGGL((lnmix_kernel<false, 2, 4>), dim3(grid), dim3(DTHREADS), lds, st, a);
+            } else {
+                if (u8) hipLaunchKernelGGL((lnmix_kernel<true, 2, 2>), dim3(grid), dim3(DTHREADS), lds, st, a);
+                else hipLaunchKernelGGL((lnmix_kernel<false, 2, 2>), dim3(grid), dim3(DTHREADS), lds, st, a);
+            }
             mark();
         }
         {
@@ -487,8 +619,8 @@ static int v4_one_impl(const rwkv_v4_model *m, const rwkv_v4_layer_state *states
             a.out_scale = (m->rescale_layer > 0 && (i + 1) % m->rescale_layer == 0) ? 0.5f : 1.f;
             a.commit_src = ws.xx_ffn; a.commit_dst = s.ffn_xx;
             const size_t lds = (size_t)F * 2;
-            if (u8) hipLaunchKernelGGL((vec_kernel<true, 4>), dim3(grid), dim3(DTHREADS), lds, st, a);
-            else hipLaunchKernelGGL((vec_kernel<false, 4>), dim3(grid), dim3(DTHREADS), lds, st, a);
+            if (u8) hipLaunchKernelGGL((vec_kernel<true, 8>), dim3(grid), dim3(DTHREADS), lds, st, a);
+            else hipLaunchKernelGGL((vec_kernel<false, 8>), dim3(grid), dim3(DTHREADS), lds, st, a);
             mark();
         }
         RWKV_LAUNCH_CHECK();

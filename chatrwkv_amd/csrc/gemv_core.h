@@ -141,6 +141,49 @@ DEV void block_sum_n(float (&v)[K], float *red) {
     }
 }
 
+// A register tile of weights: U 16-byte segments of R rows per lane.  Loading and consuming are
+// separate steps so that a kernel can put the loads of its first tile in flight *before* it
+// builds the activation vector (weights do not depend on activations).  A segment is 16 bytes
+// of a row for both weight types (16 uint8 or 8 fp16 values); nseg = row bytes / 16.
+template <bool U8, int R, int U>
+struct RowTile {
+    u32x4 w[U][R];
+
+    DEV void load(const uint8_t *const (&rows)[R], int seg0, int nseg) {
+        const int lane = threadIdx.x & 63;
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int s = seg0 + lane + 64 * u;
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                u32x4 v = {0u, 0u, 0u, 0u};
+                if (s < nseg) v = __builtin_nontemporal_load((const u32x4 *)(rows[r] + 16 * (size_t)s));
+                w[u][r] = v;
+            }
+        }
+    }
+
+    // acc[r] += <row r segments [seg0, seg0 + 64 U), xs[r]>; xs in the layout of the weight type
+    // (uint8: split lo/hi items, fp16: linear).
+    DEV void consume(const h16 *const (&xs)[R], int seg0, int nseg, float (&acc)[R]) const {
+        const int lane = threadIdx.x & 63;
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int s = seg0 + lane + 64 * u;
+            if (s < nseg) {
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+                    const h16x8 *xv = (const h16x8 *)xs[r];
+                    if (U8)
+                        acc[r] = dot16_u8(w[u][r], xv[s], xv[nseg + s], acc[r]);
+                    else
+                        acc[r] = dot8_f16(w[u][r], xv[s], acc[r]);
+                }
+            }
+        }
+    }
+};
+
 // Final value of a uint8 row from its raw dot product.
 DEV float mm8_finish(float dot, const VecSums &S, float rx, float mx) {
     return rx * (dot - 1023.5f * S.s1) + mx * S.s0 + S.s2;
