@@ -8,23 +8,35 @@
 // rank-1 corrections enter in the epilogue:
 //     y[t, m] = rx[m] * acc[t, m] + mx[m] * S0[t] + S2[t],   S0 = sum_j x[t, j],  S2 = sum_j x[t, j] my[j].
 //
-// Tiling: BT x BM outputs per workgroup of 256 threads (2 x 2 waves), K step 64, LDS double
-// buffered; both LDS tiles are [row][64 halves] with the eight 16-byte chunks of a row XOR-
-// swizzled by (row & 7) so that the ds_read_b128 of 32 consecutive rows spreads over all banks.
+// Tiling: BT x BM outputs per workgroup of 256 threads (WT x WM waves, each owning a
+// (BT/WT) x (BM/WM) block built from 32x32 MFMA tiles), K step 64, LDS double buffered; both LDS
+// tiles are [row][64 halves] with the eight 16-byte chunks of a row XOR-swizzled by (row & 7) so
+// that the ds_read_b128 of 32 consecutive rows spreads over all banks.  A wave block of
+// 128 x 128 needs 8 fragment reads per 16 MFMAs, which keeps the LDS pipe at half its peak; the
+// 64 x 64 block of the small-tile variant needs 4 reads per 4 MFMAs and is LDS-bound, so it is
+// only used when a larger tile would leave most CUs idle.
+// Workgroup ids are remapped so that the workgroups which share a weight tile (same m0,
+// different t0) run on the same XCD and the tile is fetched into that XCD's L2 once.
 #include "kernels.h"
+#include <cstdlib>
 
 namespace {
 
 constexpr int BK = 64;  // halves per LDS row
 
-DEV int swz(int row, int chunk) { return row * BK + ((chunk ^ (row & 7)) << 3); }
+// LDS address (in halves) of 16-byte chunk `chunk` (0..7) of tile row `row`.  Rows are 128 bytes.
+// The chunk index is XORed with a per-row key chosen so that a ds_read_b128 / ds_write_b128 is
+// conflict free both if the LDS serves 8 lanes x 16 B per cycle from 32 banks (8 consecutive
+// rows must hit 8 different chunk slots) and if it serves 16 lanes from 64 banks (the 8 even and
+// the 8 odd rows of 16 consecutive rows must each hit 8 different slots).
+DEV int swz(int row, int chunk) { return row * BK + ((chunk ^ ((row & 7) ^ ((row >> 3) & 1))) << 3); }
 
-template <bool W_U8, int BT, int BM>
+template <bool W_U8, int BT, int BM, int WT, int WM, int PF>
 __global__ __launch_bounds__(256) void gemm_kernel(int T, int N, int M, const h16 *__restrict__ A, int64_t lda,
                                                    const void *__restrict__ Wv, int64_t ldw, void *__restrict__ Y,
                                                    int64_t ldy, GemmEpi ep) {
-    static_assert(BT % 64 == 0 && BM % 64 == 0, "tile");
-    constexpr int MI = BT / 64, NI = BM / 64;  // 32x32 blocks per wave in each direction (2x2 waves)
+    static_assert(WT * WM == 4 && BT % (32 * WT) == 0 && BM % (32 * WM) == 0 && BM % 64 == 0, "tile");
+    constexpr int MI = BT / (32 * WT), NI = BM / (32 * WM);  // 32x32 blocks per wave in each direction
     extern __shared__ __align__(16) unsigned char smem[];
     h16 *lA[2], *lB[2];
     lA[0] = (h16 *)smem;
@@ -33,46 +45,49 @@ __global__ __launch_bounds__(256) void gemm_kernel(int T, int N, int M, const h1
     lB[1] = lA[1] + BT * BK;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wr = wave >> 1, wc = wave & 1;
-    // workgroup -> tile: consecutive workgroups walk the T direction first so that the
-    // workgroups sharing a weight tile run at the same time (the weight tile is then served
-    // from L2 for all but the first).
+    const int wr = wave / WM, wc = wave % WM;
+    // workgroup -> tile: hardware deals consecutive workgroup ids round-robin to the 8 XCDs;
+    // undo that so each XCD gets a contiguous range of tiles, which walk the T direction first.
     const int tiles_t = (T + BT - 1) / BT;
-    const int t0 = (blockIdx.x % tiles_t) * BT, m0 = (blockIdx.x / tiles_t) * BM;
+    int bid = blockIdx.x;
+    if ((gridDim.x & 7) == 0) bid = (bid & 7) * (gridDim.x >> 3) + (bid >> 3);
+    const int t0 = (bid % tiles_t) * BT, m0 = (bid / tiles_t) * BM;
 
     constexpr int A_LD = BT / 32;                    // 16-byte loads per thread for the A tile
     constexpr int B_LD = W_U8 ? BM / 64 : BM / 32;   // 16-byte loads per thread for the W tile
-    u32x4 ra[A_LD], rb[B_LD];
+    // PF k-tiles are in flight in registers (global latency under load is several k-tile times);
+    // the LDS holds the tile being multiplied and the next one.
+    u32x4 ra[PF][A_LD], rb[PF][B_LD];
 
-    auto load_tiles = [&](int kt) {
+    auto load_tiles = [&](u32x4 (&qa)[A_LD], u32x4 (&qb)[B_LD], int kt) {
         const int k0 = kt * BK;
 #pragma unroll
         for (int i = 0; i < A_LD; ++i) {
             const int row = (tid >> 3) + 32 * i, ch = tid & 7;
             const int t = min(t0 + row, T - 1);
-            ra[i] = *(const u32x4 *)(A + (size_t)t * lda + k0 + ch * 8);
+            qa[i] = *(const u32x4 *)(A + (size_t)t * lda + k0 + ch * 8);
         }
         if (W_U8) {
 #pragma unroll
             for (int i = 0; i < B_LD; ++i) {
                 const int row = (tid >> 2) + 64 * i, ch = tid & 3;
                 const int m = min(m0 + row, M - 1);
-                rb[i] = __builtin_nontemporal_load((const u32x4 *)((const uint8_t *)Wv + (size_t)m * ldw + k0 + ch * 16));
+                qb[i] = __builtin_nontemporal_load((const u32x4 *)((const uint8_t *)Wv + (size_t)m * ldw + k0 + ch * 16));
             }
         } else {
 #pragma unroll
             for (int i = 0; i < B_LD; ++i) {
                 const int row = (tid >> 3) + 32 * i, ch = tid & 7;
                 const int m = min(m0 + row, M - 1);
-                rb[i] = *(const u32x4 *)((const h16 *)Wv + (size_t)m * ldw + k0 + ch * 8);
+                qb[i] = *(const u32x4 *)((const h16 *)Wv + (size_t)m * ldw + k0 + ch * 8);
             }
         }
     };
-    auto store_tiles = [&](int buf) {
+    auto store_tiles = [&](const u32x4 (&qa)[A_LD], const u32x4 (&qb)[B_LD], int buf) {
 #pragma unroll
         for (int i = 0; i < A_LD; ++i) {
             const int row = (tid >> 3) + 32 * i, ch = tid & 7;
-            *(u32x4 *)(lA[buf] + swz(row, ch)) = ra[i];
+            *(u32x4 *)(lA[buf] + swz(row, ch)) = qa[i];
         }
         if (W_U8) {
             const h16x2 off = {(h16)1023.5f, (h16)1023.5f};
@@ -80,7 +95,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(int T, int N, int M, const h1
             for (int i = 0; i < B_LD; ++i) {
                 const int row = (tid >> 2) + 64 * i, ch = tid & 3;
                 u32x4 lo, hi;
-                const uint32_t d[4] = {rb[i].x, rb[i].y, rb[i].z, rb[i].w};
+                const uint32_t d[4] = {qb[i].x, qb[i].y, qb[i].z, qb[i].w};
                 uint32_t o[8];
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
@@ -89,14 +104,17 @@ __global__ __launch_bounds__(256) void gemm_kernel(int T, int N, int M, const h1
                 }
                 lo.x = o[0]; lo.y = o[1]; lo.z = o[2]; lo.w = o[3];
                 hi.x = o[4]; hi.y = o[5]; hi.z = o[6]; hi.w = o[7];
-                *(u32x4 *)(lB[buf] + swz(row, 2 * ch)) = lo;
-                *(u32x4 *)(lB[buf] + swz(row, 2 * ch + 1)) = hi;
+                // rows r and r+2 share the XOR key's low bit: alternate which half goes first so the
+                // 16 lanes of one write touch 16 different slots
+                const int odd = (row >> 1) & 1;
+                *(u32x4 *)(lB[buf] + swz(row, 2 * ch + odd)) = odd ? hi : lo;
+                *(u32x4 *)(lB[buf] + swz(row, 2 * ch + 1 - odd)) = odd ? lo : hi;
             }
         } else {
 #pragma unroll
             for (int i = 0; i < B_LD; ++i) {
                 const int row = (tid >> 3) + 32 * i, ch = tid & 7;
-                *(u32x4 *)(lB[buf] + swz(row, ch)) = rb[i];
+                *(u32x4 *)(lB[buf] + swz(row, ch)) = qb[i];
             }
         }
     };
@@ -110,24 +128,19 @@ __global__ __launch_bounds__(256) void gemm_kernel(int T, int N, int M, const h1
             for (int e = 0; e < 16; ++e) acc[a][b][e] = 0.f;
 
     const int nk = N / BK;
-    load_tiles(0);
-    store_tiles(0);
-    __syncthreads();
-    for (int kt = 0; kt < nk; ++kt) {
-        const int buf = kt & 1;
-        if (kt + 1 < nk) load_tiles(kt + 1);
+    auto compute = [&](int buf) {
 #pragma unroll
         for (int ks = 0; ks < BK / 16; ++ks) {
             h16x8 fa[MI], fb[NI];
             const int ch = 2 * ks + (lane >> 5);
 #pragma unroll
             for (int a = 0; a < MI; ++a) {
-                const int row = wr * (BT / 2) + a * 32 + (lane & 31);
+                const int row = wr * (BT / WT) + a * 32 + (lane & 31);
                 fa[a] = *(const h16x8 *)(lA[buf] + swz(row, ch));
             }
 #pragma unroll
             for (int b = 0; b < NI; ++b) {
-                const int row = wc * (BM / 2) + b * 32 + (lane & 31);
+                const int row = wc * (BM / WM) + b * 32 + (lane & 31);
                 fb[b] = *(const h16x8 *)(lB[buf] + swz(row, ch));
             }
 #pragma unroll
@@ -136,14 +149,31 @@ __global__ __launch_bounds__(256) void gemm_kernel(int T, int N, int M, const h1
                 for (int b = 0; b < NI; ++b)
                     acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[a], fb[b], acc[a][b], 0, 0, 0);
         }
-        if (kt + 1 < nk) store_tiles(buf ^ 1);
-        __syncthreads();
+    };
+    // tile kt lives in register slot kt % PF from PF iterations before it is multiplied until it
+    // is written to LDS buffer kt & 1 at the end of iteration kt - 1
+#pragma unroll
+    for (int p = 0; p < PF; ++p)
+        if (p < nk) load_tiles(ra[p], rb[p], p);
+    store_tiles(ra[0], rb[0], 0);
+    __syncthreads();
+    for (int kt0 = 0; kt0 < nk; kt0 += PF) {
+#pragma unroll
+        for (int p = 0; p < PF; ++p) {
+            const int kt = kt0 + p;
+            if (kt < nk) {
+                if (kt + PF < nk) load_tiles(ra[p], rb[p], kt + PF);  // slot freed when tile kt went to LDS
+                compute(kt & 1);
+                if (kt + 1 < nk) store_tiles(ra[(p + 1) % PF], rb[(p + 1) % PF], (kt + 1) & 1);
+                __syncthreads();
+            }
+        }
     }
 
     // epilogue: lane holds column m = .. + (lane & 31) and rows 8*(e/4) + 4*(lane>>5) + e%4
 #pragma unroll
     for (int b = 0; b < NI; ++b) {
-        const int m = m0 + wc * (BM / 2) + b * 32 + (lane & 31);
+        const int m = m0 + wc * (BM / WM) + b * 32 + (lane & 31);
         if (m >= M) continue;
         float rxm = 1.f, mxm = 0.f;
         if (ep.rx) { rxm = h2f(ep.rx[m]); mxm = h2f(ep.mx[m]); }
@@ -151,7 +181,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(int T, int N, int M, const h1
         for (int a = 0; a < MI; ++a) {
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
-                const int t = t0 + wr * (BT / 2) + a * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
+                const int t = t0 + wr * (BT / WT) + a * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
                 if (t >= T) continue;
                 float v = acc[a][b][e];
                 if (ep.rx) v = rxm * v + mxm * ep.s0[t] + ep.s2[t];
@@ -212,19 +242,56 @@ __global__ __launch_bounds__(256) void mm8_prepare_kernel(int T, int N, const rw
 
 }  // namespace
 
-int gemm_launch(bool w_u8, int64_t T, int64_t N, int64_t M, const rwkv_half *A, int64_t lda, const void *W,
-                int64_t ldw, void *Y, int64_t ldy, const GemmEpi &ep, hipStream_t st) {
-    constexpr int BT = 128, BM = 128;
-    const size_t lds = 2 * (size_t)(BT + BM) * BK * sizeof(h16);
+namespace {
+
+template <bool W_U8, int BT, int BM, int WT, int WM, int PF>
+int launch_cfg(int64_t T, int64_t N, int64_t M, const rwkv_half *A, int64_t lda, const void *W, int64_t ldw, void *Y,
+               int64_t ldy, const GemmEpi &ep, hipStream_t st) {
+    constexpr size_t lds = 2 * (size_t)(BT + BM) * BK * sizeof(h16);
+    static bool attr_done = false;
+    if (lds > 64 * 1024 && !attr_done) {
+        hipError_t e = hipFuncSetAttribute((const void *)gemm_kernel<W_U8, BT, BM, WT, WM, PF>,
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return (int)e;
+        attr_done = true;
+    }
     const int64_t tiles = ((T + BT - 1) / BT) * ((M + BM - 1) / BM);
-    if (w_u8)
-        hipLaunchKernelGGL((gemm_kernel<true, BT, BM>), dim3((unsigned)tiles), dim3(256), lds, st, (int)T, (int)N,
-                           (int)M, (const h16 *)A, lda, W, ldw, Y, ldy, ep);
-    else
-        hipLaunchKernelGGL((gemm_kernel<false, BT, BM>), dim3((unsigned)tiles), dim3(256), lds, st, (int)T, (int)N,
-                           (int)M, (const h16 *)A, lda, W, ldw, Y, ldy, ep);
+    hipLaunchKernelGGL((gemm_kernel<W_U8, BT, BM, WT, WM, PF>), dim3((unsigned)tiles), dim3(256), lds, st, (int)T, (int)N,
+                       (int)M, (const h16 *)A, lda, W, ldw, Y, ldy, ep);
     RWKV_LAUNCH_CHECK();
     return RWKV_OK;
+}
+
+template <bool W_U8>
+int launch_pick(int cfg, int64_t T, int64_t N, int64_t M, const rwkv_half *A, int64_t lda, const void *W, int64_t ldw,
+                void *Y, int64_t ldy, const GemmEpi &ep, hipStream_t st) {
+    switch (cfg) {
+        case 0: return launch_cfg<W_U8, 128, 128, 2, 2, 1>(T, N, M, A, lda, W, ldw, Y, ldy, ep, st);
+        case 1: return launch_cfg<W_U8, 128, 128, 2, 2, 2>(T, N, M, A, lda, W, ldw, Y, ldy, ep, st);
+        case 2: return launch_cfg<W_U8, 128, 128, 2, 2, 3>(T, N, M, A, lda, W, ldw, Y, ldy, ep, st);
+        case 3: return launch_cfg<W_U8, 128, 128, 2, 2, 4>(T, N, M, A, lda, W, ldw, Y, ldy, ep, st);
+        case 4: return launch_cfg<W_U8, 256, 128, 2, 2, 2>(T, N, M, A, lda, W, ldw, Y, ldy, ep, st);
+        case 5: return launch_cfg<W_U8, 128, 256, 2, 2, 2>(T, N, M, A, lda, W, ldw, Y, ldy, ep, st);
+        case 6: return launch_cfg<W_U8, 256, 256, 2, 2, 2>(T, N, M, A, lda, W, ldw, Y, ldy, ep, st);
+        default: return RWKV_E_DTYPE;
+    }
+}
+
+// Tile choice (RWKV_GEMM_CFG overrides it for tuning sweeps).
+int pick_cfg(int64_t T, int64_t M) {
+    const char *e = getenv("RWKV_GEMM_CFG");  // tuning override
+    if (e && *e) return atoi(e);
+    (void)T; (void)M;
+    return 3;  // 128 x 128 tile, 4 k-tiles of prefetch: the best of the sweep for every shape measured
+}
+
+}  // namespace
+
+int gemm_launch(bool w_u8, int64_t T, int64_t N, int64_t M, const rwkv_half *A, int64_t lda, const void *W,
+                int64_t ldw, void *Y, int64_t ldy, const GemmEpi &ep, hipStream_t st) {
+    const int cfg = pick_cfg(T, M);
+    return w_u8 ? launch_pick<true>(cfg, T, N, M, A, lda, W, ldw, Y, ldy, ep, st)
+                : launch_pick<false>(cfg, T, N, M, A, lda, W, ldw, Y, ldy, ep, st);
 }
 
 int mm8_prepare_launch(int64_t T, int64_t N, const rwkv_half *x, int64_t ldx, const rwkv_half *ry,
