@@ -1,0 +1,472 @@
+// Streaming one-token kernels shared by the RWKV-4 and RWKV-5/6 one-token paths:
+// the LayerNorm + token-shift + GEMV kernels and the vector GEMV kernel with its epilogues.
+//
+// A launch is short (3-15 us of streaming), so what matters is the chain of dependent memory
+// round trips, each ~2 us while HBM is saturated.  Every kernel therefore issues ALL its
+// independent loads in its first instructions -- the prologue operands (x, LayerNorm and mix
+// vectors, scales), the epilogue operands of its first rows (rx, mx, state) and the first tile
+// of weights -- and only then starts the reductions: one round trip instead of four.
+// Each workgroup redoes the O(C) prologue (a few thousand elements served from L2) against
+// hundreds of KiB of weights streamed from HBM.
+#pragma once
+#include "gemv_core.h"
+#include "kernels.h"
+
+namespace {
+
+constexpr int DTHREADS = 1024;
+constexpr int DWAVES = DTHREADS / 64;
+constexpr float LN_EPS = 1e-5f;
+constexpr int VP = 4;  // 8-element groups per thread the vector prologue keeps in registers (N <= 32768)
+
+// x for this step: the embedding row of the token (first layer) or the running activation.
+DEV const rwkv_half *resolve_x(const rwkv_half *x, const rwkv_half *emb, const int32_t *token, int C) {
+    return token ? emb + (size_t)(*token) * C : x;
+}
+
+// LDS item (16 bytes = 8 halves) index of the 8-element group j8 of an activation vector.
+template <bool U8>
+DEV int xs_item(int j8, int nseg) { return U8 ? ((j8 & 1) * nseg + (j8 >> 1)) : j8; }
+
+struct MatDev {
+    const void *w;
+    int64_t ld;
+    const rwkv_half *mx, *rx, *my, *ry;
+};
+
+// Workgroup sums of K values with ONE barrier: `red` (K * DWAVES floats) must not be in use by
+// an earlier reduction that other waves may still be reading (callers pass disjoint regions).
+// Stage 2 reads one wave's partial per lane (lane l takes wave l % 16: DWAVES == 16 == one DPP
+// row) and finishes with a 16-lane row sum.
+template <int K>
+DEV void block_sum_1b(float (&v)[K], float *red) {
+    static_assert(DWAVES == 16, "stage 2 assumes 16 waves");
+    const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
+#pragma unroll
+    for (int k = 0; k < K; ++k) v[k] = wave_sum(v[k]);
+    if (lane == 0)
+#pragma unroll
+        for (int k = 0; k < K; ++k) red[k * DWAVES + wid] = v[k];
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < K; ++k) v[k] = row16_sum(red[k * DWAVES + (lane & 15)]);
+}
+
+// LayerNorm + token-shift mixes for NJ consumers, operands staged in registers.
+// Requires C / 8 <= DTHREADS (C <= 8192): thread t owns elements [8t, 8t + 8).
+template <bool U8, int NJ>
+struct LnMixPro {
+    h16x8 x, lw, lb, sx, mix[NJ], ry[NJ], my[NJ];
+    bool own;
+
+    DEV void load(const rwkv_half *xp, int C, const rwkv_half *ln_w, const rwkv_half *ln_b, const rwkv_half *sxp,
+                  const rwkv_half *const (&mixp)[NJ], const MatDev (&mat)[NJ]) {
+        const int j8 = threadIdx.x;
+        own = j8 < (C >> 3);
+        if (!own) return;
+        x = *(const h16x8 *)(xp + 8 * j8);
+        lw = *(const h16x8 *)(ln_w + 8 * j8);
+        lb = *(const h16x8 *)(ln_b + 8 * j8);
+        if (sxp) sx = *(const h16x8 *)(sxp + 8 * j8);
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+            if (mixp[j]) mix[j] = *(const h16x8 *)(mixp[j] + 8 * j8);
+            if (U8) {
+                ry[j] = *(const h16x8 *)(mat[j].ry + 8 * j8);
+                my[j] = *(const h16x8 *)(mat[j].my + 8 * j8);
+            }
+        }
+    }
+
+    // red: 2 * DWAVES + 3 * NJ * DWAVES floats
+    // maa_form: the RWKV-6 mixing kx = xx + (prev - xx) * m instead of kx = xx * m + prev * (1 - m)
+    DEV void compute(int C, bool has_sx, const rwkv_half *const (&mixp)[NJ], h16 *const (&xs)[NJ], VecSums (&S)[NJ],
+                     rwkv_half *xx_out, float *red, bool maa_form = false) {
+        float m[2] = {0.f, 0.f};
+        if (own)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float f = (float)x[e];
+                m[0] += f;
+                m[1] += f * f;
+            }
+        block_sum_1b<2>(m, red);
+        const float mean = m[0] / C;
+        const float rstd = rsqrtf(fmaxf(m[1] / C - mean * mean, 0.f) + LN_EPS);
+        const int nseg = C >> 4, j8 = threadIdx.x;
+        float acc[3 * NJ];
+#pragma unroll
+        for (int i = 0; i < 3 * NJ; ++i) acc[i] = 0.f;
+        if (own) {
+            h16x8 xx;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) xx[e] = (h16)(((float)x[e] - mean) * rstd * (float)lw[e] + (float)lb[e]);
+            if (xx_out && blockIdx.x == 0) *(h16x8 *)(xx_out + 8 * j8) = xx;
+            const h16x8 pv = has_sx ? sx : xx;
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) {
+                h16x8 kx = xx;
+                if (mixp[j]) {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        const float mm = (float)mix[j][e];
+                        kx[e] = maa_form ? (h16)((float)xx[e] + (float)(h16)((float)pv[e] - (float)xx[e]) * mm)
+                                         : (h16)((float)xx[e] * mm + (float)pv[e] * (1.f - mm));
+                    }
+                }
+                h16x8 o = kx;
+                if (U8) {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        const float k = (float)kx[e];
+                        o[e] = (h16)(k * (float)ry[j][e]);
+                        acc[3 * j] += k;
+                        acc[3 * j + 1] += (float)o[e];
+                        acc[3 * j + 2] += k * (float)my[j][e];
+                    }
+                }
+                ((h16x8 *)xs[j])[xs_item<U8>(j8, nseg)] = o;
+            }
+        }
+        // one barrier publishes both the LDS activation vectors and the partial sums
+        block_sum_1b<3 * NJ>(acc, red + 2 * DWAVES);
+        if (U8)
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) { S[j].s0 = acc[3 * j]; S[j].s1 = acc[3 * j + 1]; S[j].s2 = acc[3 * j + 2]; }
+    }
+};
+
+template <bool U8>
+DEV const uint8_t *row_ptr(const MatDev &m, int64_t row) {
+    return (const uint8_t *)m.w + row * m.ld * (U8 ? 1 : 2);
+}
+
+template <bool U8>
+DEV float finish(float dot, const VecSums &S, float rx, float mx) {
+    return U8 ? mm8_finish(dot, S, rx, mx) : dot;
+}
+
+// Streaming body shared by the three kernels.  The row space is `ngroups` groups of K rows
+// (K = 3 for the time-mix kernel: the key, value and receptance row of one channel; K = 1
+// otherwise).  Every wave owns a contiguous range of groups and walks it as a flat sequence of
+// batches (G groups x U segments per lane), ping-ponging between two register tiles: the loads
+// of batch q+1 are in flight while batch q is multiplied.
+//   pro_load():           issue the loads of the prologue operands (called first)
+//   pro_compute():        build the LDS activation vectors (contains the workgroup barriers)
+//   rowf(g, k, row, xs):  weight row pointer and LDS activation vector of row k of group g
+//   epi_load(g) -> E:     loads of the operands the epilogue of group g needs (no dependence on
+//                         the dot products: issued together with the group's first weight tile)
+//   epi(g, dots, E):      called by one lane per group with the K reduced dot products
+template <bool U8, int G, int K, int U, class E, class ProLoad, class ProCompute, class RowFn, class EpiLoad, class EpiFn>
+DEV void stream_rows(int ngroups, int nseg, ProLoad pro_load, ProCompute pro_compute, RowFn rowf, EpiLoad epi_load,
+                     EpiFn epi) {
+    constexpr int R = G * K;
+    const int lane = threadIdx.x & 63;
+    const int wave = blockIdx.x * DWAVES + (threadIdx.x >> 6), nwaves = gridDim.x * DWAVES;
+    const int per = (ngroups + nwaves - 1) / nwaves;
+    const int g0 = min(wave * per, ngroups), g1 = min(g0 + per, ngroups);
+    const int nsb = (nseg + 64 * U - 1) / (64 * U);             // segment batches per group batch
+    const int nb = ((g1 - g0 + G - 1) / G) * nsb;               // batches of this wave
+    RowTile<U8, R, U> t0, t1;
+    E e0{}, e1{};
+    // epilogue operands live in slot (group batch index & 1): they are loaded with the first
+    // tile of a group batch and used after its last one, by when at most the next group batch
+    // has started loading
+    auto load = [&](RowTile<U8, R, U> &t, int q) {
+        const int gbi = q / nsb, gb = g0 + gbi * G, sb = q % nsb;
+        const uint8_t *rows[R];
+        const h16 *xs_unused;
+#pragma unroll
+        for (int i = 0; i < G; ++i)
+#pragma unroll
+            for (int k = 0; k < K; ++k) rowf(min(gb + i, g1 - 1), k, rows[i * K + k], xs_unused);
+        if (sb == 0 && lane < G && gb + lane < g1) {
+            const E e = epi_load(gb + lane);
+            if (gbi & 1) e1 = e; else e0 = e;
+        }
+        t.load(rows, sb * 64 * U, nseg);
+    };
+    float acc[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) acc[r] = 0.f;
+    auto process = [&](const RowTile<U8, R, U> &t, int q) {
+        const int gbi = q / nsb, sb = q % nsb, gb = g0 + gbi * G;
+        const uint8_t *row_unused;
+        const h16 *xs[R];
+#pragma unroll
+        for (int i = 0; i < G; ++i)
+#pragma unroll
+            for (int k = 0; k < K; ++k) rowf(min(gb + i, g1 - 1), k, row_unused, xs[i * K + k]);
+        t.consume(xs, sb * 64 * U, nseg, acc);
+        if (sb == nsb - 1) {
+#pragma unroll
+            for (int r = 0; r < R; ++r) acc[r] = wave_sum(acc[r]);
+            if (lane < G && gb + lane < g1) {
+                float d[K];
+#pragma unroll
+                for (int k = 0; k < K; ++k) {
+                    d[k] = acc[k];
+#pragma unroll
+                    for (int i = 1; i < G; ++i) d[k] = (lane == i) ? acc[i * K + k] : d[k];
+                }
+                epi(gb + lane, d, (gbi & 1) ? e1 : e0);
+            }
+#pragma unroll
+            for (int r = 0; r < R; ++r) acc[r] = 0.f;
+        }
+    };
+    pro_load();
+    if (nb > 0) load(t0, 0);
+    pro_compute();
+    for (int q = 0; q < nb; q += 2) {
+        if (q + 1 < nb) load(t1, q + 1);
+        process(t0, q);
+        if (q + 1 < nb) {
+            if (q + 2 < nb) load(t0, q + 2);
+            process(t1, q + 1);
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+struct AttArgs {
+    const rwkv_half *x, *emb;
+    const int32_t *token;
+    int C;
+    const rwkv_half *ln_w, *ln_b, *sx;
+    rwkv_half *xx_tmp;
+    const rwkv_half *mix[3];  // k, v, r
+    MatDev mat[3];            // key, value, receptance
+    const float *decay, *first;
+    float *aa, *bb, *pp;
+    rwkv_half *rwkv;          // out: r * wkv, fp16 [C]
+};
+
+struct AttEpi {
+    float rx[3], mx[3], u, w, aa, bb, pp;
+};
+
+template <bool U8, int G>
+__global__ __launch_bounds__(DTHREADS) void att_kernel(AttArgs a) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    __shared__ float red[(2 + 9) * DWAVES];
+    const int C = a.C;
+    h16 *xs[3] = {(h16 *)smem, (h16 *)smem + C, (h16 *)smem + 2 * C};
+    VecSums S[3];
+    LnMixPro<U8, 3> pro;
+    auto pro_load = [&]() {
+        pro.load(resolve_x(a.x, a.emb, a.token, C), C, a.ln_w, a.ln_b, a.sx, a.mix, a.mat);
+    };
+    auto pro_compute = [&]() { pro.compute(C, a.sx != nullptr, a.mix, xs, S, a.xx_tmp, red); };
+    auto rowf = [&](int c, int k, const uint8_t *&row, const h16 *&xv) {
+        row = row_ptr<U8>(a.mat[k], c);
+        xv = xs[k];
+    };
+    auto epi_load = [&](int c) {
+        AttEpi e;
+#pragma unroll
+        for (int k = 0; k < 3; ++k) {
+            e.rx[k] = U8 ? h2f(a.mat[k].rx[c]) : 1.f;
+            e.mx[k] = U8 ? h2f(a.mat[k].mx[c]) : 0.f;
+        }
+        e.u = a.first[c]; e.w = a.decay[c];
+        e.aa = a.aa[c]; e.bb = a.bb[c]; e.pp = a.pp[c];
+        return e;
+    };
+    auto epi = [&](int c, const float (&d)[3], const AttEpi &e) {
+        float k = finish<U8>(d[0], S[0], e.rx[0], e.mx[0]);
+        float v = finish<U8>(d[1], S[1], e.rx[1], e.mx[1]);
+        float r = finish<U8>(d[2], S[2], e.rx[2], e.mx[2]);
+        if (U8) { k = round_h(k); v = round_h(v); }  // uint8 path returns fp16, widened again
+        r = round_h(sigmoidf_(round_h(r)));
+        float ww = e.u + k;
+        float p = fmaxf(e.pp, ww);
+        float e1 = __expf(e.pp - p), e2 = __expf(ww - p);
+        const float wkv = (e1 * e.aa + e2 * v) / (e1 * e.bb + e2);
+        ww = e.w + e.pp;
+        p = fmaxf(ww, k);
+        e1 = __expf(ww - p);
+        e2 = __expf(k - p);
+        a.aa[c] = e1 * e.aa + e2 * v;
+        a.bb[c] = e1 * e.bb + e2;
+        a.pp[c] = p;
+        a.rwkv[c] = f2h(r * round_h(wkv));
+    };
+    stream_rows<U8, G, 3, 2, AttEpi>(C, (C * (U8 ? 1 : 2)) >> 4, pro_load, pro_compute, rowf, epi_load, epi);
+}
+
+// ------------------------------------------------------------------------------------------
+enum { EPI_SIGMOID = 0, EPI_RELU_SQ = 1, EPI_LOGITS = 2 };
+
+struct LnMixArgs {
+    const rwkv_half *x;
+    int C;
+    const rwkv_half *ln_w, *ln_b, *sx;
+    rwkv_half *xx_tmp;
+    const rwkv_half *mix[2];
+    MatDev mat[2];
+    int M[2];
+    int epi[2];
+    void *out[2];
+    int maa_form;
+};
+
+struct ScaleEpi {
+    float rx, mx;
+};
+
+template <bool U8, int NJ, int G>
+__global__ __launch_bounds__(DTHREADS) void lnmix_kernel(LnMixArgs a) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    __shared__ float red[(2 + 3 * NJ) * DWAVES];
+    const int C = a.C;
+    h16 *xs[NJ];
+    const rwkv_half *mix[NJ];
+    MatDev mat[NJ];
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) { xs[j] = (h16 *)smem + j * C; mix[j] = a.mix[j]; mat[j] = a.mat[j]; }
+    VecSums S[NJ];
+    const int M0 = a.M[0];
+    LnMixPro<U8, NJ> pro;
+    auto pro_load = [&]() { pro.load(a.x, C, a.ln_w, a.ln_b, a.sx, mix, mat); };
+    auto pro_compute = [&]() { pro.compute(C, a.sx != nullptr, mix, xs, S, a.xx_tmp, red, a.maa_form != 0); };
+    auto rowf = [&](int g, int, const uint8_t *&row, const h16 *&xv) {
+        const int j = (NJ > 1 && g >= M0) ? 1 : 0;
+        row = row_ptr<U8>(mat[j], j ? g - M0 : g);
+        xv = xs[j];
+    };
+    auto epi_load = [&](int g) {
+        const int j = (NJ > 1 && g >= M0) ? 1 : 0;
+        const int m = j ? g - M0 : g;
+        ScaleEpi e;
+        e.rx = U8 ? h2f(mat[j].rx[m]) : 1.f;
+        e.mx = U8 ? h2f(mat[j].mx[m]) : 0.f;
+        return e;
+    };
+    auto epi = [&](int g, const float (&d)[1], const ScaleEpi &e) {
+        const int j = (NJ > 1 && g >= M0) ? 1 : 0;
+        const int m = j ? g - M0 : g;
+        const float v = round_h(finish<U8>(d[0], S[j], e.rx, e.mx));
+        const int kind = a.epi[j];
+        if (kind == EPI_LOGITS) {
+            ((float *)a.out[j])[m] = v;
+        } else if (kind == EPI_SIGMOID) {
+            ((rwkv_half *)a.out[j])[m] = f2h(sigmoidf_(v));
+        } else {
+            const float t = fmaxf(v, 0.f);
+            ((rwkv_half *)a.out[j])[m] = f2h(t * t);
+        }
+    };
+    stream_rows<U8, G, 1, (G >= 4 ? 1 : 2), ScaleEpi>(M0 + (NJ > 1 ? a.M[1] : 0), (C * (U8 ? 1 : 2)) >> 4, pro_load,
+                                                      pro_compute, rowf, epi_load, epi);
+}
+
+// ------------------------------------------------------------------------------------------
+struct VecArgs {
+    const rwkv_half *vin;   // [N] fp16 input vector
+    int N, M;
+    MatDev mat;
+    const rwkv_half *x_in, *emb;  // residual source (emb row when token != NULL)
+    const int32_t *token;
+    int C;
+    const rwkv_half *gate;  // [M] or NULL
+    rwkv_half *x_out;       // [M]
+    float out_scale;
+    const rwkv_half *commit_src;  // scratch xx -> state, done by workgroup 0
+    rwkv_half *commit_dst;
+    int act;                // VACT_*
+    void *out;              // [M] fp16 (fp32 for VACT_F32) when act != VACT_RESIDUAL
+};
+
+// epilogues of vec_kernel: VACT_RESIDUAL is x_out = (x_in + gate * y) * out_scale; the others write
+// act(y) to `out` (y is first rounded to fp16 except for VACT_F32, which stores the raw sum)
+enum { VACT_RESIDUAL = 0, VACT_F16 = 1, VACT_SIGMOID = 2, VACT_RELU_SQ = 3, VACT_SILU = 4, VACT_TANH = 5, VACT_F32 = 6,
+       VACT_LOGITS = 7 /* fp16-rounded value stored as fp32 */ };
+
+struct VecEpi {
+    float rx, mx, xin, gate;
+};
+
+template <bool U8, int U>
+__global__ __launch_bounds__(DTHREADS) void vec_kernel(VecArgs a) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    __shared__ float red[3 * DWAVES];
+    const int N = a.N;
+    h16 *xs = (h16 *)smem;
+    VecSums S;
+    h16x8 pv[VP], pr[VP], pm[VP];
+    auto pro_load = [&]() {
+#pragma unroll
+        for (int i = 0; i < VP; ++i) {
+            const int j8 = threadIdx.x + i * DTHREADS;
+            if (j8 < (N >> 3)) {
+                pv[i] = *(const h16x8 *)(a.vin + 8 * j8);
+                if (U8) {
+                    pr[i] = *(const h16x8 *)(a.mat.ry + 8 * j8);
+                    pm[i] = *(const h16x8 *)(a.mat.my + 8 * j8);
+                }
+            }
+        }
+    };
+    auto pro_compute = [&]() {
+        if (blockIdx.x == 0 && a.commit_dst)
+            for (int j8 = threadIdx.x; j8 < (a.C >> 3); j8 += blockDim.x)
+                *(u32x4 *)(a.commit_dst + 8 * j8) = *(const u32x4 *)(a.commit_src + 8 * j8);
+        const int nseg = N >> 4;
+        float acc[3] = {0.f, 0.f, 0.f};
+#pragma unroll
+        for (int i = 0; i < VP; ++i) {
+            const int j8 = threadIdx.x + i * DTHREADS;
+            if (j8 < (N >> 3)) {
+                h16x8 o = pv[i];
+                if (U8) {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        const float k = (float)pv[i][e];
+                        o[e] = (h16)(k * (float)pr[i][e]);
+                        acc[0] += k;
+                        acc[1] += (float)o[e];
+                        acc[2] += k * (float)pm[i][e];
+                    }
+                }
+                ((h16x8 *)xs)[xs_item<U8>(j8, nseg)] = o;
+            }
+        }
+        block_sum_1b<3>(acc, red);  // the barrier also publishes xs
+        if (U8) { S.s0 = acc[0]; S.s1 = acc[1]; S.s2 = acc[2]; }
+    };
+    auto rowf = [&](int m, int, const uint8_t *&row, const h16 *&xv) {
+        row = row_ptr<U8>(a.mat, m);
+        xv = xs;
+    };
+    auto epi_load = [&](int m) {
+        VecEpi e;
+        e.rx = U8 ? h2f(a.mat.rx[m]) : 1.f;
+        e.mx = U8 ? h2f(a.mat.mx[m]) : 0.f;
+        e.xin = a.act == VACT_RESIDUAL ? h2f(resolve_x(a.x_in, a.emb, a.token, a.C)[m]) : 0.f;
+        e.gate = a.gate ? h2f(a.gate[m]) : 1.f;
+        return e;
+    };
+    auto epi = [&](int m, const float (&d)[1], const VecEpi &e) {
+        const float y = finish<U8>(d[0], S, e.rx, e.mx);
+        if (a.act == VACT_F32) { ((float *)a.out)[m] = y; return; }
+        float o = round_h(y);
+        if (a.act == VACT_LOGITS) { ((float *)a.out)[m] = o; return; }
+        switch (a.act) {
+            case VACT_RESIDUAL:
+                if (a.gate) o = round_h(e.gate * o);
+                o = round_h(e.xin + o);
+                a.x_out[m] = f2h(o * a.out_scale);
+                return;
+            case VACT_SIGMOID: o = sigmoidf_(o); break;
+            case VACT_RELU_SQ: o = fmaxf(o, 0.f); o = o * o; break;
+            case VACT_SILU: o = o * sigmoidf_(o); break;
+            case VACT_TANH: o = tanhf(o); break;
+            default: break;
+        }
+        ((rwkv_half *)a.out)[m] = f2h(o);
+    };
+    stream_rows<U8, 1, 1, U, VecEpi>(a.M, (N * (U8 ? 1 : 2)) >> 4, pro_load, pro_compute, rowf, epi_load, epi);
+}
+
+}  // namespace

@@ -193,6 +193,8 @@ __global__ __launch_bounds__(256) void gemm_kernel(int T, int N, int M, const h1
                 switch (ep.act) {
                     case ACT_SIGMOID: o = sigmoidf_(o); break;
                     case ACT_RELU_SQ: o = fmaxf(o, 0.f); o = o * o; break;
+                    case ACT_SILU: o = o * sigmoidf_(o); break;
+                    case ACT_TANH: o = tanhf(o); break;
                     case ACT_RESIDUAL: o = h2f(ep.res[(size_t)t * ep.ldres + m]) + o; break;
                     case ACT_GATED_RESIDUAL:
                         o = round_h(h2f(ep.gate[(size_t)t * ep.ldgate + m]) * o);

@@ -2,7 +2,7 @@
 #pragma once
 #include "common.h"
 
-enum { ACT_NONE = 0, ACT_SIGMOID = 1, ACT_RELU_SQ = 2, ACT_RESIDUAL = 3, ACT_GATED_RESIDUAL = 4 };
+enum { ACT_NONE = 0, ACT_SIGMOID = 1, ACT_RELU_SQ = 2, ACT_RESIDUAL = 3, ACT_GATED_RESIDUAL = 4, ACT_SILU = 5, ACT_TANH = 6 };
 
 // Epilogue of the MFMA contraction (gemm.hip).
 struct GemmEpi {
@@ -25,6 +25,26 @@ int gemv_f16_launch(int64_t N, int64_t M, const rwkv_half *x, const rwkv_half *w
 // kv_f32: k, v are fp32 (fp16-weight strategy) instead of fp16.
 int wkv4_fused_launch(int T, int C, const float *w, const float *u, const void *k, const void *v, int kv_f32,
                       const rwkv_half *r, rwkv_half *y, float *aa, float *bb, float *pp, hipStream_t st);
+int wkv56_fused_launch(bool v6, int T, int C, int H, float *state, const rwkv_half *r, const rwkv_half *k,
+                       const rwkv_half *v, const void *w, const float *t_decay, const float *u, const float *lnx_w,
+                       const float *lnx_b, const rwkv_half *gate, rwkv_half *out, hipStream_t st);
+// Row-wise LayerNorm + token shift + mixes for up to 4 consumers over a [T, C] activation (seq_v4.hip).
+struct SeqMixArgs {
+    int T, C;
+    const rwkv_half *x;        // [T, C]
+    const rwkv_half *ln_w, *ln_b;
+    const rwkv_half *sx;       // state (previous token's normalised activation), NULL = no token shift
+    rwkv_half *xx_last;        // scratch [C]: normalised activation of the last row (new state)
+    const rwkv_half *mix[4];   // NULL entry = consumer sees LN(x)
+    const rwkv_half *ry[4], *my[4];  // NULL ry = no scaling / sums (fp16 weights)
+    rwkv_half *xs[4];          // [T, C] outputs
+    float *s0[4], *s2[4];      // [T] outputs
+    int maa_form;              // RWKV-6 mixing kx = xx + (prev - xx) * m
+};
+
+int lnmix_seq_launch(const SeqMixArgs &a, int nj, hipStream_t st);
+int gather_emb_launch(int64_t T, int C, const int32_t *tokens, const rwkv_half *emb, rwkv_half *x, hipStream_t st);
+int copy_h16_launch(int n, const rwkv_half *src, rwkv_half *dst, hipStream_t st);
 int v4_model_check(const rwkv_v4_model *m);
 int v4_head_launch(const rwkv_v4_model *m, const rwkv_half *x, float *logits, hipStream_t st);
 int num_cu();

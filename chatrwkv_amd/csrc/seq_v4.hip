@@ -43,24 +43,12 @@ DEV void row_stats(const rwkv_half *x, int C, float *red, float &mean, float &rs
     rstd = rsqrtf(block_sum(q, red) / C + LN_EPS);
 }
 
-struct SeqMixArgs {
-    int T, C;
-    const rwkv_half *x;        // [T, C]
-    const rwkv_half *ln_w, *ln_b;
-    const rwkv_half *sx;       // state (previous token's normalised activation), NULL = no token shift
-    rwkv_half *xx_last;        // scratch [C]: normalised activation of the last row (new state)
-    const rwkv_half *mix[3];   // NULL entry = consumer sees LN(x)
-    const rwkv_half *ry[3], *my[3];  // NULL ry = no scaling / sums (fp16 weights)
-    rwkv_half *xs[3];          // [T, C] outputs
-    float *s0[3], *s2[3];      // [T] outputs
-};
-
 // One workgroup per token row.  Row t needs LN(x[t-1]) for the token shift: it is recomputed here
 // from x[t-1] (same code, same data => same bits as row t-1 computes for itself), which keeps all
 // rows independent.
 template <int NJ>
 __global__ __launch_bounds__(256) void lnmix_seq_kernel(SeqMixArgs a) {
-    __shared__ float red[2 * 3 * 4 + 4];
+    __shared__ float red[32];
     const int t = blockIdx.x, C = a.C;
     const rwkv_half *x = a.x + (size_t)t * C;
     float mean, rstd, pmean = 0.f, prstd = 0.f;
@@ -98,7 +86,8 @@ __global__ __launch_bounds__(256) void lnmix_seq_kernel(SeqMixArgs a) {
 #pragma unroll
                 for (int e = 0; e < 8; ++e) {
                     const float m = (float)mv[e];
-                    kx[e] = (h16)((float)xx[e] * m + (float)pv[e] * (1.f - m));
+                    kx[e] = a.maa_form ? (h16)((float)xx[e] + (float)(h16)((float)pv[e] - (float)xx[e]) * m)
+                                       : (h16)((float)xx[e] * m + (float)pv[e] * (1.f - m));
                 }
             }
             h16x8 o = kx;
@@ -137,6 +126,36 @@ __global__ __launch_bounds__(256) void ln_f32_f16_kernel(int C, const float *__r
     const float rstd = rsqrtf(block_sum(q, red) / C + LN_EPS);
     for (int j = threadIdx.x; j < C; j += blockDim.x) y[j] = f2h((x[j] - mean) * rstd * w[j] + b[j]);
 }
+
+}  // namespace
+
+int lnmix_seq_launch(const SeqMixArgs &a, int nj, hipStream_t st) {
+    const dim3 grid((unsigned)a.T), block(256);
+    switch (nj) {
+        case 1: hipLaunchKernelGGL(lnmix_seq_kernel<1>, grid, block, 0, st, a); break;
+        case 2: hipLaunchKernelGGL(lnmix_seq_kernel<2>, grid, block, 0, st, a); break;
+        case 3: hipLaunchKernelGGL(lnmix_seq_kernel<3>, grid, block, 0, st, a); break;
+        case 4: hipLaunchKernelGGL(lnmix_seq_kernel<4>, grid, block, 0, st, a); break;
+        default: return RWKV_E_DTYPE;
+    }
+    RWKV_LAUNCH_CHECK();
+    return RWKV_OK;
+}
+
+int gather_emb_launch(int64_t T, int C, const int32_t *tokens, const rwkv_half *emb, rwkv_half *x, hipStream_t st) {
+    hipLaunchKernelGGL(gather_emb_kernel, dim3((unsigned)T), dim3(256), 0, st, (int)T, C, tokens, emb, x);
+    RWKV_LAUNCH_CHECK();
+    return RWKV_OK;
+}
+
+int copy_h16_launch(int n, const rwkv_half *src, rwkv_half *dst, hipStream_t st) {
+    const int n16 = n >> 3;
+    hipLaunchKernelGGL(copy16_kernel, dim3((n16 + 255) / 256), dim3(256), 0, st, n16, (const u32x4 *)src, (u32x4 *)dst);
+    RWKV_LAUNCH_CHECK();
+    return RWKV_OK;
+}
+
+namespace {
 
 size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
@@ -232,7 +251,7 @@ extern "C" int rwkv_v4_forward_seq(const rwkv_v4_model *m, const rwkv_v4_layer_s
                 a.mix[j] = mix[j]; a.ry[j] = u8 ? mt[j]->ry : nullptr; a.my[j] = u8 ? mt[j]->my : nullptr;
                 a.xs[j] = ws.xs[j]; a.s0[j] = s0[j]; a.s2[j] = s2[j];
             }
-            hipLaunchKernelGGL(lnmix_seq_kernel<3>, dim3((unsigned)T), dim3(256), 0, st, a);
+            if ((rc = lnmix_seq_launch(a, 3, st))) return rc;
         }
         hipLaunchKernelGGL(copy16_kernel, dim3((n16 + 255) / 256), dim3(256), 0, st, n16, (const u32x4 *)ws.xx_att,
                            (u32x4 *)s.att_xx);
@@ -266,7 +285,7 @@ extern "C" int rwkv_v4_forward_seq(const rwkv_v4_model *m, const rwkv_v4_layer_s
                 a.mix[j] = mix[j]; a.ry[j] = u8 ? mt[j]->ry : nullptr; a.my[j] = u8 ? mt[j]->my : nullptr;
                 a.xs[j] = ws.xs[j]; a.s0[j] = s0[j]; a.s2[j] = s2[j];
             }
-            hipLaunchKernelGGL(lnmix_seq_kernel<2>, dim3((unsigned)T), dim3(256), 0, st, a);
+            if ((rc = lnmix_seq_launch(a, 2, st))) return rc;
         }
         hipLaunchKernelGGL(copy16_kernel, dim3((n16 + 255) / 256), dim3(256), 0, st, n16, (const u32x4 *)ws.xx_ffn,
                            (u32x4 *)s.ffn_xx);
@@ -293,7 +312,7 @@ extern "C" int rwkv_v4_forward_seq(const rwkv_v4_model *m, const rwkv_v4_layer_s
         a.xx_last = nullptr; a.mix[0] = nullptr;
         a.ry[0] = u8 ? m->head.ry : nullptr; a.my[0] = u8 ? m->head.my : nullptr;
         a.xs[0] = ws.xs[0]; a.s0[0] = s0[0]; a.s2[0] = s2[0];
-        hipLaunchKernelGGL(lnmix_seq_kernel<1>, dim3((unsigned)T), dim3(256), 0, st, a);
+        if ((rc = lnmix_seq_launch(a, 1, st))) return rc;
     }
     GemmEpi e{};
     e.out_scale = 1.f; e.act = ACT_NONE; e.out_dtype = RWKV_DT_F32;

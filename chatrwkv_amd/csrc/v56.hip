@@ -1,0 +1,333 @@
+// RWKV-5.x / RWKV-6 forward for any T >= 1.
+//
+// Per layer: time mix
+//   v5: lnmix_seq (LN1, token shift, static k/v/r(/g) mixes)
+//   v6: mix1 (LN1, sx = prev - xx, xxx = xx + sx * maa_x) -> tanh(xxx @ W1) -> mix2 (five rank-32
+//       products with W2 and the five data-dependent mixes) -> decay LoRA tanh(wx @ D1) @ D2
+//   r, k, v (fp16, widened by the consumer), g = SiLU(.) through mm() below
+//   wkv56 (per-head 64x64 state in registers for the whole T loop; decay exp(-exp(.)), GroupNorm
+//   and the gate fused) -> output matrix with the residual add in its epilogue
+// then the channel mix exactly as RWKV-4 (RWKV-6 mixes with kx = xx + (prev - xx) * maa).
+// mm(): T == 1 -> streaming GEMV (vec_kernel: ry scaling and the row sums in its prologue,
+// activation / residual in its epilogue); T > 1 -> mm8_prepare + MFMA GEMM with the same epilogues.
+#include "decode_kernels.h"
+
+namespace {
+
+constexpr float LN_EPS56 = 1e-5f;
+
+struct Mix1Args {
+    int T, C;
+    const rwkv_half *x, *ln_w, *ln_b, *sx, *maa_x;
+    rwkv_half *xx, *sxd, *xxx, *xx_last;
+};
+
+// grid T x 256 threads: xx = LN1(x[t]); sxd = prev - xx; xxx = xx + sxd * maa_x.
+__global__ __launch_bounds__(256) void v6_mix1_kernel(Mix1Args a) {
+    __shared__ float red[8];
+    const int t = blockIdx.x, C = a.C;
+    auto stats = [&](const rwkv_half *x, float &mean, float &rstd) {
+        float s = 0.f, q = 0.f;
+        for (int j8 = threadIdx.x; j8 < (C >> 3); j8 += blockDim.x) {
+            const h16x8 v = *(const h16x8 *)(x + 8 * j8);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) { const float f = (float)v[e]; s += f; q += f * f; }
+        }
+        s = block_sum(s, red);
+        q = block_sum(q, red);
+        mean = s / C;
+        rstd = rsqrtf(fmaxf(q / C - mean * mean, 0.f) + LN_EPS56);
+    };
+    const rwkv_half *x = a.x + (size_t)t * C;
+    float mean, rstd, pmean = 0.f, prstd = 0.f;
+    stats(x, mean, rstd);
+    if (t > 0) stats(x - C, pmean, prstd);
+    for (int j8 = threadIdx.x; j8 < (C >> 3); j8 += blockDim.x) {
+        const h16x8 xv = *(const h16x8 *)(x + 8 * j8);
+        const h16x8 wv = *(const h16x8 *)(a.ln_w + 8 * j8), bv = *(const h16x8 *)(a.ln_b + 8 * j8);
+        const h16x8 mv = *(const h16x8 *)(a.maa_x + 8 * j8);
+        h16x8 xx, pv, sd, xo;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) xx[e] = (h16)(((float)xv[e] - mean) * rstd * (float)wv[e] + (float)bv[e]);
+        if (t > 0) {
+            const h16x8 pxv = *(const h16x8 *)(x - C + 8 * j8);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) pv[e] = (h16)(((float)pxv[e] - pmean) * prstd * (float)wv[e] + (float)bv[e]);
+        } else {
+            pv = *(const h16x8 *)(a.sx + 8 * j8);
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            sd[e] = (h16)((float)pv[e] - (float)xx[e]);
+            xo[e] = (h16)((float)xx[e] + (float)(h16)((float)sd[e] * (float)mv[e]));
+        }
+        const size_t o = (size_t)t * C + 8 * j8;
+        *(h16x8 *)(a.xx + o) = xx;
+        *(h16x8 *)(a.sxd + o) = sd;
+        *(h16x8 *)(a.xxx + o) = xo;
+        if (t == a.T - 1) *(h16x8 *)(a.xx_last + 8 * j8) = xx;
+    }
+}
+
+struct Mix2Args {
+    int T, C, R;                     // R = LoRA rank (32)
+    const rwkv_half *t1;             // [T, 5R] tanh output
+    const rwkv_half *w2;             // [5][R][C]
+    const rwkv_half *xx, *sxd;       // [T, C]
+    const rwkv_half *maa[5];         // w, k, v, r, g
+    rwkv_half *out[5];               // [T, C] each
+};
+
+// grid (T, C/256): m_j[c] = sum_i t1[t, jR + i] * w2[j][i][c]; out_j = xx + sxd * (maa_j + m_j).
+__global__ __launch_bounds__(256) void v6_mix2_kernel(Mix2Args a) {
+    __shared__ float st1[5 * 64];
+    const int t = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x, R = a.R, C = a.C;
+    for (int i = threadIdx.x; i < 5 * R; i += 256) st1[i] = h2f(a.t1[(size_t)t * 5 * R + i]);
+    __syncthreads();
+    if (c >= C) return;
+    const float xx = h2f(a.xx[(size_t)t * C + c]), sd = h2f(a.sxd[(size_t)t * C + c]);
+#pragma unroll
+    for (int j = 0; j < 5; ++j) {
+        float m = 0.f;
+        const rwkv_half *w = a.w2 + (size_t)j * R * C + c;
+        for (int i = 0; i < R; ++i) m += st1[j * R + i] * h2f(w[(size_t)i * C]);
+        const float mm = round_h(h2f(a.maa[j][c]) + round_h(m));
+        a.out[j][(size_t)t * C + c] = f2h(xx + round_h(sd * mm));
+    }
+}
+
+MatDev to_dev56(const rwkv_mat &m) { return MatDev{m.w, m.ld, m.mx, m.rx, m.my, m.ry}; }
+
+struct Ctx {
+    hipStream_t st;
+    bool u8;
+    int64_t T;
+    int grid;
+    rwkv_half *xs;       // scaled-activation scratch [T, max(C, F)]
+    float *s0, *s2;      // [T]
+};
+
+// y = act(x @ W) for a model matrix (uint8 or fp16 per strategy) or an fp16 LoRA matrix.
+//   one-token: vec_kernel;  sequence: (prepare +) MFMA GEMM.  x [T, N] fp16 contiguous.
+// act: ACT_* of kernels.h; res/gate only for the residual epilogues; out fp16 [T, M].
+int mm(const Ctx &c, const rwkv_mat &m, bool mat_u8, const rwkv_half *x, int act, const rwkv_half *res,
+       const rwkv_half *gate, float out_scale, rwkv_half *out, const rwkv_half *commit_src = nullptr,
+       rwkv_half *commit_dst = nullptr, int commit_n = 0) {
+    const int N = (int)m.N, M = (int)m.M;
+    if (c.T == 1) {
+        VecArgs a{};
+        a.vin = x; a.N = N; a.M = M; a.mat = to_dev56(m);
+        a.x_in = res; a.emb = nullptr; a.token = nullptr; a.C = commit_n; a.gate = gate; a.x_out = out;
+        a.out_scale = out_scale; a.commit_src = commit_src; a.commit_dst = commit_dst; a.out = out;
+        switch (act) {
+            case ACT_NONE: a.act = VACT_F16; break;
+            case ACT_SIGMOID: a.act = VACT_SIGMOID; break;
+            case ACT_RELU_SQ: a.act = VACT_RELU_SQ; break;
+            case ACT_SILU: a.act = VACT_SILU; break;
+            case ACT_TANH: a.act = VACT_TANH; break;
+            default: a.act = VACT_RESIDUAL; break;
+        }
+        const size_t lds = (size_t)N * 2;
+        if (N > 8 * VP * DTHREADS) return RWKV_E_SHAPE;
+        if (mat_u8) {
+            if (N >= 8192) hipLaunchKernelGGL((vec_kernel<true, 8>), dim3(c.grid), dim3(DTHREADS), lds, c.st, a);
+            else hipLaunchKernelGGL((vec_kernel<true, 4>), dim3(c.grid), dim3(DTHREADS), lds, c.st, a);
+        } else {
+            if (N >= 8192) hipLaunchKernelGGL((vec_kernel<false, 8>), dim3(c.grid), dim3(DTHREADS), lds, c.st, a);
+            else hipLaunchKernelGGL((vec_kernel<false, 4>), dim3(c.grid), dim3(DTHREADS), lds, c.st, a);
+        }
+        RWKV_LAUNCH_CHECK();
+        return RWKV_OK;
+    }
+    if (commit_dst) {
+        int rc = copy_h16_launch(commit_n, commit_src, commit_dst, c.st);
+        if (rc) return rc;
+    }
+    const rwkv_half *A = x;
+    GemmEpi e{};
+    e.act = act; e.res = res; e.ldres = M; e.gate = gate; e.ldgate = M; e.out_scale = out_scale;
+    e.out_dtype = RWKV_DT_F16;
+    if (mat_u8) {
+        int rc = mm8_prepare_launch(c.T, N, x, N, m.ry, m.my, c.xs, c.s0, c.s2, c.st);
+        if (rc) return rc;
+        A = c.xs;
+        e.mx = m.mx; e.rx = m.rx; e.s0 = c.s0; e.s2 = c.s2;
+    }
+    return gemm_launch(mat_u8, c.T, N, M, A, N, m.w, m.ld, out, M, e, c.st);
+}
+
+size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
+
+struct Ws56 {
+    rwkv_half *x, *xx, *sxd, *xxx, *t1, *mix[5], *d1, *d2, *r, *k, *v, *g, *att, *vx, *xs, *xx_att, *xx_ffn;
+    float *sums;
+    size_t total;
+};
+
+Ws56 carve56(void *base, int64_t T, int64_t C, int64_t F, int64_t lm, int64_t ld) {
+    Ws56 w;
+    unsigned char *p = (unsigned char *)base;
+    auto take = [&](size_t bytes) { void *q = p; p += align256(bytes); return (rwkv_half *)q; };
+    const size_t tc = (size_t)T * C * 2, tf = (size_t)T * F * 2;
+    w.x = take(tc); w.xx = take(tc); w.sxd = take(tc); w.xxx = take(tc);
+    w.t1 = take((size_t)T * 5 * lm * 2);
+    for (int j = 0; j < 5; ++j) w.mix[j] = take(tc);
+    w.d1 = take((size_t)T * ld * 2); w.d2 = take(tc);
+    w.r = take(tc); w.k = take(tc); w.v = take(tc); w.g = take(tc); w.att = take(tc);
+    w.vx = take(tf); w.xs = take(tf > tc ? tf : tc);
+    w.xx_att = take((size_t)C * 2); w.xx_ffn = take((size_t)C * 2);
+    w.sums = (float *)take((size_t)T * 2 * sizeof(float));
+    w.total = (size_t)(p - (unsigned char *)base);
+    return w;
+}
+
+bool mat_ok56(const rwkv_mat &m, bool u8, int64_t N, int64_t M) {
+    if (!m.w || m.N != N || m.M != M || m.ld < N || !aligned16(m.w)) return false;
+    if (u8) return m.mx && m.rx && m.my && m.ry && !(m.ld & 15) && aligned16(m.my) && aligned16(m.ry);
+    return !(m.ld & 7);
+}
+
+rwkv_mat lora_mat(const rwkv_half *w, int64_t N, int64_t M) {
+    rwkv_mat m{};
+    m.w = w; m.ld = N; m.N = N; m.M = M;
+    return m;
+}
+
+}  // namespace
+
+static int v56_check(const rwkv_v56_model *m) {
+    if (!m || !m->layers || !m->emb || !m->ln_out_w || !m->ln_out_b) return RWKV_E_NULL;
+    const int64_t C = m->n_embd, F = m->n_ffn, V = m->vocab;
+    const int ver = m->version_x10;
+    if (ver != 50 && ver != 51 && ver != 52 && ver != 60) return RWKV_E_DTYPE;
+    if (m->n_layer <= 0 || C <= 0 || F <= 0 || V <= 0 || (C & 63) || (F & 63) || C > 8 * DTHREADS ||
+        F > 8 * VP * DTHREADS || m->n_head * 64 != C)
+        return RWKV_E_SHAPE;
+    if (ver == 60 && (m->lora_maa <= 0 || m->lora_maa > 64 || (m->lora_maa * 5) % 8 || m->lora_decay % 64 ||
+                      m->lora_decay <= 0))
+        return RWKV_E_SHAPE;
+    const bool u8 = m->weights_u8 != 0;
+    for (int i = 0; i < m->n_layer; ++i) {
+        const rwkv_v56_layer &l = m->layers[i];
+        if (!l.ln1_w || !l.ln1_b || !l.ln2_w || !l.ln2_b || !l.time_decay || !l.time_first || !l.lnx_w || !l.lnx_b ||
+            !l.ffn_mix_k || !l.ffn_mix_r)
+            return RWKV_E_NULL;
+        const int nmix = ver == 60 ? 6 : (ver == 50 ? 3 : 4);
+        for (int j = 0; j < nmix; ++j)
+            if (!l.att_mix[j]) return RWKV_E_NULL;
+        if (ver == 60 && (!l.tm_w1 || !l.tm_w2 || !l.td_w1 || !l.td_w2)) return RWKV_E_NULL;
+        if (!mat_ok56(l.att_key, u8, C, C) || !mat_ok56(l.att_value, u8, C, C) ||
+            !mat_ok56(l.att_receptance, u8, C, C) || !mat_ok56(l.att_output, u8, C, C) ||
+            (ver != 50 && !mat_ok56(l.att_gate, u8, C, C)) || !mat_ok56(l.ffn_key, u8, C, F) ||
+            !mat_ok56(l.ffn_receptance, u8, C, C) || !mat_ok56(l.ffn_value, u8, F, C))
+            return RWKV_E_LAYOUT;
+    }
+    if (!mat_ok56(m->head, u8, C, V)) return RWKV_E_LAYOUT;
+    return RWKV_OK;
+}
+
+extern "C" size_t rwkv_v56_workspace(const rwkv_v56_model *m, int64_t T) {
+    if (!m || T <= 0) return 0;
+    const int lm = m->lora_maa > 0 ? m->lora_maa : 32, ld = m->lora_decay > 0 ? m->lora_decay : 64;
+    return carve56((void *)256, T, m->n_embd, m->n_ffn, lm, ld).total;
+}
+
+extern "C" int rwkv_v56_forward(const rwkv_v56_model *m, const rwkv_v56_layer_state *states, const int32_t *tokens,
+                                int64_t T, int full_output, float *logits, void *workspace, size_t workspace_bytes,
+                                void *stream) {
+    int rc = v56_check(m);
+    if (rc) return rc;
+    if (!states || !tokens || !logits || !workspace) return RWKV_E_NULL;
+    if (T <= 0 || T > (1 << 20)) return RWKV_E_SHAPE;
+    if (workspace_bytes < rwkv_v56_workspace(m, T) || (((uintptr_t)workspace) & 255)) return RWKV_E_WORKSPACE;
+    for (int i = 0; i < m->n_layer; ++i) {
+        const rwkv_v56_layer_state &s = states[i];
+        if (!s.att_xx || !s.att_kv || !s.ffn_xx) return RWKV_E_NULL;
+        if (!aligned16(s.att_xx) || !aligned16(s.ffn_xx)) return RWKV_E_LAYOUT;
+    }
+    hipStream_t st = (hipStream_t)stream;
+    const int C = m->n_embd, F = m->n_ffn, H = m->n_head, ver = m->version_x10;
+    const bool u8 = m->weights_u8 != 0, v6 = ver == 60, gated = ver != 50;
+    const int lm = m->lora_maa, ld = m->lora_decay;
+    Ws56 ws = carve56(workspace, T, C, F, v6 ? lm : 32, v6 ? ld : 64);
+    Ctx c{st, u8, T, num_cu(), ws.xs, ws.sums, ws.sums + T};
+
+    if ((rc = gather_emb_launch(T, C, tokens, m->emb, ws.x, st))) return rc;
+    for (int i = 0; i < m->n_layer; ++i) {
+        const rwkv_v56_layer &l = m->layers[i];
+        const rwkv_v56_layer_state &s = states[i];
+        const rwkv_half *kx, *vx, *rx, *gx = nullptr, *wx = nullptr;
+        if (v6) {
+            Mix1Args a{(int)T, C, ws.x, l.ln1_w, l.ln1_b, s.att_xx, l.att_mix[0], ws.xx, ws.sxd, ws.xxx, ws.xx_att};
+            hipLaunchKernelGGL(v6_mix1_kernel, dim3((unsigned)T), dim3(256), 0, st, a);
+            if ((rc = mm(c, lora_mat(l.tm_w1, C, 5 * lm), false, ws.xxx, ACT_TANH, nullptr, nullptr, 1.f, ws.t1))) return rc;
+            Mix2Args b{};
+            b.T = (int)T; b.C = C; b.R = lm; b.t1 = ws.t1; b.w2 = l.tm_w2; b.xx = ws.xx; b.sxd = ws.sxd;
+            for (int j = 0; j < 5; ++j) { b.maa[j] = l.att_mix[1 + j]; b.out[j] = ws.mix[j]; }
+            hipLaunchKernelGGL(v6_mix2_kernel, dim3((unsigned)T, (unsigned)((C + 255) / 256)), dim3(256), 0, st, b);
+            wx = ws.mix[0]; kx = ws.mix[1]; vx = ws.mix[2]; rx = ws.mix[3]; gx = ws.mix[4];
+            if ((rc = mm(c, lora_mat(l.td_w1, C, ld), false, wx, ACT_TANH, nullptr, nullptr, 1.f, ws.d1))) return rc;
+            if ((rc = mm(c, lora_mat(l.td_w2, ld, C), false, ws.d1, ACT_NONE, nullptr, nullptr, 1.f, ws.d2))) return rc;
+        } else {
+            SeqMixArgs a{};
+            a.T = (int)T; a.C = C; a.x = ws.x; a.ln_w = l.ln1_w; a.ln_b = l.ln1_b; a.sx = s.att_xx;
+            a.xx_last = ws.xx_att;
+            const int nj = gated ? 4 : 3;
+            for (int j = 0; j < nj; ++j) { a.mix[j] = l.att_mix[j]; a.ry[j] = nullptr; a.my[j] = nullptr; a.xs[j] = ws.mix[j]; }
+            if ((rc = lnmix_seq_launch(a, nj, st))) return rc;
+            kx = ws.mix[0]; vx = ws.mix[1]; rx = ws.mix[2]; gx = gated ? ws.mix[3] : nullptr;
+        }
+        // the first matrix call also commits the new token-shift state (all readers of the old one are done)
+        if ((rc = mm(c, l.att_receptance, u8, rx, ACT_NONE, nullptr, nullptr, 1.f, ws.r, ws.xx_att, s.att_xx, C))) return rc;
+        if ((rc = mm(c, l.att_key, u8, kx, ACT_NONE, nullptr, nullptr, 1.f, ws.k))) return rc;
+        if ((rc = mm(c, l.att_value, u8, vx, ACT_NONE, nullptr, nullptr, 1.f, ws.v))) return rc;
+        if (gated && (rc = mm(c, l.att_gate, u8, gx, ACT_SILU, nullptr, nullptr, 1.f, ws.g))) return rc;
+        if ((rc = wkv56_fused_launch(v6, (int)T, C, H, s.att_kv, ws.r, ws.k, ws.v, v6 ? (const void *)ws.d2 : (const void *)l.time_decay,
+                                     l.time_decay, l.time_first, l.lnx_w, l.lnx_b, gated ? ws.g : nullptr, ws.att, st)))
+            return rc;
+        if ((rc = mm(c, l.att_output, u8, ws.att, ACT_RESIDUAL, ws.x, nullptr, 1.f, ws.x))) return rc;
+        // ---- channel mix
+        {
+            SeqMixArgs a{};
+            a.T = (int)T; a.C = C; a.x = ws.x; a.ln_w = l.ln2_w; a.ln_b = l.ln2_b; a.sx = s.ffn_xx;
+            a.xx_last = ws.xx_ffn; a.maa_form = v6 ? 1 : 0;
+            a.mix[0] = l.ffn_mix_r; a.mix[1] = l.ffn_mix_k;
+            for (int j = 0; j < 2; ++j) { a.ry[j] = nullptr; a.my[j] = nullptr; a.xs[j] = ws.mix[j]; }
+            if ((rc = lnmix_seq_launch(a, 2, st))) return rc;
+        }
+        if ((rc = mm(c, l.ffn_receptance, u8, ws.mix[0], ACT_SIGMOID, nullptr, nullptr, 1.f, ws.r, ws.xx_ffn, s.ffn_xx, C))) return rc;
+        if ((rc = mm(c, l.ffn_key, u8, ws.mix[1], ACT_RELU_SQ, nullptr, nullptr, 1.f, ws.vx))) return rc;
+        const float scale = (m->rescale_layer > 0 && (i + 1) % m->rescale_layer == 0) ? 0.5f : 1.f;
+        if ((rc = mm(c, l.ffn_value, u8, ws.vx, ACT_GATED_RESIDUAL, ws.x, ws.r, scale, ws.x))) return rc;
+        RWKV_LAUNCH_CHECK();
+    }
+    // ---- head
+    const bool all_rows = full_output && T > 1;
+    const int64_t TH = all_rows ? T : 1;
+    const rwkv_half *xh = all_rows ? ws.x : ws.x + (size_t)(T - 1) * C;
+    {
+        SeqMixArgs a{};
+        a.T = (int)TH; a.C = C; a.x = xh; a.ln_w = m->ln_out_w; a.ln_b = m->ln_out_b; a.sx = nullptr; a.xx_last = nullptr;
+        a.mix[0] = nullptr; a.ry[0] = nullptr; a.my[0] = nullptr; a.xs[0] = ws.xx;
+        if ((rc = lnmix_seq_launch(a, 1, st))) return rc;
+    }
+    if (TH == 1) {
+        VecArgs a{};
+        a.vin = ws.xx; a.N = C; a.M = m->vocab; a.mat = to_dev56(m->head); a.act = VACT_LOGITS; a.out = logits;
+        a.out_scale = 1.f;
+        const size_t lds = (size_t)C * 2;
+        if (u8) hipLaunchKernelGGL((vec_kernel<true, 4>), dim3(c.grid), dim3(DTHREADS), lds, st, a);
+        else hipLaunchKernelGGL((vec_kernel<false, 4>), dim3(c.grid), dim3(DTHREADS), lds, st, a);
+        RWKV_LAUNCH_CHECK();
+        return RWKV_OK;
+    }
+    const rwkv_half *A = ws.xx;
+    GemmEpi e{};
+    e.out_scale = 1.f; e.act = ACT_NONE; e.out_dtype = RWKV_DT_F32;
+    if (u8) {
+        if ((rc = mm8_prepare_launch(TH, C, ws.xx, C, m->head.ry, m->head.my, ws.xs, ws.sums, ws.sums + T, st))) return rc;
+        A = ws.xs;
+        e.mx = m->head.mx; e.rx = m->head.rx; e.s0 = ws.sums; e.s2 = ws.sums + T;
+    }
+    return gemm_launch(u8, TH, C, m->vocab, A, C, m->head.w, m->head.ld, logits, m->vocab, e, st);
+}

@@ -98,40 +98,63 @@ __global__ __launch_bounds__(64) void wkv4_kernel(int T, int C, const float *__r
 constexpr int HS = 64;   // head size
 constexpr int TS = 16;   // tokens per slab
 
-template <bool PER_TOKEN_W>
-__global__ __launch_bounds__(256) void wkv56_kernel(int T, int C, float *__restrict__ state, int state_layout,
-                                                    const float *__restrict__ r_, const float *__restrict__ k_,
-                                                    const float *__restrict__ v_, const float *__restrict__ w_,
-                                                    const float *__restrict__ u_, float *__restrict__ y_) {
+// Operand forms of the fused model path:
+//   IN_F16   r, k, v are fp16 (the fp16-rounded GEMM outputs, widened here) instead of fp32
+//   WMODE 0  w[C] fp32, constant decay in (0,1)                         (RWKV-5)
+//   WMODE 1  w[T, C] fp32, already exp(-exp(.))                          (RWKV-6 operator interface)
+//   WMODE 2  w[T, C] fp16 LoRA output; decay = exp(-exp(t_decay[c] + w)) (RWKV-6 model path)
+//   OUT_GN   instead of y fp32, write fp16( fp16(GroupNorm_head(y) * lnx_w + lnx_b) * gate )
+//            (GroupNorm over the 64 channels of the head, eps 64e-5, biased variance; gate optional)
+struct Wkv56Args {
+    int T, C;
+    float *state;
+    int state_layout;
+    const void *r, *k, *v, *w;
+    const float *u, *t_decay;
+    float *y;
+    const float *lnx_w, *lnx_b;
+    const rwkv_half *gate;
+    rwkv_half *out;
+};
+
+template <bool IN_F16, int WMODE, bool OUT_GN>
+__global__ __launch_bounds__(256) void wkv56_kernel(Wkv56Args a) {
     __shared__ __align__(16) float sr[TS][HS], sk[TS][HS], sv[TS][HS], sw[TS][HS];
     __shared__ __align__(16) float su[HS];
     __shared__ float part[TS][4][HS];
+    const int T = a.T, C = a.C;
     const int h = blockIdx.x;
     const int i = threadIdx.x & 63, q = threadIdx.x >> 6;
-    float *S = state + (size_t)h * HS * HS;
+    float *S = a.state + (size_t)h * HS * HS;
     float s[16];
 #pragma unroll
     for (int jj = 0; jj < 16; ++jj) {
         const int j = 16 * q + jj;
-        s[jj] = state_layout == 0 ? S[i * HS + j] : S[j * HS + i];
+        s[jj] = a.state_layout == 0 ? S[i * HS + j] : S[j * HS + i];
     }
+    float tdec = 0.f;
+    if (WMODE == 2) tdec = a.t_decay[h * HS + i];
     if (threadIdx.x < HS) {
-        su[threadIdx.x] = u_[h * HS + threadIdx.x];
-        if (!PER_TOKEN_W) sw[0][threadIdx.x] = w_[h * HS + threadIdx.x];
+        su[threadIdx.x] = a.u[h * HS + threadIdx.x];
+        if (WMODE == 0) sw[0][threadIdx.x] = ((const float *)a.w)[h * HS + threadIdx.x];
     }
+    auto ld = [&](const void *p, size_t o) -> float {
+        return IN_F16 ? h2f(((const rwkv_half *)p)[o]) : ((const float *)p)[o];
+    };
     for (int t0 = 0; t0 < T; t0 += TS) {
         const int nt = min(TS, T - t0);
         __syncthreads();  // previous slab fully consumed (and su / sw[0] visible)
         for (int e = threadIdx.x; e < nt * HS; e += 256) {
             const int tt = e >> 6, c = e & 63;
             const size_t o = (size_t)(t0 + tt) * C + h * HS + c;
-            sr[tt][c] = r_[o]; sk[tt][c] = k_[o]; sv[tt][c] = v_[o];
-            if (PER_TOKEN_W) sw[tt][c] = w_[o];
+            sr[tt][c] = ld(a.r, o); sk[tt][c] = ld(a.k, o); sv[tt][c] = ld(a.v, o);
+            if (WMODE == 1) sw[tt][c] = ((const float *)a.w)[o];
+            if (WMODE == 2) sw[tt][c] = expf(-expf(tdec + h2f(((const rwkv_half *)a.w)[o])));
         }
         __syncthreads();
         for (int tt = 0; tt < nt; ++tt) {
             const float vi = sv[tt][i];
-            const float *wrow = PER_TOKEN_W ? sw[tt] : sw[0];
+            const float *wrow = WMODE != 0 ? sw[tt] : sw[0];
             float y = 0.f;
 #pragma unroll
             for (int jj = 0; jj < 16; jj += 4) {
@@ -150,15 +173,29 @@ __global__ __launch_bounds__(256) void wkv56_kernel(int T, int C, float *__restr
             part[tt][q][i] = y;
         }
         __syncthreads();
-        for (int e = threadIdx.x; e < nt * HS; e += 256) {
-            const int tt = e >> 6, c = e & 63;
-            y_[(size_t)(t0 + tt) * C + h * HS + c] = (part[tt][0][c] + part[tt][1][c]) + (part[tt][2][c] + part[tt][3][c]);
+        // wave q finishes tokens q, q+4, ...: lane = channel, so the GroupNorm of a token's head is
+        // a wave reduction
+        for (int tt = q; tt < nt; tt += 4) {
+            const int c = i;
+            const float y = (part[tt][0][c] + part[tt][1][c]) + (part[tt][2][c] + part[tt][3][c]);
+            const size_t o = (size_t)(t0 + tt) * C + h * HS + c;
+            if (!OUT_GN) {
+                a.y[o] = y;
+            } else {
+                const float mean = wave_sum(y) * (1.f / HS);
+                const float d = y - mean;
+                const float var = wave_sum(d * d) * (1.f / HS);
+                float g = d * rsqrtf(var + 64e-5f) * a.lnx_w[h * HS + c] + a.lnx_b[h * HS + c];
+                g = round_h(g);
+                if (a.gate) g = g * h2f(a.gate[o]);
+                a.out[o] = f2h(g);
+            }
         }
     }
 #pragma unroll
     for (int jj = 0; jj < 16; ++jj) {
         const int j = 16 * q + jj;
-        if (state_layout == 0) S[i * HS + j] = s[jj]; else S[j * HS + i] = s[jj];
+        if (a.state_layout == 0) S[i * HS + j] = s[jj]; else S[j * HS + i] = s[jj];
     }
 }
 
@@ -201,12 +238,31 @@ static int wkv56_launch(bool v6, int64_t B, int64_t T, int64_t C, int64_t H, flo
     if (!state || !r || !k || !v || !w || !u || !y) return RWKV_E_NULL;
     if (B != 1 || T <= 0 || H <= 0 || C != H * HS) return RWKV_E_SHAPE;
     if (state_layout != 0 && state_layout != 1) return RWKV_E_DTYPE;
+    Wkv56Args a{};
+    a.T = (int)T; a.C = (int)C; a.state = state; a.state_layout = state_layout;
+    a.r = r; a.k = k; a.v = v; a.w = w; a.u = u; a.y = y;
     if (v6)
-        hipLaunchKernelGGL(wkv56_kernel<true>, dim3((unsigned)H), dim3(256), 0, (hipStream_t)stream, (int)T, (int)C,
-                           state, state_layout, r, k, v, w, u, y);
+        hipLaunchKernelGGL((wkv56_kernel<false, 1, false>), dim3((unsigned)H), dim3(256), 0, (hipStream_t)stream, a);
     else
-        hipLaunchKernelGGL(wkv56_kernel<false>, dim3((unsigned)H), dim3(256), 0, (hipStream_t)stream, (int)T, (int)C,
-                           state, state_layout, r, k, v, w, u, y);
+        hipLaunchKernelGGL((wkv56_kernel<false, 0, false>), dim3((unsigned)H), dim3(256), 0, (hipStream_t)stream, a);
+    RWKV_LAUNCH_CHECK();
+    return RWKV_OK;
+}
+
+// Model path: fp16 r, k, v; state in list layout [h][key][value]; GroupNorm (+ gate) fused; fp16 out.
+// v6: w = fp16 LoRA output [T, C], t_decay fp32 [C]; v5: w = fp32 decay [C], t_decay unused.
+int wkv56_fused_launch(bool v6, int T, int C, int H, float *state, const rwkv_half *r, const rwkv_half *k,
+                       const rwkv_half *v, const void *w, const float *t_decay, const float *u, const float *lnx_w,
+                       const float *lnx_b, const rwkv_half *gate, rwkv_half *out, hipStream_t st) {
+    if (C != H * HS) return RWKV_E_SHAPE;
+    Wkv56Args a{};
+    a.T = T; a.C = C; a.state = state; a.state_layout = 1;
+    a.r = r; a.k = k; a.v = v; a.w = w; a.u = u; a.t_decay = t_decay;
+    a.lnx_w = lnx_w; a.lnx_b = lnx_b; a.gate = gate; a.out = out;
+    if (v6)
+        hipLaunchKernelGGL((wkv56_kernel<true, 2, true>), dim3((unsigned)H), dim3(256), 0, st, a);
+    else
+        hipLaunchKernelGGL((wkv56_kernel<true, 0, true>), dim3((unsigned)H), dim3(256), 0, st, a);
     RWKV_LAUNCH_CHECK();
     return RWKV_OK;
 }

@@ -63,7 +63,33 @@ class RwkvV4Model(ctypes.Structure):
                 ("layers", ctypes.POINTER(RwkvV4Layer))]
 
 
+class RwkvV56Layer(ctypes.Structure):
+    _fields_ = [("ln1_w", _vp), ("ln1_b", _vp), ("ln2_w", _vp), ("ln2_b", _vp),
+                ("att_mix", _vp * 6),
+                ("tm_w1", _vp), ("tm_w2", _vp), ("td_w1", _vp), ("td_w2", _vp),
+                ("time_decay", _vp), ("time_first", _vp), ("lnx_w", _vp), ("lnx_b", _vp),
+                ("att_key", RwkvMat), ("att_value", RwkvMat), ("att_receptance", RwkvMat), ("att_gate", RwkvMat),
+                ("att_output", RwkvMat),
+                ("ffn_mix_k", _vp), ("ffn_mix_r", _vp),
+                ("ffn_key", RwkvMat), ("ffn_receptance", RwkvMat), ("ffn_value", RwkvMat)]
+
+
+class RwkvV56LayerState(ctypes.Structure):
+    _fields_ = [("att_xx", _vp), ("att_kv", _vp), ("ffn_xx", _vp)]
+
+
+class RwkvV56Model(ctypes.Structure):
+    _fields_ = [("version_x10", ctypes.c_int32), ("n_layer", ctypes.c_int32), ("n_embd", ctypes.c_int32),
+                ("n_ffn", ctypes.c_int32), ("vocab", ctypes.c_int32), ("n_head", ctypes.c_int32),
+                ("lora_maa", ctypes.c_int32), ("lora_decay", ctypes.c_int32),
+                ("rescale_layer", ctypes.c_int32), ("weights_u8", ctypes.c_int32),
+                ("emb", _vp), ("ln_out_w", _vp), ("ln_out_b", _vp), ("head", RwkvMat),
+                ("layers", ctypes.POINTER(RwkvV56Layer))]
+
+
 SIGNATURES.update({
+    "rwkv_v56_workspace": (_sz, [ctypes.POINTER(RwkvV56Model), _i64]),
+    "rwkv_v56_forward": (_int, [ctypes.POINTER(RwkvV56Model), ctypes.POINTER(RwkvV56LayerState), _vp, _i64, _int, _vp, _vp, _sz, _vp]),
     "rwkv_layernorm_f32_f16": (_int, [_i64, _i64, _vp, _vp, _vp, _vp, _vp]),
     "rwkv_v4_one_workspace": (_sz, [ctypes.POINTER(RwkvV4Model)]),
     "rwkv_v4_forward_one": (_int, [ctypes.POINTER(RwkvV4Model), ctypes.POINTER(RwkvV4LayerState), _vp, _vp, _vp, _sz, _vp]),

@@ -109,9 +109,10 @@ class RWKV:
                   f"{'-stream' if s.stream else ''}", end=' ')
         prxxx()
         self._wkind = _strategy.require_single_gpu(self.strategy)    # NotImplementedError otherwise
-        if self.version != 4:
-            raise NotImplementedError(f"RWKV v{self.version} is not wired into chatrwkv_amd.RWKV yet "
-                                      "(the v5/v6 operators are in chatrwkv_amd.ops)")
+        if self.version not in (4, 5, 5.1, 5.2, 6):
+            raise NotImplementedError(f"RWKV v{self.version} is not supported")
+        if int(self.version) in (5, 6) and args.n_att // max(args.n_head, 1) != 64:
+            raise NotImplementedError("RWKV-5/6 kernels are built for head size 64")
         if args.n_att != args.n_embd:
             raise NotImplementedError("n_att != n_embd")
         _lib.load()                                                   # fail early and loudly
@@ -125,7 +126,10 @@ class RWKV:
             if convert_and_save_and_exit:
                 self._save_converted(convert_and_save_and_exit, prxxx)
                 raise SystemExit(0)                                   # model.py:903
-            self._build_descriptors()
+            if self.version == 4:
+                self._build_descriptors()
+            else:
+                self._build_descriptors_v56()
         self._graphs = collections.OrderedDict()
         self._seq_ws = None
         gc.collect()
@@ -140,6 +144,10 @@ class RWKV:
         st = torch.cuda.current_stream().cuda_stream
         u8 = self._wkind == 'u8'
         out = {}
+        real_time_first = any('.time_faaaa' in k for k in w)          # model.py:764-771
+        if real_time_first:
+            w = {k.replace('.time_faaaa', '.time_first'): v for k, v in w.items()}
+        args.time_state = any('.time_state' in k for k in w)
         if not converted:
             emb = w['emb.weight'].to(device=dev, dtype=torch.float32).contiguous()
             ln_w = w['blocks.0.ln0.weight'].to(device=dev, dtype=torch.float32).contiguous()
@@ -156,7 +164,8 @@ class RWKV:
                 continue
             t = w[x]
             layer_id = int(x.split('.')[1]) if ('blocks.' in x) else 0
-            is_matrix = any(s in x for s in _MATRIX_KEYS) and not x.endswith(('_mx', '_rx', '_my', '_ry'))
+            is_matrix = (any(s in x for s in _MATRIX_KEYS) and not x.endswith(('_mx', '_rx', '_my', '_ry'))
+                         and t.dim() == 2)
             if converted:
                 if is_matrix:
                     # reference device layout [in, out] with out contiguous -> input-contiguous
@@ -182,10 +191,24 @@ class RWKV:
             t = t.detach().to('cpu')
             if '.time_' in x:
                 t = t.squeeze()
-            if '.time_decay' in x and '_w' not in x:
-                t = -torch.exp(t.float())                             # model.py:797-798
-            elif '.time_first' in x:
-                t = t.float()                                         # model.py:806-807
+            if '.time_decay' in x and '_w' not in x:                  # model.py:796-804
+                if self.version == 4:
+                    t = -torch.exp(t.float())
+                elif int(self.version) == 5:
+                    t = torch.exp(-torch.exp(t.float())).reshape(-1, 1, 1)
+                    if self.version == 5.2:
+                        t = t.reshape(args.n_head, -1, 1)
+                else:
+                    t = t.float().reshape(args.n_head, -1, 1)
+            elif '.time_first' in x:                                  # model.py:805-814
+                if self.version == 4:
+                    t = t.float()
+                else:
+                    t = (t.float() if real_time_first else torch.exp(t.float())).reshape(-1, 1, 1)
+                    if self.version in (5.2, 6):
+                        t = t.reshape(args.n_head, -1, 1)
+            elif '.ln_x' in x:                                        # model.py:815-816
+                t = t.float()
             else:
                 t = t.to(torch.float16)                               # model.py:849
             out[x] = t.contiguous().to(dev)
@@ -252,8 +275,76 @@ class RWKV:
         self._token_dev = torch.zeros(1, dtype=torch.int32, device=self.device)
         self._logits = torch.empty(m.vocab, dtype=torch.float32, device=self.device)
 
+    def _build_descriptors_v56(self):
+        """Descriptors for RWKV-5.x / 6.0.  The per-head decay / bonus tensors are flattened to [C]
+        (one value per channel; 5.0 / 5.1 broadcast the per-head value), and the RWKV-6 LoRA
+        matrices time_maa_w1 / time_decay_w1 / time_decay_w2 are kept input-contiguous."""
+        a, w, dev = self.args, self.w, self.device
+        C, H = a.n_embd, a.n_head
+        N = C // H
+        v6 = self.version == 6
+        keep = self._keep = []
+        layers = (_lib.RwkvV56Layer * a.n_layer)()
+
+        def per_channel(t):
+            t = t.to(torch.float32).reshape(H, -1)
+            t = t.expand(H, N).contiguous().reshape(C) if t.shape[1] == 1 else t.reshape(C).contiguous()
+            keep.append(t)
+            return t.data_ptr()
+
+        def kept(t):
+            keep.append(t)
+            return t.data_ptr()
+
+        for i in range(a.n_layer):
+            b, at, ff = f'blocks.{i}.', f'blocks.{i}.att.', f'blocks.{i}.ffn.'
+            l = layers[i]
+            l.ln1_w, l.ln1_b = w[b + 'ln1.weight'].data_ptr(), w[b + 'ln1.bias'].data_ptr()
+            l.ln2_w, l.ln2_b = w[b + 'ln2.weight'].data_ptr(), w[b + 'ln2.bias'].data_ptr()
+            if v6:
+                for j, c in enumerate('xwkvrg'):
+                    l.att_mix[j] = w[at + 'time_maa_' + c].data_ptr()
+                l.tm_w1 = kept(w[at + 'time_maa_w1'].t().contiguous())
+                l.tm_w2 = kept(w[at + 'time_maa_w2'].contiguous())
+                l.td_w1 = kept(w[at + 'time_decay_w1'].t().contiguous())
+                l.td_w2 = kept(w[at + 'time_decay_w2'].t().contiguous())
+                l.ffn_mix_k, l.ffn_mix_r = w[ff + 'time_maa_k'].data_ptr(), w[ff + 'time_maa_r'].data_ptr()
+            else:
+                for j, c in enumerate('kvrg' if self.version >= 5.1 else 'kvr'):
+                    l.att_mix[j] = w[at + 'time_mix_' + c].data_ptr()
+                l.ffn_mix_k, l.ffn_mix_r = w[ff + 'time_mix_k'].data_ptr(), w[ff + 'time_mix_r'].data_ptr()
+            l.time_decay = per_channel(w[at + 'time_decay'])
+            l.time_first = per_channel(w[at + 'time_first'])
+            l.lnx_w, l.lnx_b = w[at + 'ln_x.weight'].data_ptr(), w[at + 'ln_x.bias'].data_ptr()
+            l.att_key, l.att_value = self._mat(at + 'key.weight'), self._mat(at + 'value.weight')
+            l.att_receptance, l.att_output = self._mat(at + 'receptance.weight'), self._mat(at + 'output.weight')
+            if self.version >= 5.1:
+                l.att_gate = self._mat(at + 'gate.weight')
+            l.ffn_key, l.ffn_receptance = self._mat(ff + 'key.weight'), self._mat(ff + 'receptance.weight')
+            l.ffn_value = self._mat(ff + 'value.weight')
+        m = _lib.RwkvV56Model()
+        m.version_x10 = int(round(self.version * 10))
+        m.n_layer, m.n_embd, m.n_ffn, m.n_head = a.n_layer, C, a.n_ffn, H
+        m.vocab = w['emb.weight'].shape[0]
+        if v6:
+            m.lora_maa = w['blocks.0.att.time_maa_w2'].shape[1]
+            m.lora_decay = w['blocks.0.att.time_decay_w1'].shape[1]
+        m.rescale_layer = self.RESCALE_LAYER
+        m.weights_u8 = 1 if self._wkind == 'u8' else 0
+        m.emb = w['emb.weight'].data_ptr()
+        m.ln_out_w, m.ln_out_b = w['ln_out.weight'].data_ptr(), w['ln_out.bias'].data_ptr()
+        m.head = self._mat('head.weight')
+        m.layers = layers
+        self._layers, self._model = layers, m
+        self._token_dev = torch.zeros(1, dtype=torch.int32, device=dev)
+        self._logits = torch.empty(m.vocab, dtype=torch.float32, device=dev)
+        nbytes = _lib.load().rwkv_v56_workspace(ctypes.byref(m), 1)
+        self._one_ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+
     # ------------------------------------------------------------------ state
     def _new_state(self):
+        if self.version != 4:
+            return self._new_state_v56()
         """model.py:1448-1459: per layer [xx fp16 (C), aa, bb fp32 (C), pp fp32 = -1e30, ffn_xx fp16 (C)],
         carved from two flat buffers."""
         a, dev = self.args, self.device
@@ -273,8 +364,50 @@ class RWKV:
         st.views = list(st)
         return st
 
+    def _new_state_v56(self):
+        """model.py:1460-1471: per layer [xx fp16 (C), kv fp32 (H, N, N) laid out [h][key][value], ffn_xx fp16 (C)]."""
+        a, dev = self.args, self.device
+        C, L, H = a.n_embd, a.n_layer, a.n_head
+        N = C // H
+        f16 = torch.zeros(L * 2 * C, dtype=torch.float16, device=dev)
+        f32 = torch.zeros(L * H * N * N, dtype=torch.float32, device=dev)
+        st = StateList()
+        for i in range(L):
+            st.append(f16[(2 * i) * C:(2 * i + 1) * C])
+            kv = f32[i * H * N * N:(i + 1) * H * N * N].view(H, N, N)
+            if a.time_state:                                          # model.py:1467-1468
+                kv.copy_(self.w[f'blocks.{i}.att.time_state'].transpose(1, 2).to(torch.float32))
+            st.append(kv)
+            st.append(f16[(2 * i + 1) * C:(2 * i + 2) * C])
+        st.flat = (f16, f32)
+        st.views = list(st)
+        return st
+
+    def _state_desc_v56(self, state):
+        a = self.args
+        if len(state) != 3 * a.n_layer:
+            raise ValueError(f"state must hold {3 * a.n_layer} tensors")
+        H = a.n_head
+        N = a.n_embd // H
+        arr = (_lib.RwkvV56LayerState * a.n_layer)()
+        for i in range(a.n_layer):
+            xx, kv, fx = state[3 * i:3 * i + 3]
+            ok = (xx.is_cuda and xx.dtype == torch.float16 and xx.is_contiguous() and xx.numel() == a.n_embd and
+                  fx.is_cuda and fx.dtype == torch.float16 and fx.is_contiguous() and fx.numel() == a.n_embd and
+                  kv.is_cuda and kv.dtype == torch.float32 and tuple(kv.shape) == (H, N, N))
+            if not ok:
+                raise ValueError("state tensors must be GPU tensors with the layout of model.py:1460-1471")
+            if not kv.is_contiguous():
+                # the reference's CUDA sequence path hands back a transposed view (model.py:1384)
+                kv = state[3 * i + 1] = kv.contiguous()
+            s = arr[i]
+            s.att_xx, s.att_kv, s.ffn_xx = xx.data_ptr(), kv.data_ptr(), fx.data_ptr()
+        return arr
+
     def _state_desc(self, state):
         a = self.args
+        if self.version != 4:
+            return self._state_desc_v56(state)
         if len(state) != 5 * a.n_layer:
             raise ValueError(f"state must hold {5 * a.n_layer} tensors")
         arr = (_lib.RwkvV4LayerState * a.n_layer)()
@@ -291,6 +424,12 @@ class RWKV:
     # ------------------------------------------------------------------ forward
     def _launch_one(self, sdesc):
         L = _lib.load()
+        if self.version != 4:
+            rc = L.rwkv_v56_forward(ctypes.byref(self._model), sdesc, self._token_dev.data_ptr(), 1, 0,
+                                    self._logits.data_ptr(), self._one_ws.data_ptr(), self._one_ws.numel(),
+                                    torch.cuda.current_stream().cuda_stream)
+            _lib.check(rc, "rwkv_v56_forward")
+            return
         rc = L.rwkv_v4_forward_one(ctypes.byref(self._model), sdesc, self._token_dev.data_ptr(),
                                    self._logits.data_ptr(), self._one_ws.data_ptr(), self._one_ws.numel(),
                                    torch.cuda.current_stream().cuda_stream)
@@ -349,16 +488,20 @@ class RWKV:
         L = _lib.load()
         T = len(tokens)
         tok = torch.tensor(tokens, dtype=torch.int32).to(self.device)
-        nbytes = L.rwkv_v4_seq_workspace(ctypes.byref(self._model), T, int(full_output))
+        if self.version != 4:
+            nbytes = L.rwkv_v56_workspace(ctypes.byref(self._model), T)
+        else:
+            nbytes = L.rwkv_v4_seq_workspace(ctypes.byref(self._model), T, int(full_output))
         if self._seq_ws is None or self._seq_ws.numel() < nbytes:
             self._seq_ws = None
             self._seq_ws = torch.empty(nbytes, dtype=torch.uint8, device=self.device)
         V = self._model.vocab
         logits = torch.empty((T, V) if full_output else (V,), dtype=torch.float32, device=self.device)
-        rc = L.rwkv_v4_forward_seq(ctypes.byref(self._model), self._state_desc(state), tok.data_ptr(), T,
-                                   int(full_output), logits.data_ptr(), self._seq_ws.data_ptr(),
-                                   self._seq_ws.numel(), torch.cuda.current_stream().cuda_stream)
-        _lib.check(rc, "rwkv_v4_forward_seq")
+        fn = L.rwkv_v4_forward_seq if self.version == 4 else L.rwkv_v56_forward
+        rc = fn(ctypes.byref(self._model), self._state_desc(state), tok.data_ptr(), T,
+                int(full_output), logits.data_ptr(), self._seq_ws.data_ptr(),
+                self._seq_ws.numel(), torch.cuda.current_stream().cuda_stream)
+        _lib.check(rc, "forward (sequence mode)")
         return logits, state
 
     def forward(self, tokens, state, full_output=False):

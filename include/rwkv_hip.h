@@ -195,6 +195,53 @@ int rwkv_v4_forward_seq(const rwkv_v4_model *m, const rwkv_v4_layer_state *state
                         int64_t T, int full_output, float *logits, void *workspace, size_t workspace_bytes,
                         void *stream);
 
+/* =======================================================================================
+ * RWKV-5.0 / 5.1 / 5.2 / 6.0: one entry point for both modes of RWKV.forward (T == 1 streams
+ * the matrices with the GEMV kernels, T > 1 uses the MFMA contraction).  Replaces att_one_v5 /
+ * att_one_v5_1 / att_one_v6_0, cuda_att_seq_v5_2 / cuda_att_seq_v6_0 with v5_2_before / v6_0_before
+ * / v5_2_after, RUN_RWKV_5 / RUN_RWKV_6 and ffn_one(_v6) / ffn_seq(_v6)
+ * (model.py:984-1029, 1091-1340, 1363-1439).  Head size must be 64.
+ */
+typedef struct {
+    const rwkv_half *ln1_w, *ln1_b, *ln2_w, *ln2_b;   /* [C] */
+    /* RWKV-5: time_mix_k, _v, _r, _g (g NULL for 5.0), two unused.
+     * RWKV-6: time_maa_x, _w, _k, _v, _r, _g. */
+    const rwkv_half *att_mix[6];
+    const rwkv_half *tm_w1;  /* v6: time_maa_w1 transposed, [5 * lora_maa][C] fp16 */
+    const rwkv_half *tm_w2;  /* v6: time_maa_w2 [5][lora_maa][C] fp16 */
+    const rwkv_half *td_w1;  /* v6: time_decay_w1 transposed, [lora_decay][C] fp16 */
+    const rwkv_half *td_w2;  /* v6: time_decay_w2 transposed, [C][lora_decay] fp16 */
+    const float *time_decay; /* [C] fp32: v5 exp(-exp(raw)) per channel; v6 raw (model.py:799-804) */
+    const float *time_first; /* [C] fp32 (model.py:808-814) */
+    const float *lnx_w, *lnx_b; /* [C] fp32 GroupNorm affine (model.py:815-816) */
+    rwkv_mat att_key, att_value, att_receptance, att_gate /* w NULL for 5.0 */, att_output;
+    const rwkv_half *ffn_mix_k, *ffn_mix_r;           /* time_mix_* (v5) / time_maa_* (v6) */
+    rwkv_mat ffn_key, ffn_receptance, ffn_value;
+} rwkv_v56_layer;
+
+typedef struct {
+    rwkv_half *att_xx;  /* [C] fp16 */
+    float *att_kv;      /* [H][N key][N value] fp32 (model.py:1470) */
+    rwkv_half *ffn_xx;  /* [C] fp16 */
+} rwkv_v56_layer_state;
+
+typedef struct {
+    int32_t version_x10;    /* 50, 51, 52 or 60 */
+    int32_t n_layer, n_embd, n_ffn, vocab, n_head;
+    int32_t lora_maa, lora_decay;   /* v6 LoRA ranks (32 / 64 in released models) */
+    int32_t rescale_layer, weights_u8;
+    const rwkv_half *emb, *ln_out_w, *ln_out_b;
+    rwkv_mat head;
+    const rwkv_v56_layer *layers;
+} rwkv_v56_model;
+
+size_t rwkv_v56_workspace(const rwkv_v56_model *m, int64_t T);
+/* tokens: device int32 [T]; logits fp32 [vocab] (last token) or [T, vocab] (full_output != 0 and
+ * T > 1).  All state tensors are updated in place.  Only launches kernels: capturable. */
+int rwkv_v56_forward(const rwkv_v56_model *m, const rwkv_v56_layer_state *states, const int32_t *tokens,
+                     int64_t T, int full_output, float *logits, void *workspace, size_t workspace_bytes,
+                     void *stream);
+
 #ifdef __cplusplus
 }
 #endif
