@@ -11,8 +11,9 @@ synchronisation; the same K steps are also timed with a host sync per token.
 One JSON line is printed:
   value / ms_per_step   decode tokens/s (device-token loop) and ms per token
   roofline              the dominant decode kernel (channel-mix receptance+key GEMV): algorithmic
-                        bytes per launch / mean launch duration from HIP events around every launch
-                        (rwkv_v4_profile_one), against the 8 TB/s HBM peak
+                        bytes per launch / mean launch duration, HIP events around 8 x n_layer
+                        back-to-back launches over all layers' weights (rwkv_v4_time_phase), against
+                        the 8 TB/s HBM peak
   decode_hbm            whole-step figure: uint8 weight bytes per token x tokens/s / 8 TB/s
   prefill               prefill tokens/s and the MFMA fraction of the whole prefill
   cpu_baseline          the oracle's 'cpu fp32i8' path (numpy port of the reference's CPU arithmetic)
@@ -29,6 +30,10 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK = 8.0e12      # bytes/s, MI355X HBM3E
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by a 1 GiB copy
+# kernel: x2.0 / x1.0); profiles/decode_7b_fp16i8_hbm_traffic.md has the commands and the table
+MEASURED_TRAFFIC = {("v4-7b", "cuda fp16i8", 32, "ffn_rk"): 84873421 + 49152,
+                    ("v4-7b", "cuda fp16i8", 32, "att_kvr_wkv"): 51738829 + 65536}
 MFMA_F16_PEAK = 2.5e15  # flop/s dense fp16
 
 
@@ -93,6 +98,9 @@ def main():
     ap.add_argument("--prefill", type=int, default=1024)
     ap.add_argument("--layers", type=int, default=None, help="debug: fewer layers (result is then not the headline)")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run five plain 1 GiB device copies (a kernel of known HBM traffic, for scaling "
+                         "rocprofv3 FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs on ONE GPU; the path has no multi-GPU mode (--gpus must be 1)",
@@ -153,23 +161,26 @@ def main():
     torch.cuda.synchronize()
     t_host = time.perf_counter() - t0
 
-    # ---- per-kernel durations from HIP events around every launch (not under graph replay)
-    per = []
-    for _ in range(8):
-        out, state, ms = model.profile_one(nxt, state)
-        nxt = int(out.argmax())
-        per.append(ms)
-    per = np.array(per[2:])  # drop two warm-up steps
-    names = ["att_kvr_wkv", "att_output", "ffn_rk", "ffn_value"]
+    # ---- per-kernel durations: each decode phase launched back to back over all layers (every
+    # layer streams its own weights, so nothing is served from cache) between two HIP events
+    torch.cuda.synchronize()
+    names = ["att_kvr_wkv", "att_output", "ffn_rk", "ffn_value", "head"]
     scale = 1 if u8 else 2
     kbytes = {"att_kvr_wkv": 3 * C * C * scale, "att_output": C * C * scale, "ffn_rk": (C * C + C * F) * scale,
               "ffn_value": C * F * scale, "head": C * V * scale}
-    kms = {n: float(per[:, j:4 * L:4].mean()) for j, n in enumerate(names)}
-    kms["head"] = float(per[:, -1].mean())
+    kms = {n: model.time_phase(j, reps=(8 if n != "head" else 64)) for j, n in enumerate(names)}
     ktot = {n: kms[n] * (L if n != "head" else 1) for n in kms}
     dom = max(ktot, key=ktot.get)
     kernels = {n: {"ms": round(kms[n], 5), "bytes": kbytes[n], "GBps": round(kbytes[n] / (kms[n] * 1e-3) / 1e9, 1)}
                for n in kms}
+
+    if args.calibrate_copy:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     tok_s = args.steps / t_dev
     res = {
@@ -186,7 +197,8 @@ def main():
             "bound": "hbm", "kernel": {"att_kvr_wkv": "att_kernel", "att_output": "vec_kernel", "ffn_rk": "lnmix_kernel",
                                         "ffn_value": "vec_kernel", "head": "lnmix_kernel"}[dom] + f" ({dom})",
             "achieved": kbytes[dom] / (kms[dom] * 1e-3) / 1e9, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
-            "frac": kbytes[dom] / (kms[dom] * 1e-3) / HBM_PEAK, "traffic": None,
+            "frac": kbytes[dom] / (kms[dom] * 1e-3) / HBM_PEAK,
+            "traffic": MEASURED_TRAFFIC.get((args.shape, args.strategy, L, dom)),
             "bytes_per_launch": kbytes[dom], "ms_per_launch": kms[dom],
         },
         "decode_hbm": {"weight_bytes_per_token": wbytes, "achieved_GBps": wbytes * tok_s / 1e9,

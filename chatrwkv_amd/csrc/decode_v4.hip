@@ -103,8 +103,11 @@ int v4_head_launch(const rwkv_v4_model *m, const rwkv_half *x, float *logits, hi
 
 // `ev` (optional): 4 * n_layer + 2 events; ev[0] is recorded before the first launch and
 // ev[i + 1] after the i-th launch.
+// `only_phase` (measurement): -1 runs the step; 0..3 launches only that phase of every layer, 4 only
+// the head (results are then meaningless; callers pass scratch state).
 static int v4_one_impl(const rwkv_v4_model *m, const rwkv_v4_layer_state *states, const int32_t *token,
-                       float *logits, void *workspace, size_t workspace_bytes, void *stream, hipEvent_t *ev) {
+                       float *logits, void *workspace, size_t workspace_bytes, void *stream, hipEvent_t *ev,
+                       int only_phase = -1) {
     int rc = v4_model_check(m);
     if (rc) return rc;
     if (!states || !token || !logits || !workspace) return RWKV_E_NULL;
@@ -135,7 +138,7 @@ static int v4_one_impl(const rwkv_v4_model *m, const rwkv_v4_layer_state *states
         const rwkv_v4_layer &l = m->layers[i];
         const rwkv_v4_layer_state &s = states[i];
         const int32_t *tok = (i == 0) ? token : nullptr;
-        {
+        if (only_phase < 0 || only_phase == 0) {
             AttArgs a{};
             a.x = ws.x; a.emb = m->emb; a.token = tok; a.C = C;
             a.ln_w = l.ln1_w; a.ln_b = l.ln1_b; a.sx = s.att_xx; a.xx_tmp = ws.xx_att;
@@ -148,7 +151,7 @@ static int v4_one_impl(const rwkv_v4_model *m, const rwkv_v4_layer_state *states
             else hipLaunchKernelGGL((att_kernel<false, 1>), dim3(grid), dim3(DTHREADS), lds, st, a);
             mark();
         }
-        {
+        if (only_phase < 0 || only_phase == 1) {
             VecArgs a{};
             a.vin = ws.rwkv; a.N = C; a.M = C; a.mat = to_dev(l.att_output);
             a.x_in = ws.x; a.emb = m->emb; a.token = tok; a.C = C; a.gate = nullptr; a.x_out = ws.x;
@@ -158,7 +161,7 @@ static int v4_one_impl(const rwkv_v4_model *m, const rwkv_v4_layer_state *states
             else hipLaunchKernelGGL((vec_kernel<false, 4>), dim3(grid), dim3(DTHREADS), lds, st, a);
             mark();
         }
-        {
+        if (only_phase < 0 || only_phase == 2) {
             LnMixArgs a{};
             a.x = ws.x; a.C = C; a.ln_w = l.ln2_w; a.ln_b = l.ln2_b; a.sx = s.ffn_xx; a.xx_tmp = ws.xx_ffn;
             a.mix[0] = l.ffn_mix_r; a.mat[0] = to_dev(l.ffn_receptance); a.M[0] = C; a.epi[0] = EPI_SIGMOID;
@@ -179,7 +182,7 @@ static int v4_one_impl(const rwkv_v4_model *m, const rwkv_v4_layer_state *states
             }
             mark();
         }
-        {
+        if (only_phase < 0 || only_phase == 3) {
             VecArgs a{};
             a.vin = ws.vx; a.N = F; a.M = C; a.mat = to_dev(l.ffn_value);
             a.x_in = ws.x; a.emb = nullptr; a.token = nullptr; a.C = C; a.gate = ws.r_ffn; a.x_out = ws.x;
@@ -192,7 +195,7 @@ static int v4_one_impl(const rwkv_v4_model *m, const rwkv_v4_layer_state *states
         }
         RWKV_LAUNCH_CHECK();
     }
-    rc = v4_head_launch(m, ws.x, logits, st);
+    if (only_phase < 0 || only_phase == 4) rc = v4_head_launch(m, ws.x, logits, st);
     mark();
     return rc;
 }
@@ -221,5 +224,32 @@ extern "C" int rwkv_v4_profile_one(const rwkv_v4_model *m, const rwkv_v4_layer_s
     }
     for (int i = 0; i < made; ++i) (void)hipEventDestroy(ev[i]);
     delete[] ev;
+    return rc;
+}
+
+extern "C" int rwkv_v4_time_phase(const rwkv_v4_model *m, const rwkv_v4_layer_state *states, const int32_t *token,
+                                  float *logits, void *workspace, size_t workspace_bytes, void *stream, int phase,
+                                  int reps, float *ms_per_launch) {
+    if (!m || !ms_per_launch) return RWKV_E_NULL;
+    if (phase < 0 || phase > 4 || reps <= 0) return RWKV_E_SHAPE;
+    hipEvent_t e0, e1;
+    if (hipEventCreate(&e0) != hipSuccess) return (int)hipErrorOutOfMemory;
+    if (hipEventCreate(&e1) != hipSuccess) { (void)hipEventDestroy(e0); return (int)hipErrorOutOfMemory; }
+    hipStream_t st = (hipStream_t)stream;
+    int rc = v4_one_impl(m, states, token, logits, workspace, workspace_bytes, stream, nullptr, phase);  // warm-up
+    if (rc == RWKV_OK) {
+        (void)hipEventRecord(e0, st);
+        for (int r = 0; r < reps && rc == RWKV_OK; ++r)
+            rc = v4_one_impl(m, states, token, logits, workspace, workspace_bytes, stream, nullptr, phase);
+        (void)hipEventRecord(e1, st);
+        hipError_t e = hipEventSynchronize(e1);
+        float ms = 0.f;
+        if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
+        if (e != hipSuccess && rc == RWKV_OK) rc = (int)e;
+        const int launches = reps * (phase == 4 ? 1 : m->n_layer);
+        *ms_per_launch = ms / launches;
+    }
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
     return rc;
 }

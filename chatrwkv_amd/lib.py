@@ -94,6 +94,7 @@ SIGNATURES.update({
     "rwkv_v4_one_workspace": (_sz, [ctypes.POINTER(RwkvV4Model)]),
     "rwkv_v4_forward_one": (_int, [ctypes.POINTER(RwkvV4Model), ctypes.POINTER(RwkvV4LayerState), _vp, _vp, _vp, _sz, _vp]),
     "rwkv_v4_profile_one": (_int, [ctypes.POINTER(RwkvV4Model), ctypes.POINTER(RwkvV4LayerState), _vp, _vp, _vp, _sz, _vp, _vp, _i64]),
+    "rwkv_v4_time_phase": (_int, [ctypes.POINTER(RwkvV4Model), ctypes.POINTER(RwkvV4LayerState), _vp, _vp, _vp, _sz, _vp, _int, _int, _vp]),
     "rwkv_v4_seq_workspace": (_sz, [ctypes.POINTER(RwkvV4Model), _i64, _int]),
     "rwkv_v4_forward_seq": (_int, [ctypes.POINTER(RwkvV4Model), ctypes.POINTER(RwkvV4LayerState), _vp, _i64, _int, _vp, _vp, _sz, _vp]),
 })

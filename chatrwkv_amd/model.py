@@ -484,6 +484,20 @@ class RWKV:
             _lib.check(rc, "rwkv_v4_profile_one")
             return self._logits.clone(), state, list(ms)
 
+    def time_phase(self, phase, reps=4):
+        """Mean duration (ms) of one launch of decode phase 0..4 run back to back over all layers
+        (rwkv_v4_time_phase), on a scratch state."""
+        scratch = self._new_state()
+        ms = ctypes.c_float(0)
+        self._token_dev.fill_(0)
+        logits = torch.empty_like(self._logits)
+        rc = _lib.load().rwkv_v4_time_phase(ctypes.byref(self._model), self._state_desc(scratch),
+                                            self._token_dev.data_ptr(), logits.data_ptr(), self._one_ws.data_ptr(),
+                                            self._one_ws.numel(), torch.cuda.current_stream().cuda_stream,
+                                            int(phase), int(reps), ctypes.byref(ms))
+        _lib.check(rc, "rwkv_v4_time_phase")
+        return float(ms.value)
+
     def _forward_seq(self, tokens, state, full_output):
         L = _lib.load()
         T = len(tokens)

@@ -1,0 +1,43 @@
+"""Strategy planner against the plans the reference prints (tests/golden/planner.json)."""
+import json
+import os
+
+import pytest
+
+from chatrwkv_amd import strategy
+
+G = os.path.join(os.path.dirname(__file__), "golden")
+
+
+def _fmt(slots):
+    return " ".join(
+        f"{n}-{s.device}-{str(s.atype).replace('torch.', '')}-{str(s.wtype).replace('torch.', '')}"
+        f"{'-stream' if s.stream else ''}" for n, s in enumerate(slots))
+
+
+def test_plans_match_reference():
+    gold = json.load(open(os.path.join(G, "planner.json")))
+    assert len(gold["plans"]) >= 15
+    for strat, line in gold["plans"].items():
+        assert line != "ERROR", strat
+        assert _fmt(strategy.plan(strat, gold["n_layer"])) == line, strat
+
+
+@pytest.mark.parametrize("bad", ["", "gpu fp16", "cuda fp8", "cuda fp16i8 ->", "cuda  fp16", "cuda fp16 * 3", "fp16 cuda"])
+def test_invalid_strategy_raises_value_error(bad):
+    with pytest.raises(ValueError):
+        strategy.plan(bad, 4)
+
+
+def test_only_single_gpu_plans_are_accepted():
+    assert strategy.require_single_gpu(strategy.plan("cuda fp16i8", 4)) == "u8"
+    assert strategy.require_single_gpu(strategy.plan("cuda:0 fp16", 4)) == "f16"
+    assert strategy.require_single_gpu(strategy.plan("cuda fp16i8 *100", 4)) == "u8"
+    for s in ("cpu fp32", "cpu fp32i8", "cuda fp32", "cuda bf16", "cuda fp16i8 -> cpu fp32 *1", "cuda fp16 *2+",
+              "cuda fp16 -> cuda:1 fp16", "cuda:1 fp16", "cuda fp16i8 *1 -> cuda fp16"):
+        with pytest.raises(NotImplementedError):
+            strategy.require_single_gpu(strategy.plan(s, 4))
+
+
+def test_normalize_spelling():
+    assert strategy.normalize("cuda fp16i8 *2->cpu fp32") == "cuda fp16i8 *2 -> cpu fp32"
