@@ -17,7 +17,7 @@ namespace {
 constexpr int DTHREADS = 1024;
 constexpr int DWAVES = DTHREADS / 64;
 constexpr float LN_EPS = 1e-5f;
-constexpr int VP = 4;  // 8-element groups per thread the vector prologue keeps in registers (N <= 32768)
+constexpr int VP = 4;  // most 8-element groups per thread the vector prologue keeps in registers (N <= 32768)
 
 // x for this step: the embedding row of the token (first layer) or the running activation.
 DEV const rwkv_half *resolve_x(const rwkv_half *x, const rwkv_half *emb, const int32_t *token, int C) {
@@ -59,18 +59,24 @@ struct LnMixPro {
     h16x8 x, lw, lb, sx, mix[NJ], ry[NJ], my[NJ];
     bool own;
 
+    // Absent operands are replaced by a valid pointer so that the loads of an owning thread are a
+    // straight line; threads that own no elements load nothing and their (masked) arithmetic in
+    // compute() runs on don't-care registers.
     DEV void load(const rwkv_half *xp, int C, const rwkv_half *ln_w, const rwkv_half *ln_b, const rwkv_half *sxp,
                   const rwkv_half *const (&mixp)[NJ], const MatDev (&mat)[NJ]) {
+        own = (int)threadIdx.x < (C >> 3);
         const int j8 = threadIdx.x;
-        own = j8 < (C >> 3);
+        x = lw = lb = sx = h16x8{};
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) mix[j] = ry[j] = my[j] = h16x8{};
         if (!own) return;
         x = *(const h16x8 *)(xp + 8 * j8);
         lw = *(const h16x8 *)(ln_w + 8 * j8);
         lb = *(const h16x8 *)(ln_b + 8 * j8);
-        if (sxp) sx = *(const h16x8 *)(sxp + 8 * j8);
+        sx = *(const h16x8 *)((sxp ? sxp : ln_w) + 8 * j8);
 #pragma unroll
         for (int j = 0; j < NJ; ++j) {
-            if (mixp[j]) mix[j] = *(const h16x8 *)(mixp[j] + 8 * j8);
+            mix[j] = *(const h16x8 *)((mixp[j] ? mixp[j] : ln_w) + 8 * j8);
             if (U8) {
                 ry[j] = *(const h16x8 *)(mat[j].ry + 8 * j8);
                 my[j] = *(const h16x8 *)(mat[j].my + 8 * j8);
@@ -82,14 +88,17 @@ struct LnMixPro {
     // maa_form: the RWKV-6 mixing kx = xx + (prev - xx) * m instead of kx = xx * m + prev * (1 - m)
     DEV void compute(int C, bool has_sx, const rwkv_half *const (&mixp)[NJ], h16 *const (&xs)[NJ], VecSums (&S)[NJ],
                      rwkv_half *xx_out, float *red, bool maa_form = false) {
+        // all threads run the arithmetic (threads that own no elements hold a copy of the last group and
+        // are masked out of the sums and the LDS writes): the waits on the operand loads then sit on
+        // every path, and nothing stays formally outstanding into the streaming loop
         float m[2] = {0.f, 0.f};
-        if (own)
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const float f = (float)x[e];
-                m[0] += f;
-                m[1] += f * f;
-            }
+        for (int e = 0; e < 8; ++e) {
+            const float f = (float)x[e];
+            m[0] += f;
+            m[1] += f * f;
+        }
+        if (!own) { m[0] = 0.f; m[1] = 0.f; }
         block_sum_1b<2>(m, red);
         const float mean = m[0] / C;
         const float rstd = rsqrtf(fmaxf(m[1] / C - mean * mean, 0.f) + LN_EPS);
@@ -97,37 +106,38 @@ struct LnMixPro {
         float acc[3 * NJ];
 #pragma unroll
         for (int i = 0; i < 3 * NJ; ++i) acc[i] = 0.f;
-        if (own) {
-            h16x8 xx;
+        h16x8 xx;
 #pragma unroll
-            for (int e = 0; e < 8; ++e) xx[e] = (h16)(((float)x[e] - mean) * rstd * (float)lw[e] + (float)lb[e]);
-            if (xx_out && blockIdx.x == 0) *(h16x8 *)(xx_out + 8 * j8) = xx;
-            const h16x8 pv = has_sx ? sx : xx;
+        for (int e = 0; e < 8; ++e) xx[e] = (h16)(((float)x[e] - mean) * rstd * (float)lw[e] + (float)lb[e]);
+        if (own && xx_out && blockIdx.x == 0) *(h16x8 *)(xx_out + 8 * j8) = xx;
+        const h16x8 pv = has_sx ? sx : xx;
 #pragma unroll
-            for (int j = 0; j < NJ; ++j) {
-                h16x8 kx = xx;
-                if (mixp[j]) {
+        for (int j = 0; j < NJ; ++j) {
+            h16x8 kx = xx;
+            if (mixp[j]) {
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) {
-                        const float mm = (float)mix[j][e];
-                        kx[e] = maa_form ? (h16)((float)xx[e] + (float)(h16)((float)pv[e] - (float)xx[e]) * mm)
-                                         : (h16)((float)xx[e] * mm + (float)pv[e] * (1.f - mm));
-                    }
+                for (int e = 0; e < 8; ++e) {
+                    const float mm = (float)mix[j][e];
+                    kx[e] = maa_form ? (h16)((float)xx[e] + (float)(h16)((float)pv[e] - (float)xx[e]) * mm)
+                                     : (h16)((float)xx[e] * mm + (float)pv[e] * (1.f - mm));
                 }
-                h16x8 o = kx;
-                if (U8) {
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) {
-                        const float k = (float)kx[e];
-                        o[e] = (h16)(k * (float)ry[j][e]);
-                        acc[3 * j] += k;
-                        acc[3 * j + 1] += (float)o[e];
-                        acc[3 * j + 2] += k * (float)my[j][e];
-                    }
-                }
-                ((h16x8 *)xs[j])[xs_item<U8>(j8, nseg)] = o;
             }
+            h16x8 o = kx;
+            if (U8) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const float k = (float)kx[e];
+                    o[e] = (h16)(k * (float)ry[j][e]);
+                    acc[3 * j] += k;
+                    acc[3 * j + 1] += (float)o[e];
+                    acc[3 * j + 2] += k * (float)my[j][e];
+                }
+            }
+            if (own) ((h16x8 *)xs[j])[xs_item<U8>(j8, nseg)] = o;
         }
+        if (!own)
+#pragma unroll
+            for (int i = 0; i < 3 * NJ; ++i) acc[i] = 0.f;
         // one barrier publishes both the LDS activation vectors and the partial sums
         block_sum_1b<3 * NJ>(acc, red + 2 * DWAVES);
         if (U8)
@@ -135,6 +145,9 @@ struct LnMixPro {
             for (int j = 0; j < NJ; ++j) { S[j].s0 = acc[3 * j]; S[j].s1 = acc[3 * j + 1]; S[j].s2 = acc[3 * j + 2]; }
     }
 };
+
+// wave-uniform: does this wave hold any of the `groups` 8-element groups that threads 0..groups-1 own?
+DEV bool pro_owner_wave(int groups) { return __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)) * 64 < groups; }
 
 template <bool U8>
 DEV const uint8_t *row_ptr(const MatDev &m, int64_t row) {
@@ -151,52 +164,65 @@ DEV float finish(float dot, const VecSums &S, float rx, float mx) {
 // otherwise).  Every wave owns a contiguous range of groups and walks it as a flat sequence of
 // batches (G groups x U segments per lane), ping-ponging between two register tiles: the loads
 // of batch q+1 are in flight while batch q is multiplied.
+//   pro_wave:             wave-uniform: this wave's threads hold prologue operands
 //   pro_load():           issue the loads of the prologue operands (called first)
 //   pro_compute():        build the LDS activation vectors (contains the workgroup barriers)
 //   rowf(g, k, row, xs):  weight row pointer and LDS activation vector of row k of group g
-//   epi_load(g) -> E:     loads of the operands the epilogue of group g needs (no dependence on
-//                         the dot products: issued together with the group's first weight tile)
+//   epi_load(g) -> E:     loads of the operands the epilogue of group g needs, as loaded (no
+//                         arithmetic on them: that would wait for the loads where they are issued)
 //   epi(g, dots, E):      called by one lane per group with the K reduced dot products
+//
+// The hardware counts outstanding loads per wave and the compiler places its waits from a static
+// count of the loads issued after the one it needs; where control flow merges it must assume the
+// path with the fewest.  A load under a branch that sits between a tile's loads and its use
+// therefore turns "wait for this tile" into "wait for everything", and the ping-pong degenerates
+// into load - wait - compute.  So every load from the first tile on is issued unconditionally
+// (clamped indices instead of predicates; a batch past the end of a wave's work is a load of one
+// cache line that is dropped), and the loop body is a straight line of load(next) / process(current)
+// pairs with one load site per tile inside the loop.
+//
+// Epilogue operands travel with the tile buffers: the operands of a group batch are loaded into
+// the slot of the tile that carries its second segment batch (its only one when there is one
+// per group batch), and read back when its last segment batch has been reduced.
 template <bool U8, int G, int K, int U, class E, class ProLoad, class ProCompute, class RowFn, class EpiLoad, class EpiFn>
-DEV void stream_rows(int ngroups, int nseg, ProLoad pro_load, ProCompute pro_compute, RowFn rowf, EpiLoad epi_load,
-                     EpiFn epi) {
+DEV void stream_rows(int ngroups, int nseg, bool pro_wave, ProLoad pro_load, ProCompute pro_compute, RowFn rowf,
+                     EpiLoad epi_load, EpiFn epi) {
     constexpr int R = G * K;
     const int lane = threadIdx.x & 63;
-    const int wave = blockIdx.x * DWAVES + (threadIdx.x >> 6), nwaves = gridDim.x * DWAVES;
+    // the wave index through readfirstlane: the compiler then knows that everything derived from it (row
+    // ranges, batch counters, loop control) is wave-uniform and keeps it in scalar registers
+    const int wave = blockIdx.x * DWAVES + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), nwaves = gridDim.x * DWAVES;
     const int per = (ngroups + nwaves - 1) / nwaves;
     const int g0 = min(wave * per, ngroups), g1 = min(g0 + per, ngroups);
+    const int glast = max(g1 - 1, 0);
     const int nsb = (nseg + 64 * U - 1) / (64 * U);             // segment batches per group batch
     const int nb = ((g1 - g0 + G - 1) / G) * nsb;               // batches of this wave
+    const int sb_epi = nsb > 1 ? 1 : 0;                         // segment batch that carries the epilogue operands
     RowTile<U8, R, U> t0, t1;
     E e0{}, e1{};
-    // epilogue operands live in slot (group batch index & 1): they are loaded with the first
-    // tile of a group batch and used after its last one, by when at most the next group batch
-    // has started loading
-    auto load = [&](RowTile<U8, R, U> &t, int q) {
-        const int gbi = q / nsb, gb = g0 + gbi * G, sb = q % nsb;
+    auto load = [&](RowTile<U8, R, U> &t, E &e, int q) {
+        const bool real = q < nb;
+        const int gbi = q / nsb, gb = g0 + gbi * G, sb = q - gbi * nsb;
         const uint8_t *rows[R];
         const h16 *xs_unused;
 #pragma unroll
         for (int i = 0; i < G; ++i)
 #pragma unroll
-            for (int k = 0; k < K; ++k) rowf(min(gb + i, g1 - 1), k, rows[i * K + k], xs_unused);
-        if (sb == 0 && lane < G && gb + lane < g1) {
-            const E e = epi_load(gb + lane);
-            if (gbi & 1) e1 = e; else e0 = e;
-        }
-        t.load(rows, sb * 64 * U, nseg);
+            for (int k = 0; k < K; ++k) rowf(min(gb + i, glast), k, rows[i * K + k], xs_unused);
+        if (real && sb == sb_epi) e = epi_load(min(gb + min(lane, G - 1), glast));
+        t.load(rows, sb * 64 * U, nseg, real);
     };
     float acc[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) acc[r] = 0.f;
     auto process = [&](const RowTile<U8, R, U> &t, int q) {
-        const int gbi = q / nsb, sb = q % nsb, gb = g0 + gbi * G;
+        const int gbi = q / nsb, sb = q - gbi * nsb, gb = g0 + gbi * G;
         const uint8_t *row_unused;
         const h16 *xs[R];
 #pragma unroll
         for (int i = 0; i < G; ++i)
 #pragma unroll
-            for (int k = 0; k < K; ++k) rowf(min(gb + i, g1 - 1), k, row_unused, xs[i * K + k]);
+            for (int k = 0; k < K; ++k) rowf(min(gb + i, glast), k, row_unused, xs[i * K + k]);
         t.consume(xs, sb * 64 * U, nseg, acc);
         if (sb == nsb - 1) {
 #pragma unroll
@@ -209,22 +235,30 @@ DEV void stream_rows(int ngroups, int nseg, ProLoad pro_load, ProCompute pro_com
 #pragma unroll
                     for (int i = 1; i < G; ++i) d[k] = (lane == i) ? acc[i * K + k] : d[k];
                 }
-                epi(gb + lane, d, (gbi & 1) ? e1 : e0);
+                epi(gb + lane, d, ((q - (nsb - 1) + sb_epi) & 1) ? e1 : e0);
             }
 #pragma unroll
             for (int r = 0; r < R; ++r) acc[r] = 0.f;
         }
     };
     pro_load();
-    if (nb > 0) load(t0, 0);
+    // The vector memory path of a CU returns data in request order across its waves: a prologue operand
+    // (an L2 hit) requested after another wave's weight tile (HBM) comes back after that tile.  The barrier
+    // puts the prologue requests of all 16 waves in front of every tile request, so the prologue can run
+    // while the first tiles are in flight instead of after them.
+    __builtin_amdgcn_s_barrier();
+    // Waves whose threads hold prologue operands start the prologue at once and fetch their first tile after
+    // it: issuing a tile blocks while the CU's request queue is full, and the prologue's workgroup barriers
+    // would wait for that.  The other waves have nothing to do in the prologue but to pass its barriers, and
+    // their first tiles keep HBM busy meanwhile.
+    if (!pro_wave) load(t0, e0, 0);
     pro_compute();
+    if (pro_wave) load(t0, e0, 0);
     for (int q = 0; q < nb; q += 2) {
-        if (q + 1 < nb) load(t1, q + 1);
+        load(t1, e1, q + 1);
         process(t0, q);
-        if (q + 1 < nb) {
-            if (q + 2 < nb) load(t0, q + 2);
-            process(t1, q + 1);
-        }
+        load(t0, e0, q + 2);
+        if (q + 1 < nb) process(t1, q + 1);
     }
 }
 
@@ -243,7 +277,8 @@ struct AttArgs {
 };
 
 struct AttEpi {
-    float rx[3], mx[3], u, w, aa, bb, pp;
+    rwkv_half rx[3], mx[3];  // as loaded; converted in the epilogue
+    float u, w, aa, bb, pp;
 };
 
 template <bool U8, int G>
@@ -263,20 +298,18 @@ __global__ __launch_bounds__(DTHREADS) void att_kernel(AttArgs a) {
         xv = xs[k];
     };
     auto epi_load = [&](int c) {
-        AttEpi e;
+        AttEpi e{};
+        if (U8)
 #pragma unroll
-        for (int k = 0; k < 3; ++k) {
-            e.rx[k] = U8 ? h2f(a.mat[k].rx[c]) : 1.f;
-            e.mx[k] = U8 ? h2f(a.mat[k].mx[c]) : 0.f;
-        }
+            for (int k = 0; k < 3; ++k) { e.rx[k] = a.mat[k].rx[c]; e.mx[k] = a.mat[k].mx[c]; }
         e.u = a.first[c]; e.w = a.decay[c];
         e.aa = a.aa[c]; e.bb = a.bb[c]; e.pp = a.pp[c];
         return e;
     };
     auto epi = [&](int c, const float (&d)[3], const AttEpi &e) {
-        float k = finish<U8>(d[0], S[0], e.rx[0], e.mx[0]);
-        float v = finish<U8>(d[1], S[1], e.rx[1], e.mx[1]);
-        float r = finish<U8>(d[2], S[2], e.rx[2], e.mx[2]);
+        float k = finish<U8>(d[0], S[0], h2f(e.rx[0]), h2f(e.mx[0]));
+        float v = finish<U8>(d[1], S[1], h2f(e.rx[1]), h2f(e.mx[1]));
+        float r = finish<U8>(d[2], S[2], h2f(e.rx[2]), h2f(e.mx[2]));
         if (U8) { k = round_h(k); v = round_h(v); }  // uint8 path returns fp16, widened again
         r = round_h(sigmoidf_(round_h(r)));
         float ww = e.u + k;
@@ -292,7 +325,7 @@ __global__ __launch_bounds__(DTHREADS) void att_kernel(AttArgs a) {
         a.pp[c] = p;
         a.rwkv[c] = f2h(r * round_h(wkv));
     };
-    stream_rows<U8, G, 3, 2, AttEpi>(C, (C * (U8 ? 1 : 2)) >> 4, pro_load, pro_compute, rowf, epi_load, epi);
+    stream_rows<U8, G, 3, 2, AttEpi>(C, (C * (U8 ? 1 : 2)) >> 4, pro_owner_wave(C >> 3), pro_load, pro_compute, rowf, epi_load, epi);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -312,7 +345,7 @@ struct LnMixArgs {
 };
 
 struct ScaleEpi {
-    float rx, mx;
+    rwkv_half rx, mx;  // as loaded
 };
 
 template <bool U8, int NJ, int G>
@@ -338,15 +371,14 @@ __global__ __launch_bounds__(DTHREADS) void lnmix_kernel(LnMixArgs a) {
     auto epi_load = [&](int g) {
         const int j = (NJ > 1 && g >= M0) ? 1 : 0;
         const int m = j ? g - M0 : g;
-        ScaleEpi e;
-        e.rx = U8 ? h2f(mat[j].rx[m]) : 1.f;
-        e.mx = U8 ? h2f(mat[j].mx[m]) : 0.f;
+        ScaleEpi e{};
+        if (U8) { e.rx = mat[j].rx[m]; e.mx = mat[j].mx[m]; }
         return e;
     };
     auto epi = [&](int g, const float (&d)[1], const ScaleEpi &e) {
         const int j = (NJ > 1 && g >= M0) ? 1 : 0;
         const int m = j ? g - M0 : g;
-        const float v = round_h(finish<U8>(d[0], S[j], e.rx, e.mx));
+        const float v = round_h(finish<U8>(d[0], S[j], h2f(e.rx), h2f(e.mx)));
         const int kind = a.epi[j];
         if (kind == EPI_LOGITS) {
             ((float *)a.out[j])[m] = v;
@@ -357,7 +389,8 @@ __global__ __launch_bounds__(DTHREADS) void lnmix_kernel(LnMixArgs a) {
             ((rwkv_half *)a.out[j])[m] = f2h(t * t);
         }
     };
-    stream_rows<U8, G, 1, (G >= 4 ? 1 : 2), ScaleEpi>(M0 + (NJ > 1 ? a.M[1] : 0), (C * (U8 ? 1 : 2)) >> 4, pro_load,
+    stream_rows<U8, G, 1, (G >= 4 ? 1 : 2), ScaleEpi>(M0 + (NJ > 1 ? a.M[1] : 0), (C * (U8 ? 1 : 2)) >> 4,
+                                                      pro_owner_wave(C >> 3), pro_load,
                                                       pro_compute, rowf, epi_load, epi);
 }
 
@@ -384,22 +417,24 @@ enum { VACT_RESIDUAL = 0, VACT_F16 = 1, VACT_SIGMOID = 2, VACT_RELU_SQ = 3, VACT
        VACT_LOGITS = 7 /* fp16-rounded value stored as fp32 */ };
 
 struct VecEpi {
-    float rx, mx, xin, gate;
+    rwkv_half rx, mx, xin, gate;  // as loaded
 };
 
-template <bool U8, int U>
+// The prologue is done by the first OW waves, VPN 8-element groups of the input vector per thread
+// (N <= 512 * OW * VPN); the other waves already stream weights meanwhile.
+template <bool U8, int U, int VPN, int OW>
 __global__ __launch_bounds__(DTHREADS) void vec_kernel(VecArgs a) {
     extern __shared__ __align__(16) unsigned char smem[];
     __shared__ float red[3 * DWAVES];
     const int N = a.N;
     h16 *xs = (h16 *)smem;
     VecSums S;
-    h16x8 pv[VP], pr[VP], pm[VP];
+    h16x8 pv[VPN], pr[VPN], pm[VPN];
     auto pro_load = [&]() {
 #pragma unroll
-        for (int i = 0; i < VP; ++i) {
-            const int j8 = threadIdx.x + i * DTHREADS;
-            if (j8 < (N >> 3)) {
+        for (int i = 0; i < VPN; ++i) {
+            const int j8 = threadIdx.x + i * 64 * OW;
+            if ((int)threadIdx.x < 64 * OW && j8 < (N >> 3)) {
                 pv[i] = *(const h16x8 *)(a.vin + 8 * j8);
                 if (U8) {
                     pr[i] = *(const h16x8 *)(a.mat.ry + 8 * j8);
@@ -409,15 +444,12 @@ __global__ __launch_bounds__(DTHREADS) void vec_kernel(VecArgs a) {
         }
     };
     auto pro_compute = [&]() {
-        if (blockIdx.x == 0 && a.commit_dst)
-            for (int j8 = threadIdx.x; j8 < (a.C >> 3); j8 += blockDim.x)
-                *(u32x4 *)(a.commit_dst + 8 * j8) = *(const u32x4 *)(a.commit_src + 8 * j8);
         const int nseg = N >> 4;
         float acc[3] = {0.f, 0.f, 0.f};
 #pragma unroll
-        for (int i = 0; i < VP; ++i) {
-            const int j8 = threadIdx.x + i * DTHREADS;
-            if (j8 < (N >> 3)) {
+        for (int i = 0; i < VPN; ++i) {
+            const int j8 = threadIdx.x + i * 64 * OW;
+            if ((int)threadIdx.x < 64 * OW && j8 < (N >> 3)) {
                 h16x8 o = pv[i];
                 if (U8) {
 #pragma unroll
@@ -440,22 +472,21 @@ __global__ __launch_bounds__(DTHREADS) void vec_kernel(VecArgs a) {
         xv = xs;
     };
     auto epi_load = [&](int m) {
-        VecEpi e;
-        e.rx = U8 ? h2f(a.mat.rx[m]) : 1.f;
-        e.mx = U8 ? h2f(a.mat.mx[m]) : 0.f;
-        e.xin = a.act == VACT_RESIDUAL ? h2f(resolve_x(a.x_in, a.emb, a.token, a.C)[m]) : 0.f;
-        e.gate = a.gate ? h2f(a.gate[m]) : 1.f;
+        VecEpi e{};
+        if (U8) { e.rx = a.mat.rx[m]; e.mx = a.mat.mx[m]; }
+        if (a.act == VACT_RESIDUAL) e.xin = resolve_x(a.x_in, a.emb, a.token, a.C)[m];
+        if (a.gate) e.gate = a.gate[m];
         return e;
     };
     auto epi = [&](int m, const float (&d)[1], const VecEpi &e) {
-        const float y = finish<U8>(d[0], S, e.rx, e.mx);
+        const float y = finish<U8>(d[0], S, h2f(e.rx), h2f(e.mx));
         if (a.act == VACT_F32) { ((float *)a.out)[m] = y; return; }
         float o = round_h(y);
         if (a.act == VACT_LOGITS) { ((float *)a.out)[m] = o; return; }
         switch (a.act) {
             case VACT_RESIDUAL:
-                if (a.gate) o = round_h(e.gate * o);
-                o = round_h(e.xin + o);
+                if (a.gate) o = round_h(h2f(e.gate) * o);
+                o = round_h(h2f(e.xin) + o);
                 a.x_out[m] = f2h(o * a.out_scale);
                 return;
             case VACT_SIGMOID: o = sigmoidf_(o); break;
@@ -466,7 +497,28 @@ __global__ __launch_bounds__(DTHREADS) void vec_kernel(VecArgs a) {
         }
         ((rwkv_half *)a.out)[m] = f2h(o);
     };
-    stream_rows<U8, 1, 1, U, VecEpi>(a.M, (N * (U8 ? 1 : 2)) >> 4, pro_load, pro_compute, rowf, epi_load, epi);
+    stream_rows<U8, 1, 1, U, VecEpi>(a.M, (N * (U8 ? 1 : 2)) >> 4, pro_owner_wave(min(N >> 3, 64 * OW)), pro_load, pro_compute, rowf, epi_load, epi);
+    // the token-shift state every workgroup of the previous launch read: committed after this workgroup's
+    // rows, so that the copy's load -> store dependency does not sit in front of the weight stream
+    if (blockIdx.x == 0 && a.commit_dst)
+        for (int j8 = threadIdx.x; j8 < (a.C >> 3); j8 += blockDim.x)
+            *(u32x4 *)(a.commit_dst + 8 * j8) = *(const u32x4 *)(a.commit_src + 8 * j8);
 }
+
+// Launches the vector GEMV with the tile depth and prologue shape that fit N (N <= 8192 * VP).
+#define RWKV_VEC_CASE(U, VPN, OW)                                                                              \
+    do {                                                                                                       \
+        if (u8) hipLaunchKernelGGL((vec_kernel<true, U, VPN, OW>), dim3(grid), dim3(DTHREADS), lds, st, a);    \
+        else hipLaunchKernelGGL((vec_kernel<false, U, VPN, OW>), dim3(grid), dim3(DTHREADS), lds, st, a);     \
+    } while (0)
+inline void vec_launch(bool u8, const VecArgs &a, int grid, hipStream_t st) {
+    const size_t lds = (size_t)a.N * 2;
+    const int groups = a.N >> 3;
+    if (groups <= 512) RWKV_VEC_CASE(4, 1, 8);
+    else if (groups <= 1024) RWKV_VEC_CASE(4, 2, 8);
+    else if (groups <= 2048) RWKV_VEC_CASE(8, 4, 8);
+    else RWKV_VEC_CASE(8, 4, 16);
+}
+#undef RWKV_VEC_CASE
 
 }  // namespace

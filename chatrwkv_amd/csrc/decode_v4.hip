@@ -156,9 +156,7 @@ static int v4_one_impl(const rwkv_v4_model *m, const rwkv_v4_layer_state *states
             a.vin = ws.rwkv; a.N = C; a.M = C; a.mat = to_dev(l.att_output);
             a.x_in = ws.x; a.emb = m->emb; a.token = tok; a.C = C; a.gate = nullptr; a.x_out = ws.x;
             a.out_scale = 1.f; a.commit_src = ws.xx_att; a.commit_dst = s.att_xx; a.act = VACT_RESIDUAL;
-            const size_t lds = (size_t)C * 2;
-            if (u8) hipLaunchKernelGGL((vec_kernel<true, 4>), dim3(grid), dim3(DTHREADS), lds, st, a);
-            else hipLaunchKernelGGL((vec_kernel<false, 4>), dim3(grid), dim3(DTHREADS), lds, st, a);
+            vec_launch(u8, a, grid, st);
             mark();
         }
         if (only_phase < 0 || only_phase == 2) {
@@ -188,9 +186,7 @@ static int v4_one_impl(const rwkv_v4_model *m, const rwkv_v4_layer_state *states
             a.x_in = ws.x; a.emb = nullptr; a.token = nullptr; a.C = C; a.gate = ws.r_ffn; a.x_out = ws.x;
             a.out_scale = (m->rescale_layer > 0 && (i + 1) % m->rescale_layer == 0) ? 0.5f : 1.f;
             a.commit_src = ws.xx_ffn; a.commit_dst = s.ffn_xx; a.act = VACT_RESIDUAL;
-            const size_t lds = (size_t)F * 2;
-            if (u8) hipLaunchKernelGGL((vec_kernel<true, 8>), dim3(grid), dim3(DTHREADS), lds, st, a);
-            else hipLaunchKernelGGL((vec_kernel<false, 8>), dim3(grid), dim3(DTHREADS), lds, st, a);
+            vec_launch(u8, a, grid, st);
             mark();
         }
         RWKV_LAUNCH_CHECK();

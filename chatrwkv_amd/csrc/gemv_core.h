@@ -149,17 +149,18 @@ template <bool U8, int R, int U>
 struct RowTile {
     u32x4 w[U][R];
 
-    DEV void load(const uint8_t *const (&rows)[R], int seg0, int nseg) {
+    // No load is predicated: a lane past the end of the row re-reads its last segment (consume() skips
+    // it), and with real == false (wave-uniform; a batch past the end of the wave's work) all lanes read
+    // the first segment of the row, one cache line, and the tile is never consumed.  A load under a
+    // branch would make the compiler's static s_waitcnt counting assume that it may not have been
+    // issued, and every wait on an earlier load would then drain this tile too.
+    DEV void load(const uint8_t *const (&rows)[R], int seg0, int nseg, bool real = true) {
         const int lane = threadIdx.x & 63;
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            const int s = seg0 + lane + 64 * u;
+            const int s = real ? min(seg0 + lane + 64 * u, nseg - 1) : 0;
 #pragma unroll
-            for (int r = 0; r < R; ++r) {
-                u32x4 v = {0u, 0u, 0u, 0u};
-                if (s < nseg) v = __builtin_nontemporal_load((const u32x4 *)(rows[r] + 16 * (size_t)s));
-                w[u][r] = v;
-            }
+            for (int r = 0; r < R; ++r) w[u][r] = __builtin_nontemporal_load((const u32x4 *)(rows[r] + 16 * (size_t)s));
         }
     }
 

@@ -127,15 +127,8 @@ int mm(const Ctx &c, const rwkv_mat &m, bool mat_u8, const rwkv_half *x, int act
             case ACT_TANH: a.act = VACT_TANH; break;
             default: a.act = VACT_RESIDUAL; break;
         }
-        const size_t lds = (size_t)N * 2;
         if (N > 8 * VP * DTHREADS) return RWKV_E_SHAPE;
-        if (mat_u8) {
-            if (N >= 8192) hipLaunchKernelGGL((vec_kernel<true, 8>), dim3(c.grid), dim3(DTHREADS), lds, c.st, a);
-            else hipLaunchKernelGGL((vec_kernel<true, 4>), dim3(c.grid), dim3(DTHREADS), lds, c.st, a);
-        } else {
-            if (N >= 8192) hipLaunchKernelGGL((vec_kernel<false, 8>), dim3(c.grid), dim3(DTHREADS), lds, c.st, a);
-            else hipLaunchKernelGGL((vec_kernel<false, 4>), dim3(c.grid), dim3(DTHREADS), lds, c.st, a);
-        }
+        vec_launch(mat_u8, a, c.grid, c.st);
         RWKV_LAUNCH_CHECK();
         return RWKV_OK;
     }
@@ -315,9 +308,7 @@ extern "C" int rwkv_v56_forward(const rwkv_v56_model *m, const rwkv_v56_layer_st
         VecArgs a{};
         a.vin = ws.xx; a.N = C; a.M = m->vocab; a.mat = to_dev56(m->head); a.act = VACT_LOGITS; a.out = logits;
         a.out_scale = 1.f;
-        const size_t lds = (size_t)C * 2;
-        if (u8) hipLaunchKernelGGL((vec_kernel<true, 4>), dim3(c.grid), dim3(DTHREADS), lds, st, a);
-        else hipLaunchKernelGGL((vec_kernel<false, 4>), dim3(c.grid), dim3(DTHREADS), lds, st, a);
+        vec_launch(u8, a, c.grid, st);
         RWKV_LAUNCH_CHECK();
         return RWKV_OK;
     }
