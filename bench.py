@@ -37,8 +37,11 @@ MEASURED_TRAFFIC = {("v4-7b", "cuda fp16i8", 32, "ffn_rk"): 84873421 + 49152,
 MFMA_F16_PEAK = 2.5e15  # flop/s dense fp16
 
 
-def u8_weight_bytes(L, C, F, V):
-    return L * (5 * C * C + 2 * C * F) + C * V
+def u8_weight_bytes(L, C, F, V, version=4):
+    """uint8 matrix bytes one decoded token streams: v4/v5 layers have 5 C x C matrices (v5.1+ a gate: 6),
+    v6 has 6; all have the two C x F channel-mix matrices; plus the head."""
+    per_layer = (5 if version < 5.1 else 6) * C * C + 2 * C * F
+    return L * per_layer + C * V
 
 
 def cpu_baseline(shape, budget_s=25.0):
@@ -96,6 +99,7 @@ def main():
     ap.add_argument("--shape", default="v4-7b")
     ap.add_argument("--strategy", default="cuda fp16i8")
     ap.add_argument("--prefill", type=int, default=1024)
+    ap.add_argument("--chunk", type=int, default=0, help="prefill in calls of this many tokens (0: one call)")
     ap.add_argument("--layers", type=int, default=None, help="debug: fewer layers (result is then not the headline)")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -122,17 +126,25 @@ def main():
     del ck
     torch.cuda.empty_cache()
     u8 = args.strategy.endswith("i8")
-    wbytes = u8_weight_bytes(L, C, F, V) * (1 if u8 else 2)
+    wbytes = u8_weight_bytes(L, C, F, V, version) * (1 if u8 else 2)
 
     # ---- prefill: one call over `prefill` tokens (median of 3, after one warm-up call)
     ptoks = synth.random_tokens(args.prefill, V, seed=2)
-    model.forward(ptoks, None)
+    chunk = args.chunk if args.chunk > 0 else args.prefill
+
+    def prefill():
+        out, state = None, None
+        for i in range(0, len(ptoks), chunk):
+            out, state = model.forward(ptoks[i:i + chunk], state)
+        return out, state
+
+    prefill()
     torch.cuda.synchronize()
     pt = []
     for _ in range(3):
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
-        out, state = model.forward(ptoks, None)
+        out, state = prefill()
         e1.record()
         torch.cuda.synchronize()
         pt.append(e0.elapsed_time(e1) * 1e-3)
@@ -164,15 +176,30 @@ def main():
     # ---- per-kernel durations: each decode phase launched back to back over all layers (every
     # layer streams its own weights, so nothing is served from cache) between two HIP events
     torch.cuda.synchronize()
-    names = ["att_kvr_wkv", "att_output", "ffn_rk", "ffn_value", "head"]
-    scale = 1 if u8 else 2
-    kbytes = {"att_kvr_wkv": 3 * C * C * scale, "att_output": C * C * scale, "ffn_rk": (C * C + C * F) * scale,
-              "ffn_value": C * F * scale, "head": C * V * scale}
-    kms = {n: model.time_phase(j, reps=(8 if n != "head" else 64)) for j, n in enumerate(names)}
-    ktot = {n: kms[n] * (L if n != "head" else 1) for n in kms}
-    dom = max(ktot, key=ktot.get)
-    kernels = {n: {"ms": round(kms[n], 5), "bytes": kbytes[n], "GBps": round(kbytes[n] / (kms[n] * 1e-3) / 1e9, 1)}
-               for n in kms}
+    tok_s = args.steps / t_dev
+    if version == 4:
+        names = ["att_kvr_wkv", "att_output", "ffn_rk", "ffn_value", "head"]
+        scale = 1 if u8 else 2
+        kbytes = {"att_kvr_wkv": 3 * C * C * scale, "att_output": C * C * scale, "ffn_rk": (C * C + C * F) * scale,
+                  "ffn_value": C * F * scale, "head": C * V * scale}
+        kms = {n: model.time_phase(j, reps=(8 if n != "head" else 64)) for j, n in enumerate(names)}
+        ktot = {n: kms[n] * (L if n != "head" else 1) for n in kms}
+        dom = max(ktot, key=ktot.get)
+        kernels = {n: {"ms": round(kms[n], 5), "bytes": kbytes[n], "GBps": round(kbytes[n] / (kms[n] * 1e-3) / 1e9, 1)}
+                   for n in kms}
+        kname = {"att_kvr_wkv": "att_kernel", "att_output": "vec_kernel", "ffn_rk": "lnmix_kernel",
+                 "ffn_value": "vec_kernel", "head": "lnmix_kernel"}[dom] + f" ({dom})"
+        roof = {"bound": "hbm", "kernel": kname, "achieved": kbytes[dom] / (kms[dom] * 1e-3) / 1e9,
+                "peak": HBM_PEAK / 1e9, "unit": "GB/s", "frac": kbytes[dom] / (kms[dom] * 1e-3) / HBM_PEAK,
+                "traffic": MEASURED_TRAFFIC.get((args.shape, args.strategy, L, dom)),
+                "bytes_per_launch": kbytes[dom], "ms_per_launch": kms[dom]}
+    else:
+        # RWKV-5/6 one-token steps are a chain of the same streaming GEMV launches with no per-phase timing
+        # entry; the roofline figure is then the whole step: uint8 matrix bytes per token over the step time
+        kernels = None
+        roof = {"bound": "hbm", "kernel": "whole one-token step (vec_kernel chain)", "achieved": wbytes * tok_s / 1e9,
+                "peak": HBM_PEAK / 1e9, "unit": "GB/s", "frac": wbytes * tok_s / HBM_PEAK, "traffic": None,
+                "bytes_per_launch": wbytes, "ms_per_launch": 1e3 / tok_s}
 
     if args.calibrate_copy:
         src = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
@@ -182,25 +209,18 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    tok_s = args.steps / t_dev
     res = {
-        "metric": "7B fp16i8 decode tok/s (% HBM peak) + prefill tok/s, 1 MI355X",
+        "metric": "7B fp16i8 decode tok/s (% HBM peak) + prefill tok/s, 1 MI355X" if args.shape == "v4-7b" and u8 else
+                  f"{args.shape} '{args.strategy}' decode tok/s (% HBM peak) + prefill tok/s, 1 MI355X",
         "value": tok_s, "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": 1e3 * t_dev / args.steps, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "u8 weights, fp16 activations, fp32 accumulate" if u8 else "fp16",
         "data": "synthetic (random-init weights, random tokens)",
         "config": {"workload": f"RWKV-4 {args.shape} ({L} layers, n_embd {C}, ffn {F}, vocab {V}) '{args.strategy}', "
-                               f"batch 1: prefill {args.prefill} tokens in one call, then greedy decode "
-                               f"(BASELINE.json configs[2])",
+                               f"batch 1: prefill {args.prefill} tokens in {'one call' if chunk >= args.prefill else f'calls of {chunk}'}, "
+                               f"then greedy decode" + (" (BASELINE.json configs[2])" if args.shape == "v4-7b" else ""),
                    "strategy": args.strategy, "prefill_tokens": args.prefill},
-        "roofline": {
-            "bound": "hbm", "kernel": {"att_kvr_wkv": "att_kernel", "att_output": "vec_kernel", "ffn_rk": "lnmix_kernel",
-                                        "ffn_value": "vec_kernel", "head": "lnmix_kernel"}[dom] + f" ({dom})",
-            "achieved": kbytes[dom] / (kms[dom] * 1e-3) / 1e9, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
-            "frac": kbytes[dom] / (kms[dom] * 1e-3) / HBM_PEAK,
-            "traffic": MEASURED_TRAFFIC.get((args.shape, args.strategy, L, dom)),
-            "bytes_per_launch": kbytes[dom], "ms_per_launch": kms[dom],
-        },
+        "roofline": roof,
         "decode_hbm": {"weight_bytes_per_token": wbytes, "achieved_GBps": wbytes * tok_s / 1e9,
                        "frac_of_peak": wbytes * tok_s / HBM_PEAK},
         "decode_tok_s_host_sync": args.steps / t_host,

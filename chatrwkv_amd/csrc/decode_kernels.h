@@ -52,6 +52,23 @@ DEV void block_sum_1b(float (&v)[K], float *red) {
     for (int k = 0; k < K; ++k) v[k] = row16_sum(red[k * DWAVES + (lane & 15)]);
 }
 
+// fp16 element-wise helpers, one rounding per operation (no contraction into fma): what the
+// reference's fp16 tensor expressions compute.  Compiled to packed fp16 instructions.
+#pragma clang fp contract(off)
+DEV h16x8 mul_h(h16x8 a, h16x8 b) { return a * b; }
+// xx * m + prev * (1 - m)
+DEV h16x8 mix_lerp(h16x8 xx, h16x8 prev, h16x8 m) {
+    const h16x8 one = {(h16)1.f, (h16)1.f, (h16)1.f, (h16)1.f, (h16)1.f, (h16)1.f, (h16)1.f, (h16)1.f};
+    const h16x8 a = xx * m, t = one - m, b = prev * t;
+    return a + b;
+}
+// xx + (prev - xx) * m
+DEV h16x8 mix_maa(h16x8 xx, h16x8 prev, h16x8 m) {
+    const h16x8 d = prev - xx, t = d * m;
+    return xx + t;
+}
+#pragma clang fp contract(fast)
+
 // LayerNorm + token-shift mixes for NJ consumers, operands staged in registers.
 // Requires C / 8 <= DTHREADS (C <= 8192): thread t owns elements [8t, 8t + 8).
 template <bool U8, int NJ>
@@ -88,17 +105,19 @@ struct LnMixPro {
     // maa_form: the RWKV-6 mixing kx = xx + (prev - xx) * m instead of kx = xx * m + prev * (1 - m)
     DEV void compute(int C, bool has_sx, const rwkv_half *const (&mixp)[NJ], h16 *const (&xs)[NJ], VecSums (&S)[NJ],
                      rwkv_half *xx_out, float *red, bool maa_form = false) {
-        // all threads run the arithmetic (threads that own no elements hold a copy of the last group and
-        // are masked out of the sums and the LDS writes): the waits on the operand loads then sit on
-        // every path, and nothing stays formally outstanding into the streaming loop
+        // All threads run the arithmetic (threads that own no elements work on zeros and are masked out
+        // of the LDS writes): the waits on the operand loads then sit on every path.  The prologue is
+        // bound by VALU issue (its ~10 operand vectors live in two waves per SIMD), so the element-wise
+        // chain uses packed fp16 instructions, which round after every operation exactly as the
+        // reference's fp16 tensor arithmetic does, and v_dot2_f32_f16 for the fp32 sums.
+        const h16x2 ones = {(h16)1.f, (h16)1.f};
         float m[2] = {0.f, 0.f};
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            const float f = (float)x[e];
-            m[0] += f;
-            m[1] += f * f;
+        for (int e = 0; e < 8; e += 2) {
+            const h16x2 xp = {x[e], x[e + 1]};
+            m[0] = __builtin_amdgcn_fdot2(xp, ones, m[0], false);
+            m[1] = __builtin_amdgcn_fdot2(xp, xp, m[1], false);
         }
-        if (!own) { m[0] = 0.f; m[1] = 0.f; }
         block_sum_1b<2>(m, red);
         const float mean = m[0] / C;
         const float rstd = rsqrtf(fmaxf(m[1] / C - mean * mean, 0.f) + LN_EPS);
@@ -114,30 +133,20 @@ struct LnMixPro {
 #pragma unroll
         for (int j = 0; j < NJ; ++j) {
             h16x8 kx = xx;
-            if (mixp[j]) {
-#pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    const float mm = (float)mix[j][e];
-                    kx[e] = maa_form ? (h16)((float)xx[e] + (float)(h16)((float)pv[e] - (float)xx[e]) * mm)
-                                     : (h16)((float)xx[e] * mm + (float)pv[e] * (1.f - mm));
-                }
-            }
+            if (mixp[j]) kx = maa_form ? mix_maa(xx, pv, mix[j]) : mix_lerp(xx, pv, mix[j]);
             h16x8 o = kx;
             if (U8) {
+                o = mul_h(kx, ry[j]);
 #pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    const float k = (float)kx[e];
-                    o[e] = (h16)(k * (float)ry[j][e]);
-                    acc[3 * j] += k;
-                    acc[3 * j + 1] += (float)o[e];
-                    acc[3 * j + 2] += k * (float)my[j][e];
+                for (int e = 0; e < 8; e += 2) {
+                    const h16x2 kp = {kx[e], kx[e + 1]}, op = {o[e], o[e + 1]}, mp = {my[j][e], my[j][e + 1]};
+                    acc[3 * j] = __builtin_amdgcn_fdot2(kp, ones, acc[3 * j], false);
+                    acc[3 * j + 1] = __builtin_amdgcn_fdot2(op, ones, acc[3 * j + 1], false);
+                    acc[3 * j + 2] = __builtin_amdgcn_fdot2(kp, mp, acc[3 * j + 2], false);
                 }
             }
             if (own) ((h16x8 *)xs[j])[xs_item<U8>(j8, nseg)] = o;
         }
-        if (!own)
-#pragma unroll
-            for (int i = 0; i < 3 * NJ; ++i) acc[i] = 0.f;
         // one barrier publishes both the LDS activation vectors and the partial sums
         block_sum_1b<3 * NJ>(acc, red + 2 * DWAVES);
         if (U8)
@@ -452,13 +461,14 @@ __global__ __launch_bounds__(DTHREADS) void vec_kernel(VecArgs a) {
             if ((int)threadIdx.x < 64 * OW && j8 < (N >> 3)) {
                 h16x8 o = pv[i];
                 if (U8) {
+                    const h16x2 ones = {(h16)1.f, (h16)1.f};
+                    o = mul_h(pv[i], pr[i]);
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) {
-                        const float k = (float)pv[i][e];
-                        o[e] = (h16)(k * (float)pr[i][e]);
-                        acc[0] += k;
-                        acc[1] += (float)o[e];
-                        acc[2] += k * (float)pm[i][e];
+                    for (int e = 0; e < 8; e += 2) {
+                        const h16x2 kp = {pv[i][e], pv[i][e + 1]}, op = {o[e], o[e + 1]}, mp = {pm[i][e], pm[i][e + 1]};
+                        acc[0] = __builtin_amdgcn_fdot2(kp, ones, acc[0], false);
+                        acc[1] = __builtin_amdgcn_fdot2(op, ones, acc[1], false);
+                        acc[2] = __builtin_amdgcn_fdot2(kp, mp, acc[2], false);
                     }
                 }
                 ((h16x8 *)xs)[xs_item<U8>(j8, nseg)] = o;
@@ -503,6 +513,144 @@ __global__ __launch_bounds__(DTHREADS) void vec_kernel(VecArgs a) {
     if (blockIdx.x == 0 && a.commit_dst)
         for (int j8 = threadIdx.x; j8 < (a.C >> 3); j8 += blockDim.x)
             *(u32x4 *)(a.commit_dst + 8 * j8) = *(const u32x4 *)(a.commit_src + 8 * j8);
+}
+
+// ------------------------------------------------------------------------------------------
+// Several GEMVs of the same shape [N -> M] in one launch, each with its own input vector
+// (RWKV-5/6 time mix: receptance, key, value and gate rows over the r/k/v/g mixes).
+struct MultiVecArgs {
+    int N, M, nm;                // nm matrices (<= 4)
+    const rwkv_half *vin[4];     // [N] fp16 each
+    MatDev mat[4];
+    int act[4];                  // VACT_F16 / VACT_SILU / VACT_SIGMOID ...
+    rwkv_half *out[4];           // [M] fp16 each
+    const rwkv_half *commit_src; // scratch xx -> token-shift state, done by workgroup 0
+    rwkv_half *commit_dst;
+    int commit_n;
+};
+
+// NM input vectors of N <= 4096 elements (one 8-element group per thread of the first 8 waves).
+template <bool U8, int NM>
+__global__ __launch_bounds__(DTHREADS) void multi_vec_kernel(MultiVecArgs a) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    __shared__ float red[3 * NM * DWAVES];
+    const int N = a.N, M = a.M;
+    h16 *xs[NM];
+#pragma unroll
+    for (int j = 0; j < NM; ++j) xs[j] = (h16 *)smem + (size_t)j * N;
+    VecSums S[NM];
+    h16x8 pv[NM], pr[NM], pm[NM];
+    const bool own = (int)threadIdx.x < (N >> 3);
+    auto pro_load = [&]() {
+#pragma unroll
+        for (int j = 0; j < NM; ++j) pv[j] = pr[j] = pm[j] = h16x8{};
+        if (!own) return;
+#pragma unroll
+        for (int j = 0; j < NM; ++j) {
+            pv[j] = *(const h16x8 *)(a.vin[j] + 8 * threadIdx.x);
+            if (U8) {
+                pr[j] = *(const h16x8 *)(a.mat[j].ry + 8 * threadIdx.x);
+                pm[j] = *(const h16x8 *)(a.mat[j].my + 8 * threadIdx.x);
+            }
+        }
+    };
+    auto pro_compute = [&]() {
+        const int nseg = N >> 4;
+        const h16x2 ones = {(h16)1.f, (h16)1.f};
+        float acc[3 * NM];
+#pragma unroll
+        for (int i = 0; i < 3 * NM; ++i) acc[i] = 0.f;
+#pragma unroll
+        for (int j = 0; j < NM; ++j) {
+            h16x8 o = pv[j];
+            if (U8) {
+                o = mul_h(pv[j], pr[j]);
+#pragma unroll
+                for (int e = 0; e < 8; e += 2) {
+                    const h16x2 kp = {pv[j][e], pv[j][e + 1]}, op = {o[e], o[e + 1]}, mp = {pm[j][e], pm[j][e + 1]};
+                    acc[3 * j] = __builtin_amdgcn_fdot2(kp, ones, acc[3 * j], false);
+                    acc[3 * j + 1] = __builtin_amdgcn_fdot2(op, ones, acc[3 * j + 1], false);
+                    acc[3 * j + 2] = __builtin_amdgcn_fdot2(kp, mp, acc[3 * j + 2], false);
+                }
+            }
+            if (own) ((h16x8 *)xs[j])[xs_item<U8>(threadIdx.x, nseg)] = o;
+        }
+        block_sum_1b<3 * NM>(acc, red);  // the barrier also publishes xs
+        if (U8)
+#pragma unroll
+            for (int j = 0; j < NM; ++j) { S[j].s0 = acc[3 * j]; S[j].s1 = acc[3 * j + 1]; S[j].s2 = acc[3 * j + 2]; }
+    };
+    // a group is one output index m with its NM rows (row m of every matrix), so the matrix number is a
+    // compile-time constant everywhere (an array of per-matrix fields indexed at run time would go to scratch)
+    struct Epi { rwkv_half rx[NM], mx[NM]; };
+    auto rowf = [&](int m, int k, const uint8_t *&row, const h16 *&xv) {
+        row = row_ptr<U8>(a.mat[k], m);
+        xv = xs[k];
+    };
+    auto epi_load = [&](int m) {
+        Epi e{};
+        if (U8)
+#pragma unroll
+            for (int k = 0; k < NM; ++k) { e.rx[k] = a.mat[k].rx[m]; e.mx[k] = a.mat[k].mx[m]; }
+        return e;
+    };
+    auto epi = [&](int m, const float (&d)[NM], const Epi &e) {
+#pragma unroll
+        for (int k = 0; k < NM; ++k) {
+            float o = round_h(finish<U8>(d[k], S[k], h2f(e.rx[k]), h2f(e.mx[k])));
+            switch (a.act[k]) {
+                case VACT_SIGMOID: o = sigmoidf_(o); break;
+                case VACT_RELU_SQ: o = fmaxf(o, 0.f); o = o * o; break;
+                case VACT_SILU: o = o * sigmoidf_(o); break;
+                case VACT_TANH: o = tanhf(o); break;
+                default: break;
+            }
+            a.out[k][m] = f2h(o);
+        }
+    };
+    stream_rows<U8, 1, NM, 2, Epi>(M, (N * (U8 ? 1 : 2)) >> 4, pro_owner_wave(N >> 3), pro_load, pro_compute, rowf, epi_load, epi);
+    if (blockIdx.x == 0 && a.commit_dst)
+        for (int j8 = threadIdx.x; j8 < (a.commit_n >> 3); j8 += blockDim.x)
+            *(u32x4 *)(a.commit_dst + 8 * j8) = *(const u32x4 *)(a.commit_src + 8 * j8);
+}
+
+inline void multi_vec_launch(bool u8, const MultiVecArgs &a, int grid, hipStream_t st) {
+    const size_t lds = (size_t)a.nm * a.N * 2;
+    if (a.nm == 4) {
+        if (u8) hipLaunchKernelGGL((multi_vec_kernel<true, 4>), dim3(grid), dim3(DTHREADS), lds, st, a);
+        else hipLaunchKernelGGL((multi_vec_kernel<false, 4>), dim3(grid), dim3(DTHREADS), lds, st, a);
+    } else {
+        if (u8) hipLaunchKernelGGL((multi_vec_kernel<true, 3>), dim3(grid), dim3(DTHREADS), lds, st, a);
+        else hipLaunchKernelGGL((multi_vec_kernel<false, 3>), dim3(grid), dim3(DTHREADS), lds, st, a);
+    }
+}
+
+// LN + token shift + two GEMVs (channel-mix receptance and key) in one launch; picks the tile depth that
+// divides a wave's share of the rows.
+inline void lnmix2_launch(bool u8, const LnMixArgs &a, int grid, hipStream_t st) {
+    const size_t lds = 2 * (size_t)a.C * 2;
+    const int per = (a.M[0] + a.M[1] + grid * DWAVES - 1) / (grid * DWAVES);
+    if (per % 5 == 0) {
+        if (u8) hipLaunchKernelGGL((lnmix_kernel<true, 2, 5>), dim3(grid), dim3(DTHREADS), lds, st, a);
+        else hipLaunchKernelGGL((lnmix_kernel<false, 2, 5>), dim3(grid), dim3(DTHREADS), lds, st, a);
+    } else if (per >= 4) {
+        if (u8) hipLaunchKernelGGL((lnmix_kernel<true, 2, 4>), dim3(grid), dim3(DTHREADS), lds, st, a);
+        else hipLaunchKernelGGL((lnmix_kernel<false, 2, 4>), dim3(grid), dim3(DTHREADS), lds, st, a);
+    } else {
+        if (u8) hipLaunchKernelGGL((lnmix_kernel<true, 2, 2>), dim3(grid), dim3(DTHREADS), lds, st, a);
+        else hipLaunchKernelGGL((lnmix_kernel<false, 2, 2>), dim3(grid), dim3(DTHREADS), lds, st, a);
+    }
+}
+
+// LN_out(x) @ head -> fp32 logits (fp16-rounded values) in one launch.
+inline void lnhead_launch(bool u8, const rwkv_half *x, int C, const rwkv_half *ln_w, const rwkv_half *ln_b,
+                          const MatDev &head, int vocab, float *logits, int grid, hipStream_t st) {
+    LnMixArgs h{};
+    h.x = x; h.C = C; h.ln_w = ln_w; h.ln_b = ln_b; h.sx = nullptr; h.xx_tmp = nullptr;
+    h.mix[0] = nullptr; h.mat[0] = head; h.M[0] = vocab; h.epi[0] = EPI_LOGITS; h.out[0] = logits;
+    const size_t lds = (size_t)C * 2;
+    if (u8) hipLaunchKernelGGL((lnmix_kernel<true, 1, 4>), dim3(grid), dim3(DTHREADS), lds, st, h);
+    else hipLaunchKernelGGL((lnmix_kernel<false, 1, 4>), dim3(grid), dim3(DTHREADS), lds, st, h);
 }
 
 // Launches the vector GEMV with the tile depth and prologue shape that fit N (N <= 8192 * VP).

@@ -87,16 +87,7 @@ extern "C" size_t rwkv_v4_one_workspace(const rwkv_v4_model *m) {
 // Head: LN_out(x) @ head -> fp32 logits (fp16-rounded).  Shared by the one-token and the
 // sequence entry points (last token only).
 int v4_head_launch(const rwkv_v4_model *m, const rwkv_half *x, float *logits, hipStream_t st) {
-    const int C = m->n_embd;
-    LnMixArgs h{};
-    h.x = x; h.C = C; h.ln_w = m->ln_out_w; h.ln_b = m->ln_out_b; h.sx = nullptr; h.xx_tmp = nullptr;
-    h.mix[0] = nullptr; h.mat[0] = to_dev(m->head); h.M[0] = m->vocab; h.epi[0] = EPI_LOGITS; h.out[0] = logits;
-    const size_t lds = (size_t)C * 2;
-    const int grid = num_cu();
-    if (m->weights_u8)
-        hipLaunchKernelGGL((lnmix_kernel<true, 1, 4>), dim3(grid), dim3(DTHREADS), lds, st, h);
-    else
-        hipLaunchKernelGGL((lnmix_kernel<false, 1, 4>), dim3(grid), dim3(DTHREADS), lds, st, h);
+    lnhead_launch(m->weights_u8 != 0, x, m->n_embd, m->ln_out_w, m->ln_out_b, to_dev(m->head), m->vocab, logits, num_cu(), st);
     RWKV_LAUNCH_CHECK();
     return RWKV_OK;
 }
@@ -166,18 +157,7 @@ static int v4_one_impl(const rwkv_v4_model *m, const rwkv_v4_layer_state *states
             a.out[0] = ws.r_ffn;
             a.mix[1] = l.ffn_mix_k; a.mat[1] = to_dev(l.ffn_key); a.M[1] = F; a.epi[1] = EPI_RELU_SQ;
             a.out[1] = ws.vx;
-            const size_t lds = 2 * (size_t)C * 2;
-            const int per = (C + F + grid * DWAVES - 1) / (grid * DWAVES);
-            if (per % 5 == 0) {
-                if (u8) hipLaunchKernelGGL((lnmix_kernel<true, 2, 5>), dim3(grid), dim3(DTHREADS), lds, st, a);
-                else hipLaunchKernelGGL((lnmix_kernel<false, 2, 5>), dim3(grid), dim3(DTHREADS), lds, st, a);
-            } else if (per >= 4) {
-                if (u8) hipLaunchKernelGGL((lnmix_kernel<true, 2, 4>), dim3(grid), dim3(DTHREADS), lds, st, a);
-                else hipLaunchKernelGGL((lnmix_kernel<false, 2, 4>), dim3(grid), dim3(DTHREADS), lds, st, a);
-            } else {
-                if (u8) hipLaunchKernelGGL((lnmix_kernel<true, 2, 2>), dim3(grid), dim3(DTHREADS), lds, st, a);
-                else hipLaunchKernelGGL((lnmix_kernel<false, 2, 2>), dim3(grid), dim3(DTHREADS), lds, st, a);
-            }
+            lnmix2_launch(u8, a, grid, st);
             mark();
         }
         if (only_phase < 0 || only_phase == 3) {

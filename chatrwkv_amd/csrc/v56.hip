@@ -78,22 +78,28 @@ struct Mix2Args {
     rwkv_half *out[5];               // [T, C] each
 };
 
-// grid (T, C/256): m_j[c] = sum_i t1[t, jR + i] * w2[j][i][c]; out_j = xx + sxd * (maa_j + m_j).
+// grid (T, C/256, 5): m_j[c] = sum_i t1[t, jR + i] * w2[j][i][c]; out_j = xx + sxd * (maa_j + m_j).
+// One (channel, mix) per thread; the rank loop loads 16 coefficients before it adds them (in index order).
 __global__ __launch_bounds__(256) void v6_mix2_kernel(Mix2Args a) {
-    __shared__ float st1[5 * 64];
-    const int t = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x, R = a.R, C = a.C;
-    for (int i = threadIdx.x; i < 5 * R; i += 256) st1[i] = h2f(a.t1[(size_t)t * 5 * R + i]);
+    __shared__ float st1[64];
+    const int t = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x, j = blockIdx.z, R = a.R, C = a.C;
+    for (int i = threadIdx.x; i < R; i += 256) st1[i] = h2f(a.t1[(size_t)t * 5 * R + j * R + i]);
     __syncthreads();
     if (c >= C) return;
     const float xx = h2f(a.xx[(size_t)t * C + c]), sd = h2f(a.sxd[(size_t)t * C + c]);
+    const rwkv_half maa = a.maa[j][c];
+    const rwkv_half *w = a.w2 + (size_t)j * R * C + c;
+    float m = 0.f;
+    for (int i0 = 0; i0 < R; i0 += 16) {
+        rwkv_half wv[16];
 #pragma unroll
-    for (int j = 0; j < 5; ++j) {
-        float m = 0.f;
-        const rwkv_half *w = a.w2 + (size_t)j * R * C + c;
-        for (int i = 0; i < R; ++i) m += st1[j * R + i] * h2f(w[(size_t)i * C]);
-        const float mm = round_h(h2f(a.maa[j][c]) + round_h(m));
-        a.out[j][(size_t)t * C + c] = f2h(xx + round_h(sd * mm));
+        for (int i = 0; i < 16; ++i) wv[i] = w[(size_t)min(i0 + i, R - 1) * C];
+#pragma unroll
+        for (int i = 0; i < 16; ++i)
+            if (i0 + i < R) m += st1[i0 + i] * h2f(wv[i]);
     }
+    const float mm = round_h(h2f(maa) + round_h(m));
+    a.out[j][(size_t)t * C + c] = f2h(xx + round_h(sd * mm));
 }
 
 MatDev to_dev56(const rwkv_mat &m) { return MatDev{m.w, m.ld, m.mx, m.rx, m.my, m.ry}; }
@@ -257,7 +263,7 @@ extern "C" int rwkv_v56_forward(const rwkv_v56_model *m, const rwkv_v56_layer_st
             Mix2Args b{};
             b.T = (int)T; b.C = C; b.R = lm; b.t1 = ws.t1; b.w2 = l.tm_w2; b.xx = ws.xx; b.sxd = ws.sxd;
             for (int j = 0; j < 5; ++j) { b.maa[j] = l.att_mix[1 + j]; b.out[j] = ws.mix[j]; }
-            hipLaunchKernelGGL(v6_mix2_kernel, dim3((unsigned)T, (unsigned)((C + 255) / 256)), dim3(256), 0, st, b);
+            hipLaunchKernelGGL(v6_mix2_kernel, dim3((unsigned)T, (unsigned)((C + 255) / 256), 5), dim3(256), 0, st, b);
             wx = ws.mix[0]; kx = ws.mix[1]; vx = ws.mix[2]; rx = ws.mix[3]; gx = ws.mix[4];
             if ((rc = mm(c, lora_mat(l.td_w1, C, ld), false, wx, ACT_TANH, nullptr, nullptr, 1.f, ws.d1))) return rc;
             if ((rc = mm(c, lora_mat(l.td_w2, ld, C), false, ws.d1, ACT_NONE, nullptr, nullptr, 1.f, ws.d2))) return rc;
@@ -271,15 +277,40 @@ extern "C" int rwkv_v56_forward(const rwkv_v56_model *m, const rwkv_v56_layer_st
             kx = ws.mix[0]; vx = ws.mix[1]; rx = ws.mix[2]; gx = gated ? ws.mix[3] : nullptr;
         }
         // the first matrix call also commits the new token-shift state (all readers of the old one are done)
-        if ((rc = mm(c, l.att_receptance, u8, rx, ACT_NONE, nullptr, nullptr, 1.f, ws.r, ws.xx_att, s.att_xx, C))) return rc;
-        if ((rc = mm(c, l.att_key, u8, kx, ACT_NONE, nullptr, nullptr, 1.f, ws.k))) return rc;
-        if ((rc = mm(c, l.att_value, u8, vx, ACT_NONE, nullptr, nullptr, 1.f, ws.v))) return rc;
-        if (gated && (rc = mm(c, l.att_gate, u8, gx, ACT_SILU, nullptr, nullptr, 1.f, ws.g))) return rc;
+        if (T == 1 && C <= 8 * 512) {
+            // one launch for the receptance, key, value (and gate) rows
+            MultiVecArgs a{};
+            a.N = C; a.M = C; a.nm = gated ? 4 : 3;
+            a.vin[0] = rx; a.mat[0] = to_dev56(l.att_receptance); a.act[0] = VACT_F16; a.out[0] = ws.r;
+            a.vin[1] = kx; a.mat[1] = to_dev56(l.att_key); a.act[1] = VACT_F16; a.out[1] = ws.k;
+            a.vin[2] = vx; a.mat[2] = to_dev56(l.att_value); a.act[2] = VACT_F16; a.out[2] = ws.v;
+            if (gated) { a.vin[3] = gx; a.mat[3] = to_dev56(l.att_gate); a.act[3] = VACT_SILU; a.out[3] = ws.g; }
+            a.commit_src = ws.xx_att; a.commit_dst = s.att_xx; a.commit_n = C;
+            multi_vec_launch(u8, a, c.grid, st);
+        } else {
+            if ((rc = mm(c, l.att_receptance, u8, rx, ACT_NONE, nullptr, nullptr, 1.f, ws.r, ws.xx_att, s.att_xx, C))) return rc;
+            if ((rc = mm(c, l.att_key, u8, kx, ACT_NONE, nullptr, nullptr, 1.f, ws.k))) return rc;
+            if ((rc = mm(c, l.att_value, u8, vx, ACT_NONE, nullptr, nullptr, 1.f, ws.v))) return rc;
+            if (gated && (rc = mm(c, l.att_gate, u8, gx, ACT_SILU, nullptr, nullptr, 1.f, ws.g))) return rc;
+        }
         if ((rc = wkv56_fused_launch(v6, (int)T, C, H, s.att_kv, ws.r, ws.k, ws.v, v6 ? (const void *)ws.d2 : (const void *)l.time_decay,
                                      l.time_decay, l.time_first, l.lnx_w, l.lnx_b, gated ? ws.g : nullptr, ws.att, st)))
             return rc;
         if ((rc = mm(c, l.att_output, u8, ws.att, ACT_RESIDUAL, ws.x, nullptr, 1.f, ws.x))) return rc;
         // ---- channel mix
+        const float scale = (m->rescale_layer > 0 && (i + 1) % m->rescale_layer == 0) ? 0.5f : 1.f;
+        if (T == 1) {
+            // LN2 + token shift + receptance and key rows in one launch, then the value rows
+            LnMixArgs a{};
+            a.x = ws.x; a.C = C; a.ln_w = l.ln2_w; a.ln_b = l.ln2_b; a.sx = s.ffn_xx; a.xx_tmp = ws.xx_ffn;
+            a.mix[0] = l.ffn_mix_r; a.mat[0] = to_dev56(l.ffn_receptance); a.M[0] = C; a.epi[0] = EPI_SIGMOID; a.out[0] = ws.r;
+            a.mix[1] = l.ffn_mix_k; a.mat[1] = to_dev56(l.ffn_key); a.M[1] = F; a.epi[1] = EPI_RELU_SQ; a.out[1] = ws.vx;
+            a.maa_form = v6 ? 1 : 0;
+            lnmix2_launch(u8, a, c.grid, st);
+            if ((rc = mm(c, l.ffn_value, u8, ws.vx, ACT_GATED_RESIDUAL, ws.x, ws.r, scale, ws.x, ws.xx_ffn, s.ffn_xx, C))) return rc;
+            RWKV_LAUNCH_CHECK();
+            continue;
+        }
         {
             SeqMixArgs a{};
             a.T = (int)T; a.C = C; a.x = ws.x; a.ln_w = l.ln2_w; a.ln_b = l.ln2_b; a.sx = s.ffn_xx;
@@ -290,7 +321,6 @@ extern "C" int rwkv_v56_forward(const rwkv_v56_model *m, const rwkv_v56_layer_st
         }
         if ((rc = mm(c, l.ffn_receptance, u8, ws.mix[0], ACT_SIGMOID, nullptr, nullptr, 1.f, ws.r, ws.xx_ffn, s.ffn_xx, C))) return rc;
         if ((rc = mm(c, l.ffn_key, u8, ws.mix[1], ACT_RELU_SQ, nullptr, nullptr, 1.f, ws.vx))) return rc;
-        const float scale = (m->rescale_layer > 0 && (i + 1) % m->rescale_layer == 0) ? 0.5f : 1.f;
         if ((rc = mm(c, l.ffn_value, u8, ws.vx, ACT_GATED_RESIDUAL, ws.x, ws.r, scale, ws.x))) return rc;
         RWKV_LAUNCH_CHECK();
     }
@@ -298,19 +328,16 @@ extern "C" int rwkv_v56_forward(const rwkv_v56_model *m, const rwkv_v56_layer_st
     const bool all_rows = full_output && T > 1;
     const int64_t TH = all_rows ? T : 1;
     const rwkv_half *xh = all_rows ? ws.x : ws.x + (size_t)(T - 1) * C;
+    if (TH == 1) {
+        lnhead_launch(u8, xh, C, m->ln_out_w, m->ln_out_b, to_dev56(m->head), m->vocab, logits, c.grid, st);
+        RWKV_LAUNCH_CHECK();
+        return RWKV_OK;
+    }
     {
         SeqMixArgs a{};
         a.T = (int)TH; a.C = C; a.x = xh; a.ln_w = m->ln_out_w; a.ln_b = m->ln_out_b; a.sx = nullptr; a.xx_last = nullptr;
         a.mix[0] = nullptr; a.ry[0] = nullptr; a.my[0] = nullptr; a.xs[0] = ws.xx;
         if ((rc = lnmix_seq_launch(a, 1, st))) return rc;
-    }
-    if (TH == 1) {
-        VecArgs a{};
-        a.vin = ws.xx; a.N = C; a.M = m->vocab; a.mat = to_dev56(m->head); a.act = VACT_LOGITS; a.out = logits;
-        a.out_scale = 1.f;
-        vec_launch(u8, a, c.grid, st);
-        RWKV_LAUNCH_CHECK();
-        return RWKV_OK;
     }
     const rwkv_half *A = ws.xx;
     GemmEpi e{};
