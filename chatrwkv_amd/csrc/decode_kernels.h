@@ -338,7 +338,7 @@ __global__ __launch_bounds__(DTHREADS) void att_kernel(AttArgs a) {
 }
 
 // ------------------------------------------------------------------------------------------
-enum { EPI_SIGMOID = 0, EPI_RELU_SQ = 1, EPI_LOGITS = 2 };
+enum { EPI_SIGMOID = 0, EPI_RELU_SQ = 1, EPI_LOGITS = 2, EPI_TANH = 3 };
 
 struct LnMixArgs {
     const rwkv_half *x;
@@ -391,6 +391,8 @@ __global__ __launch_bounds__(DTHREADS) void lnmix_kernel(LnMixArgs a) {
         const int kind = a.epi[j];
         if (kind == EPI_LOGITS) {
             ((float *)a.out[j])[m] = v;
+        } else if (kind == EPI_TANH) {
+            ((rwkv_half *)a.out[j])[m] = f2h(tanhf(v));
         } else if (kind == EPI_SIGMOID) {
             ((rwkv_half *)a.out[j])[m] = f2h(sigmoidf_(v));
         } else {
@@ -640,6 +642,13 @@ inline void lnmix2_launch(bool u8, const LnMixArgs &a, int grid, hipStream_t st)
         if (u8) hipLaunchKernelGGL((lnmix_kernel<true, 2, 2>), dim3(grid), dim3(DTHREADS), lds, st, a);
         else hipLaunchKernelGGL((lnmix_kernel<false, 2, 2>), dim3(grid), dim3(DTHREADS), lds, st, a);
     }
+}
+
+// LN + token shift + one mix + a GEMV over a FEW rows of an fp16 matrix (RWKV-6: the first LoRA product of
+// the data-dependent mixes), one row per wave.
+inline void lnmix1_small_launch(const LnMixArgs &a, hipStream_t st) {
+    const int grid = (a.M[0] + DWAVES - 1) / DWAVES;
+    hipLaunchKernelGGL((lnmix_kernel<false, 1, 1>), dim3(grid), dim3(DTHREADS), (size_t)a.C * 2, st, a);
 }
 
 // LN_out(x) @ head -> fp32 logits (fp16-rounded values) in one launch.

@@ -27,7 +27,8 @@ int wkv4_fused_launch(int T, int C, const float *w, const float *u, const void *
                       const rwkv_half *r, rwkv_half *y, float *aa, float *bb, float *pp, hipStream_t st);
 int wkv56_fused_launch(bool v6, int T, int C, int H, float *state, const rwkv_half *r, const rwkv_half *k,
                        const rwkv_half *v, const void *w, const float *t_decay, const float *u, const float *lnx_w,
-                       const float *lnx_b, const rwkv_half *gate, rwkv_half *out, hipStream_t st);
+                       const float *lnx_b, const rwkv_half *gate, rwkv_half *out, hipStream_t st,
+                       const rwkv_half *dw2 = nullptr, int ld = 0);  // dw2: v6 with w = tanh(. @ D1), product with D2 in-kernel
 // Row-wise LayerNorm + token shift + mixes for up to 4 consumers over a [T, C] activation (seq_v4.hip).
 struct SeqMixArgs {
     int T, C;

@@ -73,7 +73,8 @@ struct Mix2Args {
     int T, C, R;                     // R = LoRA rank (32)
     const rwkv_half *t1;             // [T, 5R] tanh output
     const rwkv_half *w2;             // [5][R][C]
-    const rwkv_half *xx, *sxd;       // [T, C]
+    const rwkv_half *xx, *sxd;       // [T, C]; sxd NULL (T == 1): prev - xx is formed here from `prev`
+    const rwkv_half *prev;           // [C] token-shift state
     const rwkv_half *maa[5];         // w, k, v, r, g
     rwkv_half *out[5];               // [T, C] each
 };
@@ -86,7 +87,8 @@ __global__ __launch_bounds__(256) void v6_mix2_kernel(Mix2Args a) {
     for (int i = threadIdx.x; i < R; i += 256) st1[i] = h2f(a.t1[(size_t)t * 5 * R + j * R + i]);
     __syncthreads();
     if (c >= C) return;
-    const float xx = h2f(a.xx[(size_t)t * C + c]), sd = h2f(a.sxd[(size_t)t * C + c]);
+    const float xx = h2f(a.xx[(size_t)t * C + c]);
+    const float sd = a.sxd ? h2f(a.sxd[(size_t)t * C + c]) : round_h(h2f(a.prev[c]) - xx);
     const rwkv_half maa = a.maa[j][c];
     const rwkv_half *w = a.w2 + (size_t)j * R * C + c;
     float m = 0.f;
@@ -257,16 +259,27 @@ extern "C" int rwkv_v56_forward(const rwkv_v56_model *m, const rwkv_v56_layer_st
         const rwkv_v56_layer_state &s = states[i];
         const rwkv_half *kx, *vx, *rx, *gx = nullptr, *wx = nullptr;
         if (v6) {
-            Mix1Args a{(int)T, C, ws.x, l.ln1_w, l.ln1_b, s.att_xx, l.att_mix[0], ws.xx, ws.sxd, ws.xxx, ws.xx_att};
-            hipLaunchKernelGGL(v6_mix1_kernel, dim3((unsigned)T), dim3(256), 0, st, a);
-            if ((rc = mm(c, lora_mat(l.tm_w1, C, 5 * lm), false, ws.xxx, ACT_TANH, nullptr, nullptr, 1.f, ws.t1))) return rc;
             Mix2Args b{};
-            b.T = (int)T; b.C = C; b.R = lm; b.t1 = ws.t1; b.w2 = l.tm_w2; b.xx = ws.xx; b.sxd = ws.sxd;
+            if (T == 1) {
+                // LN1 + xxx = xx + (prev - xx) * maa_x + the first LoRA product (tanh) in one launch
+                LnMixArgs a{};
+                a.x = ws.x; a.C = C; a.ln_w = l.ln1_w; a.ln_b = l.ln1_b; a.sx = s.att_xx; a.xx_tmp = ws.xx_att;
+                a.mix[0] = l.att_mix[0]; a.mat[0] = MatDev{l.tm_w1, C, nullptr, nullptr, nullptr, nullptr};
+                a.M[0] = 5 * lm; a.epi[0] = EPI_TANH; a.out[0] = ws.t1; a.maa_form = 1;
+                lnmix1_small_launch(a, st);
+                b.xx = ws.xx_att; b.sxd = nullptr; b.prev = s.att_xx;
+            } else {
+                Mix1Args a{(int)T, C, ws.x, l.ln1_w, l.ln1_b, s.att_xx, l.att_mix[0], ws.xx, ws.sxd, ws.xxx, ws.xx_att};
+                hipLaunchKernelGGL(v6_mix1_kernel, dim3((unsigned)T), dim3(256), 0, st, a);
+                if ((rc = mm(c, lora_mat(l.tm_w1, C, 5 * lm), false, ws.xxx, ACT_TANH, nullptr, nullptr, 1.f, ws.t1))) return rc;
+                b.xx = ws.xx; b.sxd = ws.sxd; b.prev = nullptr;
+            }
+            b.T = (int)T; b.C = C; b.R = lm; b.t1 = ws.t1; b.w2 = l.tm_w2;
             for (int j = 0; j < 5; ++j) { b.maa[j] = l.att_mix[1 + j]; b.out[j] = ws.mix[j]; }
             hipLaunchKernelGGL(v6_mix2_kernel, dim3((unsigned)T, (unsigned)((C + 255) / 256), 5), dim3(256), 0, st, b);
             wx = ws.mix[0]; kx = ws.mix[1]; vx = ws.mix[2]; rx = ws.mix[3]; gx = ws.mix[4];
             if ((rc = mm(c, lora_mat(l.td_w1, C, ld), false, wx, ACT_TANH, nullptr, nullptr, 1.f, ws.d1))) return rc;
-            if ((rc = mm(c, lora_mat(l.td_w2, ld, C), false, ws.d1, ACT_NONE, nullptr, nullptr, 1.f, ws.d2))) return rc;
+            if (T > 1 && (rc = mm(c, lora_mat(l.td_w2, ld, C), false, ws.d1, ACT_NONE, nullptr, nullptr, 1.f, ws.d2))) return rc;
         } else {
             SeqMixArgs a{};
             a.T = (int)T; a.C = C; a.x = ws.x; a.ln_w = l.ln1_w; a.ln_b = l.ln1_b; a.sx = s.att_xx;
@@ -293,8 +306,12 @@ extern "C" int rwkv_v56_forward(const rwkv_v56_model *m, const rwkv_v56_layer_st
             if ((rc = mm(c, l.att_value, u8, vx, ACT_NONE, nullptr, nullptr, 1.f, ws.v))) return rc;
             if (gated && (rc = mm(c, l.att_gate, u8, gx, ACT_SILU, nullptr, nullptr, 1.f, ws.g))) return rc;
         }
-        if ((rc = wkv56_fused_launch(v6, (int)T, C, H, s.att_kv, ws.r, ws.k, ws.v, v6 ? (const void *)ws.d2 : (const void *)l.time_decay,
-                                     l.time_decay, l.time_first, l.lnx_w, l.lnx_b, gated ? ws.g : nullptr, ws.att, st)))
+        // one token of v6: the second decay LoRA product is done inside the WKV kernel
+        const bool d2_fused = v6 && T == 1;
+        if ((rc = wkv56_fused_launch(v6, (int)T, C, H, s.att_kv, ws.r, ws.k, ws.v,
+                                     v6 ? (const void *)(d2_fused ? ws.d1 : ws.d2) : (const void *)l.time_decay, l.time_decay,
+                                     l.time_first, l.lnx_w, l.lnx_b, gated ? ws.g : nullptr, ws.att, st,
+                                     d2_fused ? l.td_w2 : nullptr, ld)))
             return rc;
         if ((rc = mm(c, l.att_output, u8, ws.att, ACT_RESIDUAL, ws.x, nullptr, 1.f, ws.x))) return rc;
         // ---- channel mix

@@ -1,4 +1,5 @@
 // WKV recurrences: RWKV-4 (per channel, running-maximum form) and RWKV-5/6 (per-head 64x64 state).
+#include "gemv_core.h"
 #include "kernels.h"
 
 namespace {
@@ -115,6 +116,8 @@ struct Wkv56Args {
     const float *lnx_w, *lnx_b;
     const rwkv_half *gate;
     rwkv_half *out;
+    const rwkv_half *dw2;  // WMODE 3: second decay LoRA matrix, row c = ld coefficients of channel c
+    int ld;                // WMODE 3: LoRA rank (multiple of 8); w = tanh(. @ D1) [T, ld] fp16
 };
 
 template <bool IN_F16, int WMODE, bool OUT_GN>
@@ -133,7 +136,7 @@ __global__ __launch_bounds__(256) void wkv56_kernel(Wkv56Args a) {
         s[jj] = a.state_layout == 0 ? S[i * HS + j] : S[j * HS + i];
     }
     float tdec = 0.f;
-    if (WMODE == 2) tdec = a.t_decay[h * HS + i];
+    if (WMODE >= 2) tdec = a.t_decay[h * HS + i];
     if (threadIdx.x < HS) {
         su[threadIdx.x] = a.u[h * HS + threadIdx.x];
         if (WMODE == 0) sw[0][threadIdx.x] = ((const float *)a.w)[h * HS + threadIdx.x];
@@ -150,6 +153,15 @@ __global__ __launch_bounds__(256) void wkv56_kernel(Wkv56Args a) {
             sr[tt][c] = ld(a.r, o); sk[tt][c] = ld(a.k, o); sv[tt][c] = ld(a.v, o);
             if (WMODE == 1) sw[tt][c] = ((const float *)a.w)[o];
             if (WMODE == 2) sw[tt][c] = expf(-expf(tdec + h2f(((const rwkv_half *)a.w)[o])));
+            if (WMODE == 3) {
+                // decay LoRA: the rank-ld product for this channel, rounded to fp16 like the matrix product it replaces
+                const rwkv_half *wr = a.dw2 + (size_t)(h * HS + c) * a.ld;
+                const rwkv_half *dv = (const rwkv_half *)a.w + (size_t)(t0 + tt) * a.ld;
+                float acc = 0.f;
+                for (int j8 = 0; j8 < (a.ld >> 3); ++j8)
+                    acc = dot8_f16(*(const u32x4 *)(wr + 8 * j8), *(const h16x8 *)(dv + 8 * j8), acc);
+                sw[tt][c] = expf(-expf(tdec + round_h(acc)));
+            }
         }
         __syncthreads();
         for (int tt = 0; tt < nt; ++tt) {
@@ -253,13 +265,17 @@ static int wkv56_launch(bool v6, int64_t B, int64_t T, int64_t C, int64_t H, flo
 // v6: w = fp16 LoRA output [T, C], t_decay fp32 [C]; v5: w = fp32 decay [C], t_decay unused.
 int wkv56_fused_launch(bool v6, int T, int C, int H, float *state, const rwkv_half *r, const rwkv_half *k,
                        const rwkv_half *v, const void *w, const float *t_decay, const float *u, const float *lnx_w,
-                       const float *lnx_b, const rwkv_half *gate, rwkv_half *out, hipStream_t st) {
+                       const float *lnx_b, const rwkv_half *gate, rwkv_half *out, hipStream_t st,
+                       const rwkv_half *dw2, int ld) {
     if (C != H * HS) return RWKV_E_SHAPE;
     Wkv56Args a{};
     a.T = T; a.C = C; a.state = state; a.state_layout = 1;
     a.r = r; a.k = k; a.v = v; a.w = w; a.u = u; a.t_decay = t_decay;
-    a.lnx_w = lnx_w; a.lnx_b = lnx_b; a.gate = gate; a.out = out;
-    if (v6)
+    a.lnx_w = lnx_w; a.lnx_b = lnx_b; a.gate = gate; a.out = out; a.dw2 = dw2; a.ld = ld;
+    if (v6 && dw2) {
+        if (ld <= 0 || (ld & 7)) return RWKV_E_SHAPE;
+        hipLaunchKernelGGL((wkv56_kernel<true, 3, true>), dim3((unsigned)H), dim3(256), 0, st, a);
+    } else if (v6)
         hipLaunchKernelGGL((wkv56_kernel<true, 2, true>), dim3((unsigned)H), dim3(256), 0, st, a);
     else
         hipLaunchKernelGGL((wkv56_kernel<true, 0, true>), dim3((unsigned)H), dim3(256), 0, st, a);
