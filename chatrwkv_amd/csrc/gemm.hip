@@ -31,10 +31,51 @@ constexpr int BK = 64;  // halves per LDS row
 // the 8 odd rows of 16 consecutive rows must each hit 8 different slots).
 DEV int swz(int row, int chunk) { return row * BK + ((chunk ^ ((row & 7) ^ ((row >> 3) & 1))) << 3); }
 
-template <bool W_U8, int BT, int BM, int WT, int WM, int PF>
+// Epilogue of one output element: rank-1 corrections of the uint8 format, activation / residual, store.
+DEV void gemm_epilogue(float v, int t, int m, float rxm, float mxm, const GemmEpi &ep, void *Y, int64_t ldy) {
+    if (ep.rx) v = rxm * v + mxm * ep.s0[t] + ep.s2[t];
+    if (ep.raw_f32) {
+        ((float *)Y)[(size_t)t * ldy + m] = v;
+        return;
+    }
+    float o = round_h(v);
+    switch (ep.act) {
+        case ACT_SIGMOID: o = sigmoidf_(o); break;
+        case ACT_RELU_SQ: o = fmaxf(o, 0.f); o = o * o; break;
+        case ACT_SILU: o = o * sigmoidf_(o); break;
+        case ACT_TANH: o = tanhf(o); break;
+        case ACT_RESIDUAL: o = h2f(ep.res[(size_t)t * ep.ldres + m]) + o; break;
+        case ACT_GATED_RESIDUAL:
+            o = round_h(h2f(ep.gate[(size_t)t * ep.ldgate + m]) * o);
+            o = h2f(ep.res[(size_t)t * ep.ldres + m]) + o;
+            break;
+        default: break;
+    }
+    if (ep.out_scale != 1.f) o = round_h(o) * ep.out_scale;
+    if (ep.out_dtype == RWKV_DT_F32)
+        ((float *)Y)[(size_t)t * ldy + m] = round_h(o);
+    else
+        ((rwkv_half *)Y)[(size_t)t * ldy + m] = f2h(o);
+}
+
+// Split-K second pass: sums the KS partial slabs [KS][T][M] in slab order (deterministic) and runs the epilogue.
+__global__ __launch_bounds__(256) void splitk_epilogue_kernel(int T, int M, int KS, const float *__restrict__ part, void *Y,
+                                                              int64_t ldy, GemmEpi ep) {
+    const int64_t n = (int64_t)T * M;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
+        const int t = (int)(i / M), m = (int)(i - (int64_t)t * M);
+        float v = 0.f;
+        for (int k = 0; k < KS; ++k) v += part[(size_t)k * n + i];
+        float rxm = 1.f, mxm = 0.f;
+        if (ep.rx) { rxm = h2f(ep.rx[m]); mxm = h2f(ep.mx[m]); }
+        gemm_epilogue(v, t, m, rxm, mxm, ep, Y, ldy);
+    }
+}
+
+template <bool W_U8, int BT, int BM, int WT, int WM, int PF, bool SPLIT>
 __global__ __launch_bounds__(256) void gemm_kernel(int T, int N, int M, const h16 *__restrict__ A, int64_t lda,
                                                    const void *__restrict__ Wv, int64_t ldw, void *__restrict__ Y,
-                                                   int64_t ldy, GemmEpi ep) {
+                                                   int64_t ldy, GemmEpi ep, int nk_split, float *__restrict__ part) {
     static_assert(WT * WM == 4 && BT % (32 * WT) == 0 && BM % (32 * WM) == 0 && BM % 64 == 0, "tile");
     constexpr int MI = BT / (32 * WT), NI = BM / (32 * WM);  // 32x32 blocks per wave in each direction
     extern __shared__ __align__(16) unsigned char smem[];
@@ -59,8 +100,10 @@ __global__ __launch_bounds__(256) void gemm_kernel(int T, int N, int M, const h1
     // the LDS holds the tile being multiplied and the next one.
     u32x4 ra[PF][A_LD], rb[PF][B_LD];
 
+    // split-K: blockIdx.y owns k-tiles [kbase, kbase + nk) and writes raw partial sums to its slab
+    const int kbase = SPLIT ? blockIdx.y * nk_split : 0;
     auto load_tiles = [&](u32x4 (&qa)[A_LD], u32x4 (&qb)[B_LD], int kt) {
-        const int k0 = kt * BK;
+        const int k0 = (kbase + kt) * BK;
 #pragma unroll
         for (int i = 0; i < A_LD; ++i) {
             const int row = (tid >> 3) + 32 * i, ch = tid & 7;
@@ -127,7 +170,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(int T, int N, int M, const h1
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[a][b][e] = 0.f;
 
-    const int nk = N / BK;
+    const int nk = SPLIT ? nk_split : N / BK;
     auto compute = [&](int buf) {
 #pragma unroll
         for (int ks = 0; ks < BK / 16; ++ks) {
@@ -171,42 +214,21 @@ __global__ __launch_bounds__(256) void gemm_kernel(int T, int N, int M, const h1
     }
 
     // epilogue: lane holds column m = .. + (lane & 31) and rows 8*(e/4) + 4*(lane>>5) + e%4
+    float *slab = SPLIT ? part + (size_t)blockIdx.y * T * M : nullptr;
 #pragma unroll
     for (int b = 0; b < NI; ++b) {
         const int m = m0 + wc * (BM / WM) + b * 32 + (lane & 31);
         if (m >= M) continue;
         float rxm = 1.f, mxm = 0.f;
-        if (ep.rx) { rxm = h2f(ep.rx[m]); mxm = h2f(ep.mx[m]); }
+        if (!SPLIT && ep.rx) { rxm = h2f(ep.rx[m]); mxm = h2f(ep.mx[m]); }
 #pragma unroll
         for (int a = 0; a < MI; ++a) {
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
                 const int t = t0 + wr * (BT / WT) + a * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
                 if (t >= T) continue;
-                float v = acc[a][b][e];
-                if (ep.rx) v = rxm * v + mxm * ep.s0[t] + ep.s2[t];
-                if (ep.raw_f32) {
-                    ((float *)Y)[(size_t)t * ldy + m] = v;
-                    continue;
-                }
-                float o = round_h(v);
-                switch (ep.act) {
-                    case ACT_SIGMOID: o = sigmoidf_(o); break;
-                    case ACT_RELU_SQ: o = fmaxf(o, 0.f); o = o * o; break;
-                    case ACT_SILU: o = o * sigmoidf_(o); break;
-                    case ACT_TANH: o = tanhf(o); break;
-                    case ACT_RESIDUAL: o = h2f(ep.res[(size_t)t * ep.ldres + m]) + o; break;
-                    case ACT_GATED_RESIDUAL:
-                        o = round_h(h2f(ep.gate[(size_t)t * ep.ldgate + m]) * o);
-                        o = h2f(ep.res[(size_t)t * ep.ldres + m]) + o;
-                        break;
-                    default: break;
-                }
-                if (ep.out_scale != 1.f) o = round_h(o) * ep.out_scale;
-                if (ep.out_dtype == RWKV_DT_F32)
-                    ((float *)Y)[(size_t)t * ldy + m] = round_h(o);
-                else
-                    ((rwkv_half *)Y)[(size_t)t * ldy + m] = f2h(o);
+                if (SPLIT) slab[(size_t)t * M + m] = acc[a][b][e];
+                else gemm_epilogue(acc[a][b][e], t, m, rxm, mxm, ep, Y, ldy);
             }
         }
     }
@@ -252,14 +274,35 @@ int launch_cfg(int64_t T, int64_t N, int64_t M, const rwkv_half *A, int64_t lda,
     constexpr size_t lds = 2 * (size_t)(BT + BM) * BK * sizeof(h16);
     static bool attr_done = false;
     if (lds > 64 * 1024 && !attr_done) {
-        hipError_t e = hipFuncSetAttribute((const void *)gemm_kernel<W_U8, BT, BM, WT, WM, PF>,
+        hipError_t e = hipFuncSetAttribute((const void *)gemm_kernel<W_U8, BT, BM, WT, WM, PF, false>,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return (int)e;
         attr_done = true;
     }
     const int64_t tiles = ((T + BT - 1) / BT) * ((M + BM - 1) / BM);
-    hipLaunchKernelGGL((gemm_kernel<W_U8, BT, BM, WT, WM, PF>), dim3((unsigned)tiles), dim3(256), lds, st, (int)T, (int)N,
-                       (int)M, (const h16 *)A, lda, W, ldw, Y, ldy, ep);
+    // Too few tiles to fill the chip (short prompts, narrow matrices): split the contraction over KS
+    // workgroups per tile; partial sums go to fp32 slabs and a second pass reduces them in slab order.
+    int ks = 1;
+    const int nk = (int)(N / BK);
+    if (ep.splitk_ws && tiles <= 128 && lds <= 64 * 1024) {
+        for (int c = 8; c >= 2; c >>= 1) {
+            if (nk % c || nk / c < 8) continue;                                   // whole k-tiles, several per split
+            if (tiles * c > 512) continue;                                        // two workgroups per CU are enough
+            if ((size_t)c * T * M * sizeof(float) > ep.splitk_bytes) continue;    // slabs must fit
+            ks = c;
+            break;
+        }
+    }
+    if (ks > 1) {
+        hipLaunchKernelGGL((gemm_kernel<W_U8, BT, BM, WT, WM, PF, true>), dim3((unsigned)tiles, (unsigned)ks), dim3(256), lds, st,
+                           (int)T, (int)N, (int)M, (const h16 *)A, lda, W, ldw, Y, ldy, ep, nk / ks, ep.splitk_ws);
+        const int64_t n = T * M;
+        const unsigned blocks = (unsigned)((n + 1023) / 1024 < 4096 ? (n + 1023) / 1024 : 4096);
+        hipLaunchKernelGGL(splitk_epilogue_kernel, dim3(blocks), dim3(256), 0, st, (int)T, (int)M, ks, ep.splitk_ws, Y, ldy, ep);
+    } else {
+        hipLaunchKernelGGL((gemm_kernel<W_U8, BT, BM, WT, WM, PF, false>), dim3((unsigned)tiles), dim3(256), lds, st, (int)T,
+                           (int)N, (int)M, (const h16 *)A, lda, W, ldw, Y, ldy, ep, nk, (float *)nullptr);
+    }
     RWKV_LAUNCH_CHECK();
     return RWKV_OK;
 }
@@ -307,7 +350,7 @@ int mm8_prepare_launch(int64_t T, int64_t N, const rwkv_half *x, int64_t ldx, co
 
 extern "C" size_t rwkv_mm8_seq_workspace(int64_t B, int64_t N) {
     if (B <= 0 || N <= 0) return 0;
-    return (size_t)B * N * 2 + 256 + (size_t)B * 8;
+    return (((size_t)B * N * 2 + 255) & ~(size_t)255) + (((size_t)B * 8 + 255) & ~(size_t)255) + RWKV_SPLITK_WS_BYTES;
 }
 
 extern "C" int rwkv_mm8_seq_f16(int64_t B, int64_t N, int64_t M, const rwkv_half *x, int64_t x_stride,
@@ -329,6 +372,8 @@ extern "C" int rwkv_mm8_seq_f16(int64_t B, int64_t N, int64_t M, const rwkv_half
     if (rc) return rc;
     GemmEpi ep{};
     ep.mx = mx; ep.rx = rx; ep.s0 = s0; ep.s2 = s2; ep.act = ACT_NONE; ep.out_scale = 1.f; ep.out_dtype = RWKV_DT_F16;
+    ep.splitk_ws = (float *)((unsigned char *)workspace + xs_bytes + (((size_t)B * 8 + 255) & ~(size_t)255));
+    ep.splitk_bytes = RWKV_SPLITK_WS_BYTES;
     return gemm_launch(true, B, N, M, xs, N, w, w_stride_m, y, y_stride, ep, st);
 }
 

@@ -14,7 +14,12 @@ struct GemmEpi {
     float out_scale;               // applied to the final fp16 value (1 or 0.5)
     int out_dtype;                 // RWKV_DT_F16 / RWKV_DT_F32 (the fp16-rounded value widened)
     int raw_f32;                   // 1: store the fp32 accumulator unrounded (out_dtype must be F32)
+    float *splitk_ws;              // scratch for split-K partial sums (NULL: never split)
+    size_t splitk_bytes;
 };
+
+// Size of the split-K scratch the model-level entry points reserve in their workspaces.
+constexpr size_t RWKV_SPLITK_WS_BYTES = (size_t)64 << 20;
 
 int gemm_launch(bool w_u8, int64_t T, int64_t N, int64_t M, const rwkv_half *A, int64_t lda, const void *W,
                 int64_t ldw, void *Y, int64_t ldy, const GemmEpi &ep, hipStream_t st);

@@ -163,6 +163,7 @@ struct SeqWs {
     rwkv_half *x, *xs[3], *r, *rwkv, *vx, *xsv, *xx_att, *xx_ffn;
     void *k, *v;       // fp16 (uint8 weights) or fp32 (fp16 weights)
     float *sums;       // 8 * T floats
+    float *splitk;     // RWKV_SPLITK_WS_BYTES of split-K scratch for the contraction kernel
     size_t total;
 };
 
@@ -182,12 +183,15 @@ SeqWs carve(void *base, int64_t T, int64_t C, int64_t F) {
     w.xx_att = (rwkv_half *)take((size_t)C * 2);
     w.xx_ffn = (rwkv_half *)take((size_t)C * 2);
     w.sums = (float *)take((size_t)T * 8 * sizeof(float));
+    w.splitk = (float *)take(RWKV_SPLITK_WS_BYTES);
     w.total = (size_t)(p - (unsigned char *)base);
     return w;
 }
 
 int run_gemm(const rwkv_mat &m, bool u8, int64_t T, const rwkv_half *A, const float *s0, const float *s2, void *Y,
-             int64_t ldy, GemmEpi ep, hipStream_t st) {
+             int64_t ldy, GemmEpi ep, hipStream_t st, float *splitk) {
+    ep.splitk_ws = splitk;
+    ep.splitk_bytes = RWKV_SPLITK_WS_BYTES;
     ep.mx = u8 ? m.mx : nullptr;
     ep.rx = u8 ? m.rx : nullptr;
     ep.s0 = s0;
@@ -259,10 +263,10 @@ extern "C" int rwkv_v4_forward_seq(const rwkv_v4_model *m, const rwkv_v4_layer_s
         e.out_scale = 1.f;
         // k, v: uint8 weights return fp16 (widened by the consumer); fp16 weights return fp32 directly
         e.act = ACT_NONE; e.out_dtype = u8 ? RWKV_DT_F16 : RWKV_DT_F32; e.raw_f32 = u8 ? 0 : 1;
-        if ((rc = run_gemm(l.att_key, u8, T, ws.xs[0], s0[0], s2[0], ws.k, C, e, st))) return rc;
-        if ((rc = run_gemm(l.att_value, u8, T, ws.xs[1], s0[1], s2[1], ws.v, C, e, st))) return rc;
+        if ((rc = run_gemm(l.att_key, u8, T, ws.xs[0], s0[0], s2[0], ws.k, C, e, st, ws.splitk))) return rc;
+        if ((rc = run_gemm(l.att_value, u8, T, ws.xs[1], s0[1], s2[1], ws.v, C, e, st, ws.splitk))) return rc;
         e.act = ACT_SIGMOID; e.out_dtype = RWKV_DT_F16; e.raw_f32 = 0;
-        if ((rc = run_gemm(l.att_receptance, u8, T, ws.xs[2], s0[2], s2[2], ws.r, C, e, st))) return rc;
+        if ((rc = run_gemm(l.att_receptance, u8, T, ws.xs[2], s0[2], s2[2], ws.r, C, e, st, ws.splitk))) return rc;
         if ((rc = wkv4_fused_launch((int)T, C, l.time_decay, l.time_first, ws.k, ws.v, u8 ? 0 : 1, ws.r, ws.rwkv, s.aa,
                                     s.bb, s.pp, st)))
             return rc;
@@ -273,7 +277,7 @@ extern "C" int rwkv_v4_forward_seq(const rwkv_v4_model *m, const rwkv_v4_layer_s
             a_out = ws.xs[0];
         }
         e.act = ACT_RESIDUAL; e.res = ws.x; e.ldres = C;
-        if ((rc = run_gemm(l.att_output, u8, T, a_out, s0[0], s2[0], ws.x, C, e, st))) return rc;
+        if ((rc = run_gemm(l.att_output, u8, T, a_out, s0[0], s2[0], ws.x, C, e, st, ws.splitk))) return rc;
         // ---- channel mix
         {
             SeqMixArgs a{};
@@ -292,9 +296,9 @@ extern "C" int rwkv_v4_forward_seq(const rwkv_v4_model *m, const rwkv_v4_layer_s
         e = GemmEpi{};
         e.out_scale = 1.f; e.out_dtype = RWKV_DT_F16;
         e.act = ACT_SIGMOID;
-        if ((rc = run_gemm(l.ffn_receptance, u8, T, ws.xs[0], s0[0], s2[0], ws.r, C, e, st))) return rc;
+        if ((rc = run_gemm(l.ffn_receptance, u8, T, ws.xs[0], s0[0], s2[0], ws.r, C, e, st, ws.splitk))) return rc;
         e.act = ACT_RELU_SQ;
-        if ((rc = run_gemm(l.ffn_key, u8, T, ws.xs[1], s0[1], s2[1], ws.vx, F, e, st))) return rc;
+        if ((rc = run_gemm(l.ffn_key, u8, T, ws.xs[1], s0[1], s2[1], ws.vx, F, e, st, ws.splitk))) return rc;
         const rwkv_half *a_v = ws.vx;
         if (u8) {
             if ((rc = mm8_prepare_launch(T, F, ws.vx, F, l.ffn_value.ry, l.ffn_value.my, ws.xsv, s0v, s2v, st))) return rc;
@@ -302,7 +306,7 @@ extern "C" int rwkv_v4_forward_seq(const rwkv_v4_model *m, const rwkv_v4_layer_s
         }
         e.act = ACT_GATED_RESIDUAL; e.gate = ws.r; e.ldgate = C; e.res = ws.x; e.ldres = C;
         e.out_scale = (m->rescale_layer > 0 && (i + 1) % m->rescale_layer == 0) ? 0.5f : 1.f;
-        if ((rc = run_gemm(l.ffn_value, u8, T, a_v, s0v, s2v, ws.x, C, e, st))) return rc;
+        if ((rc = run_gemm(l.ffn_value, u8, T, a_v, s0v, s2v, ws.x, C, e, st, ws.splitk))) return rc;
         RWKV_LAUNCH_CHECK();
     }
     if (!full_output) return v4_head_launch(m, ws.x + (size_t)(T - 1) * C, logits, st);
@@ -316,7 +320,7 @@ extern "C" int rwkv_v4_forward_seq(const rwkv_v4_model *m, const rwkv_v4_layer_s
     }
     GemmEpi e{};
     e.out_scale = 1.f; e.act = ACT_NONE; e.out_dtype = RWKV_DT_F32;
-    if ((rc = run_gemm(m->head, u8, T, ws.xs[0], s0[0], s2[0], logits, m->vocab, e, st))) return rc;
+    if ((rc = run_gemm(m->head, u8, T, ws.xs[0], s0[0], s2[0], logits, m->vocab, e, st, ws.splitk))) return rc;
     RWKV_LAUNCH_CHECK();
     return RWKV_OK;
 }

@@ -113,6 +113,7 @@ struct Ctx {
     int grid;
     rwkv_half *xs;       // scaled-activation scratch [T, max(C, F)]
     float *s0, *s2;      // [T]
+    float *splitk;       // RWKV_SPLITK_WS_BYTES of split-K scratch
 };
 
 // y = act(x @ W) for a model matrix (uint8 or fp16 per strategy) or an fp16 LoRA matrix.
@@ -147,7 +148,7 @@ int mm(const Ctx &c, const rwkv_mat &m, bool mat_u8, const rwkv_half *x, int act
     const rwkv_half *A = x;
     GemmEpi e{};
     e.act = act; e.res = res; e.ldres = M; e.gate = gate; e.ldgate = M; e.out_scale = out_scale;
-    e.out_dtype = RWKV_DT_F16;
+    e.out_dtype = RWKV_DT_F16; e.splitk_ws = c.splitk; e.splitk_bytes = RWKV_SPLITK_WS_BYTES;
     if (mat_u8) {
         int rc = mm8_prepare_launch(c.T, N, x, N, m.ry, m.my, c.xs, c.s0, c.s2, c.st);
         if (rc) return rc;
@@ -161,7 +162,7 @@ size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
 struct Ws56 {
     rwkv_half *x, *xx, *sxd, *xxx, *t1, *mix[5], *d1, *d2, *r, *k, *v, *g, *att, *vx, *xs, *xx_att, *xx_ffn;
-    float *sums;
+    float *sums, *splitk;
     size_t total;
 };
 
@@ -178,6 +179,7 @@ Ws56 carve56(void *base, int64_t T, int64_t C, int64_t F, int64_t lm, int64_t ld
     w.vx = take(tf); w.xs = take(tf > tc ? tf : tc);
     w.xx_att = take((size_t)C * 2); w.xx_ffn = take((size_t)C * 2);
     w.sums = (float *)take((size_t)T * 2 * sizeof(float));
+    w.splitk = (float *)take(RWKV_SPLITK_WS_BYTES);
     w.total = (size_t)(p - (unsigned char *)base);
     return w;
 }
@@ -251,7 +253,7 @@ extern "C" int rwkv_v56_forward(const rwkv_v56_model *m, const rwkv_v56_layer_st
     const bool u8 = m->weights_u8 != 0, v6 = ver == 60, gated = ver != 50;
     const int lm = m->lora_maa, ld = m->lora_decay;
     Ws56 ws = carve56(workspace, T, C, F, v6 ? lm : 32, v6 ? ld : 64);
-    Ctx c{st, u8, T, num_cu(), ws.xs, ws.sums, ws.sums + T};
+    Ctx c{st, u8, T, num_cu(), ws.xs, ws.sums, ws.sums + T, ws.splitk};
 
     if ((rc = gather_emb_launch(T, C, tokens, m->emb, ws.x, st))) return rc;
     for (int i = 0; i < m->n_layer; ++i) {
@@ -358,7 +360,7 @@ extern "C" int rwkv_v56_forward(const rwkv_v56_model *m, const rwkv_v56_layer_st
     }
     const rwkv_half *A = ws.xx;
     GemmEpi e{};
-    e.out_scale = 1.f; e.act = ACT_NONE; e.out_dtype = RWKV_DT_F32;
+    e.out_scale = 1.f; e.act = ACT_NONE; e.out_dtype = RWKV_DT_F32; e.splitk_ws = ws.splitk; e.splitk_bytes = RWKV_SPLITK_WS_BYTES;
     if (u8) {
         if ((rc = mm8_prepare_launch(TH, C, ws.xx, C, m->head.ry, m->head.my, ws.xs, ws.sums, ws.sums + T, st))) return rc;
         A = ws.xs;
