@@ -29,7 +29,9 @@ int gemv_f16_launch(int64_t N, int64_t M, const rwkv_half *x, const rwkv_half *w
                     int y_dtype, hipStream_t st);
 // kv_f32: k, v are fp32 (fp16-weight strategy) instead of fp16.
 int wkv4_fused_launch(int T, int C, const float *w, const float *u, const void *k, const void *v, int kv_f32,
-                      const rwkv_half *r, rwkv_half *y, float *aa, float *bb, float *pp, hipStream_t st);
+                      const rwkv_half *r, rwkv_half *y, float *aa, float *bb, float *pp, hipStream_t st,
+                      float *scratch = nullptr);  // scratch (wkv4_scratch_bytes): long calls run as a chunked scan
+size_t wkv4_scratch_bytes(int64_t T, int64_t C);
 int wkv56_fused_launch(bool v6, int T, int C, int H, float *state, const rwkv_half *r, const rwkv_half *k,
                        const rwkv_half *v, const void *w, const float *t_decay, const float *u, const float *lnx_w,
                        const float *lnx_b, const rwkv_half *gate, rwkv_half *out, hipStream_t st,

@@ -164,6 +164,7 @@ struct SeqWs {
     void *k, *v;       // fp16 (uint8 weights) or fp32 (fp16 weights)
     float *sums;       // 8 * T floats
     float *splitk;     // RWKV_SPLITK_WS_BYTES of split-K scratch for the contraction kernel
+    float *wkv;        // chunk summaries of the WKV scan
     size_t total;
 };
 
@@ -184,6 +185,7 @@ SeqWs carve(void *base, int64_t T, int64_t C, int64_t F) {
     w.xx_ffn = (rwkv_half *)take((size_t)C * 2);
     w.sums = (float *)take((size_t)T * 8 * sizeof(float));
     w.splitk = (float *)take(RWKV_SPLITK_WS_BYTES);
+    w.wkv = (float *)take(wkv4_scratch_bytes(T, C));
     w.total = (size_t)(p - (unsigned char *)base);
     return w;
 }
@@ -268,7 +270,7 @@ extern "C" int rwkv_v4_forward_seq(const rwkv_v4_model *m, const rwkv_v4_layer_s
         e.act = ACT_SIGMOID; e.out_dtype = RWKV_DT_F16; e.raw_f32 = 0;
         if ((rc = run_gemm(l.att_receptance, u8, T, ws.xs[2], s0[2], s2[2], ws.r, C, e, st, ws.splitk))) return rc;
         if ((rc = wkv4_fused_launch((int)T, C, l.time_decay, l.time_first, ws.k, ws.v, u8 ? 0 : 1, ws.r, ws.rwkv, s.aa,
-                                    s.bb, s.pp, st)))
+                                    s.bb, s.pp, st, ws.wkv)))
             return rc;
         const rwkv_half *a_out = ws.rwkv;
         if (u8) {

@@ -88,6 +88,113 @@ __global__ __launch_bounds__(64) void wkv4_kernel(int T, int C, const float *__r
 }
 
 // ---------------------------------------------------------------------------------------
+// RWKV-4 over a long sequence: the recurrence is a scan with an associative combine, so T is cut into
+// chunks that run in parallel.  A state (a, b, p) stands for the sums A = a e^p, B = b e^p; n steps of
+// decay add n w to p, and two states merge under the larger exponent.
+//   pass 1  (chunk j, channel c): state after the chunk's tokens starting from the empty state
+//   pass 2  (chunk j, channel c): incoming state = fold of the call's initial state and the summaries of
+//           chunks 0..j-1 (decay by one chunk length between them), then the ordinary per-token steps of
+//           the chunk; the last chunk stores the final state.
+// Twice the arithmetic of the sequential kernel on T/L times as many lanes.
+// scratch: (nchunks + 1) x 3 x C floats; slot 0 holds a copy of the initial state (the final state is
+// written over the caller's while other chunks may still read it).
+// ---------------------------------------------------------------------------------------
+DEV void wkv4_merge(float &a, float &b, float &p, float a2, float b2, float p2) {
+    const float q = fmaxf(p, p2);
+    const float e1 = __expf(p - q), e2 = __expf(p2 - q);
+    a = e1 * a + e2 * a2;
+    b = e1 * b + e2 * b2;
+    p = q;
+}
+
+template <int MODE>
+__global__ __launch_bounds__(64) void wkv4_chunk_summary_kernel(int T, int C, int L, const float *__restrict__ w_,
+                                                                Wkv4IO<MODE> io, const float *__restrict__ aa_,
+                                                                const float *__restrict__ bb_, const float *__restrict__ pp_,
+                                                                float *__restrict__ scratch) {
+    constexpr int UNR = 8;
+    const int c = blockIdx.x * 64 + threadIdx.x, j = blockIdx.y;
+    if (c >= C) return;
+    if (j == 0) {
+        scratch[c] = aa_[c]; scratch[C + c] = bb_[c]; scratch[2 * C + c] = pp_[c];
+    }
+    const float w = w_[c];
+    const int t0 = j * L, t1 = min(T, t0 + L);
+    float aa = 0.f, bb = 0.f, pp = -1e38f;
+    auto step = [&](float kk, float vv) {
+        const float ww = w + pp;
+        const float p = fmaxf(ww, kk);
+        const float e1 = __expf(ww - p), e2 = __expf(kk - p);
+        aa = e1 * aa + e2 * vv;
+        bb = e1 * bb + e2;
+        pp = p;
+    };
+    int t = t0;
+    for (; t + UNR <= t1; t += UNR) {
+        float kk[UNR], vv[UNR];
+#pragma unroll
+        for (int i = 0; i < UNR; ++i) {
+            const size_t o = (size_t)(t + i) * C + c;
+            kk[i] = io.ldk(o); vv[i] = io.ldv(o);
+        }
+#pragma unroll
+        for (int i = 0; i < UNR; ++i) step(kk[i], vv[i]);
+    }
+    for (; t < t1; ++t) step(io.ldk((size_t)t * C + c), io.ldv((size_t)t * C + c));
+    float *o = scratch + (size_t)(j + 1) * 3 * C;
+    o[c] = aa; o[C + c] = bb; o[2 * C + c] = pp;
+}
+
+template <int MODE>
+__global__ __launch_bounds__(64) void wkv4_chunk_apply_kernel(int T, int C, int L, const float *__restrict__ w_,
+                                                              const float *__restrict__ u_, Wkv4IO<MODE> io,
+                                                              float *__restrict__ aa_, float *__restrict__ bb_,
+                                                              float *__restrict__ pp_, const float *__restrict__ scratch) {
+    constexpr int UNR = 8;
+    const int c = blockIdx.x * 64 + threadIdx.x, j = blockIdx.y;
+    if (c >= C) return;
+    const float u = u_[c], w = w_[c];
+    const int t0 = j * L, t1 = min(T, t0 + L);
+    float aa = scratch[c], bb = scratch[C + c], pp = scratch[2 * C + c];
+    const float wl = w * (float)L;
+    for (int i = 0; i < j; ++i) {
+        const float *sm = scratch + (size_t)(i + 1) * 3 * C;
+        pp += wl;
+        wkv4_merge(aa, bb, pp, sm[c], sm[C + c], sm[2 * C + c]);
+    }
+    int t = t0;
+    for (; t + UNR <= t1; t += UNR) {
+        float kk[UNR], vv[UNR], rr[UNR];
+#pragma unroll
+        for (int i = 0; i < UNR; ++i) {
+            const size_t o = (size_t)(t + i) * C + c;
+            kk[i] = io.ldk(o); vv[i] = io.ldv(o); rr[i] = io.ldr(o);
+        }
+#pragma unroll
+        for (int i = 0; i < UNR; ++i) {
+            float out;
+            wkv4_step(kk[i], vv[i], u, w, aa, bb, pp, out);
+            io.st((size_t)(t + i) * C + c, out, rr[i]);
+        }
+    }
+    for (; t < t1; ++t) {
+        const size_t o = (size_t)t * C + c;
+        float out;
+        const float rr = io.ldr(o);
+        wkv4_step(io.ldk(o), io.ldv(o), u, w, aa, bb, pp, out);
+        io.st(o, out, rr);
+    }
+    if (t1 == T) { aa_[c] = aa; bb_[c] = bb; pp_[c] = pp; }
+}
+
+// Chunk length for a T-token call: about sqrt(T), a multiple of 8.
+int wkv4_chunk_len(int T) {
+    int L = 16;
+    while (L * L < T && L < 128) L <<= 1;
+    return L;
+}
+
+// ---------------------------------------------------------------------------------------
 // RWKV-5 / RWKV-6.  One workgroup of 256 threads per head (N = 64).  Thread (i, q), i = value
 // index 0..63, q = key quarter 0..3, keeps S[i][16q .. 16q+16) in registers for the whole call.
 // Tokens are processed in slabs of TS: r, k, v, w of the slab are staged in LDS once (one
@@ -230,15 +337,33 @@ extern "C" int rwkv_wkv4_forward(int64_t B, int64_t T, int64_t C, const float *w
 }
 
 // fused variant used by the model path: k, v (fp16 or fp32) and fp16 r in; y = fp16(r * fp16(wkv)).
+size_t wkv4_scratch_bytes(int64_t T, int64_t C) {
+    if (T < 64) return 256;
+    const int L = wkv4_chunk_len((int)T);
+    return (size_t)((T + L - 1) / L + 1) * 3 * (size_t)C * sizeof(float);
+}
+
+template <int MODE>
+static void wkv4_fused_run(int T, int C, const float *w, const float *u, Wkv4IO<MODE> io, float *aa, float *bb, float *pp,
+                           float *scratch, hipStream_t st) {
+    if (T >= 64 && scratch) {
+        const int L = wkv4_chunk_len(T);
+        const dim3 grid((unsigned)((C + 63) / 64), (unsigned)((T + L - 1) / L));
+        hipLaunchKernelGGL(wkv4_chunk_summary_kernel<MODE>, grid, dim3(64), 0, st, T, C, L, w, io, aa, bb, pp, scratch);
+        hipLaunchKernelGGL(wkv4_chunk_apply_kernel<MODE>, grid, dim3(64), 0, st, T, C, L, w, u, io, aa, bb, pp, scratch);
+    } else {
+        hipLaunchKernelGGL(wkv4_kernel<MODE>, dim3((unsigned)((C + 63) / 64), 1), dim3(64), 0, st, T, C, w, u, io, aa, bb, pp);
+    }
+}
+
 int wkv4_fused_launch(int T, int C, const float *w, const float *u, const void *k, const void *v, int kv_f32,
-                      const rwkv_half *r, rwkv_half *y, float *aa, float *bb, float *pp, hipStream_t st) {
-    const dim3 grid((unsigned)((C + 63) / 64), 1);
+                      const rwkv_half *r, rwkv_half *y, float *aa, float *bb, float *pp, hipStream_t st, float *scratch) {
     if (kv_f32) {
         Wkv4IO<2> io{(const float *)k, (const float *)v, y, r};
-        hipLaunchKernelGGL(wkv4_kernel<2>, grid, dim3(64), 0, st, T, C, w, u, io, aa, bb, pp);
+        wkv4_fused_run<2>(T, C, w, u, io, aa, bb, pp, scratch, st);
     } else {
         Wkv4IO<1> io{(const rwkv_half *)k, (const rwkv_half *)v, y, r};
-        hipLaunchKernelGGL(wkv4_kernel<1>, grid, dim3(64), 0, st, T, C, w, u, io, aa, bb, pp);
+        wkv4_fused_run<1>(T, C, w, u, io, aa, bb, pp, scratch, st);
     }
     RWKV_LAUNCH_CHECK();
     return RWKV_OK;

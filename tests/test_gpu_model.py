@@ -98,6 +98,27 @@ def test_tiny_forward_parity(tiny_models, strat):
     assert d_last <= 2e-3, d_last
 
 
+@pytest.mark.parametrize("strat", ["cuda fp16i8", "cuda fp16"])
+@pytest.mark.parametrize("T", [100, 203])
+def test_long_prompt_chunked_scan(tiny_models, strat, T):
+    """Prompts of 64 tokens and more run the RWKV-4 recurrence as a chunked scan (ragged last chunk here);
+    logits and state must match the oracle's token-by-token recurrence, and a second call must pick the
+    state up where the first left it."""
+    m, o = tiny_models[strat]
+    toks = synth.random_tokens(T + 70, TINY["vocab"], seed=PROMPT_SEED + T)
+    full, st = m.forward(toks[:T], None, full_output=True)
+    ofull, ost = o.forward(toks[:T], None, full_output=True)
+    d_full = float(np.abs(_np(full) - ofull).max())
+    assert d_full <= LOGIT_TOL, d_full
+    assert _argmax_agree(_np(full), ofull, d_full)
+    for i, (a, b) in enumerate(zip(st, ost)):
+        np.testing.assert_allclose(_np(a), b.astype(np.float32), rtol=2e-2, atol=2e-2, err_msg=f"state {i}")
+    out, st = m.forward(toks[T:], st)
+    oout, ost = o.forward(toks[T:], ost)
+    d = float(np.abs(_np(out) - oout).max())
+    assert d <= LOGIT_TOL, d
+
+
 def test_state_contract(tiny_models):
     m, _ = tiny_models["cuda fp16i8"]
     C, L = TINY["n_embd"], TINY["n_layer"]
