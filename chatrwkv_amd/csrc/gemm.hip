@@ -193,23 +193,23 @@ __global__ __launch_bounds__(256) void gemm_kernel(int T, int N, int M, const h1
                     acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[a], fb[b], acc[a][b], 0, 0, 0);
         }
     };
-    // tile kt lives in register slot kt % PF from PF iterations before it is multiplied until it
-    // is written to LDS buffer kt & 1 at the end of iteration kt - 1
+    // Tile kt lives in register slot kt % PF from PF iterations before it is multiplied until it is written
+    // to LDS buffer kt & 1 at the end of iteration kt - 1.  Every global load is issued unconditionally (past
+    // the end the last k-tile is read again and never used): the compiler places its waits from a static
+    // count of the loads issued after the one it needs, and a load under a branch would make it assume the
+    // fewest, i.e. drain the whole prefetch queue before every LDS store.
 #pragma unroll
-    for (int p = 0; p < PF; ++p)
-        if (p < nk) load_tiles(ra[p], rb[p], p);
+    for (int p = 0; p < PF; ++p) load_tiles(ra[p], rb[p], min(p, nk - 1));
     store_tiles(ra[0], rb[0], 0);
     __syncthreads();
     for (int kt0 = 0; kt0 < nk; kt0 += PF) {
 #pragma unroll
         for (int p = 0; p < PF; ++p) {
             const int kt = kt0 + p;
-            if (kt < nk) {
-                if (kt + PF < nk) load_tiles(ra[p], rb[p], kt + PF);  // slot freed when tile kt went to LDS
-                compute(kt & 1);
-                if (kt + 1 < nk) store_tiles(ra[(p + 1) % PF], rb[(p + 1) % PF], (kt + 1) & 1);
-                __syncthreads();
-            }
+            load_tiles(ra[p], rb[p], min(kt + PF, nk - 1));  // slot freed when tile kt went to LDS
+            if (kt < nk) compute(kt & 1);
+            if (kt + 1 < nk) store_tiles(ra[(p + 1) % PF], rb[(p + 1) % PF], (kt + 1) & 1);
+            __syncthreads();
         }
     }
 

@@ -201,6 +201,45 @@ int run_gemm(const rwkv_mat &m, bool u8, int64_t T, const rwkv_half *A, const fl
     return gemm_launch(u8, T, m.N, m.M, A, m.N, m.w, m.ld, Y, ldy, ep, st);
 }
 
+// Two side streams (default priority) for contractions that are independent of each other and too small
+// to fill the chip alone: k / v / r of the time mix and r / k of the channel mix run side by side.
+struct SideStreams {
+    hipStream_t s[2];
+    hipEvent_t fork, join[2];
+    bool ok;
+};
+
+SideStreams *side_streams() {
+    static SideStreams ss{};
+    static bool tried = false;
+    if (!tried) {
+        tried = true;
+        ss.ok = hipStreamCreateWithFlags(&ss.s[0], hipStreamNonBlocking) == hipSuccess &&
+                hipStreamCreateWithFlags(&ss.s[1], hipStreamNonBlocking) == hipSuccess &&
+                hipEventCreateWithFlags(&ss.fork, hipEventDisableTiming) == hipSuccess &&
+                hipEventCreateWithFlags(&ss.join[0], hipEventDisableTiming) == hipSuccess &&
+                hipEventCreateWithFlags(&ss.join[1], hipEventDisableTiming) == hipSuccess;
+    }
+    return ss.ok ? &ss : nullptr;
+}
+
+// after fork, work launched on side stream j sees everything queued on `st` so far
+bool fork_streams(SideStreams *ss, hipStream_t st, int n) {
+    if (hipEventRecord(ss->fork, st) != hipSuccess) return false;
+    for (int j = 0; j < n; ++j)
+        if (hipStreamWaitEvent(ss->s[j], ss->fork, 0) != hipSuccess) return false;
+    return true;
+}
+
+// after join, work launched on `st` sees everything queued on the side streams
+bool join_streams(SideStreams *ss, hipStream_t st, int n) {
+    for (int j = 0; j < n; ++j) {
+        if (hipEventRecord(ss->join[j], ss->s[j]) != hipSuccess) return false;
+        if (hipStreamWaitEvent(st, ss->join[j], 0) != hipSuccess) return false;
+    }
+    return true;
+}
+
 }  // namespace
 
 extern "C" int rwkv_layernorm_f32_f16(int64_t T, int64_t C, const float *x, const float *w, const float *b,
@@ -242,6 +281,7 @@ extern "C" int rwkv_v4_forward_seq(const rwkv_v4_model *m, const rwkv_v4_layer_s
     const int n16 = C >> 3;
 
     hipLaunchKernelGGL(gather_emb_kernel, dim3((unsigned)T), dim3(256), 0, st, (int)T, C, tokens, m->emb, ws.x);
+    SideStreams *ss = T >= 256 ? side_streams() : nullptr;
 
     for (int i = 0; i < m->n_layer; ++i) {
         const rwkv_v4_layer &l = m->layers[i];
@@ -265,10 +305,14 @@ extern "C" int rwkv_v4_forward_seq(const rwkv_v4_model *m, const rwkv_v4_layer_s
         e.out_scale = 1.f;
         // k, v: uint8 weights return fp16 (widened by the consumer); fp16 weights return fp32 directly
         e.act = ACT_NONE; e.out_dtype = u8 ? RWKV_DT_F16 : RWKV_DT_F32; e.raw_f32 = u8 ? 0 : 1;
+        // side by side when none of them would split K (the split-K scratch is shared)
+        const bool par = ss && (T / 128) * (C / 128) > 128 && fork_streams(ss, st, 2);
+        hipStream_t sv = par ? ss->s[0] : st, sr = par ? ss->s[1] : st;
         if ((rc = run_gemm(l.att_key, u8, T, ws.xs[0], s0[0], s2[0], ws.k, C, e, st, ws.splitk))) return rc;
-        if ((rc = run_gemm(l.att_value, u8, T, ws.xs[1], s0[1], s2[1], ws.v, C, e, st, ws.splitk))) return rc;
+        if ((rc = run_gemm(l.att_value, u8, T, ws.xs[1], s0[1], s2[1], ws.v, C, e, sv, ws.splitk))) return rc;
         e.act = ACT_SIGMOID; e.out_dtype = RWKV_DT_F16; e.raw_f32 = 0;
-        if ((rc = run_gemm(l.att_receptance, u8, T, ws.xs[2], s0[2], s2[2], ws.r, C, e, st, ws.splitk))) return rc;
+        if ((rc = run_gemm(l.att_receptance, u8, T, ws.xs[2], s0[2], s2[2], ws.r, C, e, sr, ws.splitk))) return rc;
+        if (par && !join_streams(ss, st, 2)) return (int)hipErrorUnknown;
         if ((rc = wkv4_fused_launch((int)T, C, l.time_decay, l.time_first, ws.k, ws.v, u8 ? 0 : 1, ws.r, ws.rwkv, s.aa,
                                     s.bb, s.pp, st, ws.wkv)))
             return rc;
@@ -298,9 +342,11 @@ extern "C" int rwkv_v4_forward_seq(const rwkv_v4_model *m, const rwkv_v4_layer_s
         e = GemmEpi{};
         e.out_scale = 1.f; e.out_dtype = RWKV_DT_F16;
         e.act = ACT_SIGMOID;
-        if ((rc = run_gemm(l.ffn_receptance, u8, T, ws.xs[0], s0[0], s2[0], ws.r, C, e, st, ws.splitk))) return rc;
+        const bool par2 = ss && (T / 128) * (C / 128) > 128 && fork_streams(ss, st, 1);
+        if ((rc = run_gemm(l.ffn_receptance, u8, T, ws.xs[0], s0[0], s2[0], ws.r, C, e, par2 ? ss->s[0] : st, ws.splitk))) return rc;
         e.act = ACT_RELU_SQ;
         if ((rc = run_gemm(l.ffn_key, u8, T, ws.xs[1], s0[1], s2[1], ws.vx, F, e, st, ws.splitk))) return rc;
+        if (par2 && !join_streams(ss, st, 1)) return (int)hipErrorUnknown;
         const rwkv_half *a_v = ws.vx;
         if (u8) {
             if ((rc = mm8_prepare_launch(T, F, ws.vx, F, l.ffn_value.ry, l.ffn_value.my, ws.xsv, s0v, s2v, st))) return rc;
