@@ -32,8 +32,8 @@ if ROOT not in sys.path:
 HBM_PEAK = 8.0e12      # bytes/s, MI355X HBM3E
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by a 1 GiB copy
 # kernel: x2.0 / x1.0); profiles/decode_7b_fp16i8_hbm_traffic.md has the commands and the table
-MEASURED_TRAFFIC = {("v4-7b", "cuda fp16i8", 32, "ffn_rk"): 84873421 + 49152,
-                    ("v4-7b", "cuda fp16i8", 32, "att_kvr_wkv"): 51738829 + 65536}
+MEASURED_TRAFFIC = {("v4-7b", "cuda fp16i8", 32, "ffn_rk"): 85068800 + 49254,
+                    ("v4-7b", "cuda fp16i8", 32, "att_kvr_wkv"): 52143309 + 65536}
 MFMA_F16_PEAK = 2.5e15  # flop/s dense fp16
 
 
