@@ -201,9 +201,9 @@ DEV void stream_rows(int ngroups, int nseg, bool pro_wave, ProLoad pro_load, Pro
     // the wave index through readfirstlane: the compiler then knows that everything derived from it (row
     // ranges, batch counters, loop control) is wave-uniform and keeps it in scalar registers
     const int wave = blockIdx.x * DWAVES + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), nwaves = gridDim.x * DWAVES;
-    const int per = (ngroups + nwaves - 1) / nwaves;
-    const int g0 = min(wave * per, ngroups), g1 = min(g0 + per, ngroups);
-    const int glast = max(g1 - 1, 0);
+    // balanced split: every wave gets floor or ceil of ngroups / nwaves groups
+    const int g0 = (int)((int64_t)wave * ngroups / nwaves), g1 = (int)((int64_t)(wave + 1) * ngroups / nwaves);
+    const int glast = g1 > g0 ? g1 - 1 : min(g0, ngroups - 1);
     const int nsb = (nseg + 64 * U - 1) / (64 * U);             // segment batches per group batch
     const int nb = ((g1 - g0 + G - 1) / G) * nsb;               // batches of this wave
     const int sb_epi = nsb > 1 ? 1 : 0;                         // segment batch that carries the epilogue operands
