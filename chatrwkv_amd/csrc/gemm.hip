@@ -215,20 +215,21 @@ __global__ __launch_bounds__(256) void gemm_kernel(int T, int N, int M, const h1
 
     // epilogue: lane holds column m = .. + (lane & 31) and rows 8*(e/4) + 4*(lane>>5) + e%4
     float *slab = SPLIT ? part + (size_t)blockIdx.y * T * M : nullptr;
-#pragma unroll
+#pragma clang loop unroll(full)
     for (int b = 0; b < NI; ++b) {
         const int m = m0 + wc * (BM / WM) + b * 32 + (lane & 31);
-        if (m >= M) continue;
+        const bool m_ok = m < M;
         float rxm = 1.f, mxm = 0.f;
-        if (!SPLIT && ep.rx) { rxm = h2f(ep.rx[m]); mxm = h2f(ep.mx[m]); }
-#pragma unroll
+        if (!SPLIT && ep.rx && m_ok) { rxm = h2f(ep.rx[m]); mxm = h2f(ep.mx[m]); }
+#pragma clang loop unroll(full)
         for (int a = 0; a < MI; ++a) {
-#pragma unroll
+#pragma clang loop unroll(full)
             for (int e = 0; e < 16; ++e) {
                 const int t = t0 + wr * (BT / WT) + a * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
-                if (t >= T) continue;
-                if (SPLIT) slab[(size_t)t * M + m] = acc[a][b][e];
-                else gemm_epilogue(acc[a][b][e], t, m, rxm, mxm, ep, Y, ldy);
+                if (m_ok && t < T) {
+                    if (SPLIT) slab[(size_t)t * M + m] = acc[a][b][e];
+                    else gemm_epilogue(acc[a][b][e], t, m, rxm, mxm, ep, Y, ldy);
+                }
             }
         }
     }

@@ -91,6 +91,8 @@ SIGNATURES.update({
     "rwkv_v56_workspace": (_sz, [ctypes.POINTER(RwkvV56Model), _i64]),
     "rwkv_v56_forward": (_int, [ctypes.POINTER(RwkvV56Model), ctypes.POINTER(RwkvV56LayerState), _vp, _i64, _int, _vp, _vp, _sz, _vp]),
     "rwkv_layernorm_f32_f16": (_int, [_i64, _i64, _vp, _vp, _vp, _vp, _vp]),
+    "rwkv_sample_logits": (_int, [_vp, _i64, ctypes.c_float, ctypes.c_float, ctypes.c_int32, _vp, ctypes.c_int32, _vp, _vp, _vp,
+                                  ctypes.c_float, ctypes.c_float, ctypes.c_float, _vp, _vp, _vp, _vp]),
     "rwkv_v4_one_workspace": (_sz, [ctypes.POINTER(RwkvV4Model)]),
     "rwkv_v4_forward_one": (_int, [ctypes.POINTER(RwkvV4Model), ctypes.POINTER(RwkvV4LayerState), _vp, _vp, _vp, _sz, _vp]),
     "rwkv_v4_profile_one": (_int, [ctypes.POINTER(RwkvV4Model), ctypes.POINTER(RwkvV4LayerState), _vp, _vp, _vp, _sz, _vp, _vp, _i64]),

@@ -129,6 +129,25 @@ int rwkv_wkv6_forward(int64_t B, int64_t T, int64_t C, int64_t H, float *state, 
 int rwkv_layernorm_f32_f16(int64_t T, int64_t C, const float *x, const float *w, const float *b,
                            rwkv_half *y, void *stream);
 
+/* Sampling step after the head, on the device: replaces PIPELINE.sample_logits (rwkv/utils.py:55-88) and the
+ * logit adjustments / occurrence bookkeeping of PIPELINE.generate (utils.py:103-106, 112-123).
+ *   logits [V] fp32 (V <= 65536), not modified.
+ *   token_ban [n_ban] int32 ids set to -inf (may be NULL when n_ban == 0).
+ *   seen [V] uint8 / occurrence [V] fp32: the reference's `occurrence` dict as dense tables (both NULL: no
+ *     penalties); every seen id pays alpha_presence + occurrence * alpha_frequency; after the draw all seen
+ *     entries are multiplied by alpha_decay and the drawn id gets token_weight[id] (1 when token_weight is
+ *     NULL; the reference uses 0 for ids that decode to blanks or digits) added / set and is marked seen.
+ *   temperature 0 selects top_p 0 (the largest probability alone), as in the reference.
+ *   u: device pointer to one uniform number in [0, 1): the draw is the first index, in index order, whose
+ *     running sum of the filtered probabilities exceeds u * total.
+ *   probs [V] fp32 or NULL: the filtered, temperature-scaled, un-normalised probabilities (what the
+ *     reference hands to torch.multinomial).
+ *   token: device int32, the drawn id.  One launch, no host synchronisation. */
+int rwkv_sample_logits(const float *logits, int64_t V, float temperature, float top_p, int32_t top_k,
+                       const int32_t *token_ban, int32_t n_ban, uint8_t *seen, float *occurrence,
+                       const float *token_weight, float alpha_presence, float alpha_frequency, float alpha_decay,
+                       const float *u, float *probs, int32_t *token, void *stream);
+
 /* =======================================================================================
  * Model-level entry points: one call runs RWKV.forward (model.py:1443-1677) for RWKV-4 on
  * one GPU, with the elementwise chains of att_one / ffn_one / cuda_att_seq / ffn_seq

@@ -12,8 +12,11 @@ Modules
   quant.py   uint8 quantizer + dequantisation          (model.py:818-847, 91-97)
   ops.py     LayerNorm/GroupNorm, mm8, WKV v4/v5/v6     (model.py:984-1340, cuda/*.cu)
   model.py   checkpoint conversion + forward            (model.py:613-903, 1443-1677)
+  sampling.py  sampling step after the path           (utils.py:55-88, 103-123)
 
 How each function is pinned (what a wrong sign / index / dropped term would trip):
+  sampling.*           the reference's own draws for seeded numpy generators
+                       (tests/golden/sampler.npz) + hand-worked cuts, ties, penalties.
   quantize_u8          golden vectors written by the reference's own loader
                        (tests/golden/quant_*.npz) + invariants (0 and 255 in
                        every row and column, reconstruction bound).
