@@ -59,16 +59,21 @@ DEV void gemm_epilogue(float v, int t, int m, float rxm, float mxm, const GemmEp
 }
 
 // Split-K second pass: sums the KS partial slabs [KS][T][M] in slab order (deterministic) and runs the epilogue.
+// Four consecutive outputs per thread (M % 4 == 0).
 __global__ __launch_bounds__(256) void splitk_epilogue_kernel(int T, int M, int KS, const float *__restrict__ part, void *Y,
                                                               int64_t ldy, GemmEpi ep) {
-    const int64_t n = (int64_t)T * M;
-    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
-        const int t = (int)(i / M), m = (int)(i - (int64_t)t * M);
-        float v = 0.f;
-        for (int k = 0; k < KS; ++k) v += part[(size_t)k * n + i];
-        float rxm = 1.f, mxm = 0.f;
-        if (ep.rx) { rxm = h2f(ep.rx[m]); mxm = h2f(ep.mx[m]); }
-        gemm_epilogue(v, t, m, rxm, mxm, ep, Y, ldy);
+    const int64_t n4 = (int64_t)T * M / 4, n = (int64_t)T * M;
+    const int m4 = M / 4;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n4; i += (int64_t)gridDim.x * 256) {
+        const int t = (int)(i / m4), m = (int)(i - (int64_t)t * m4) * 4;
+        f32x4 v = *(const f32x4 *)(part + 4 * i);
+        for (int k = 1; k < KS; ++k) v += *(const f32x4 *)(part + (size_t)k * n + 4 * i);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            float rxm = 1.f, mxm = 0.f;
+            if (ep.rx) { rxm = h2f(ep.rx[m + e]); mxm = h2f(ep.mx[m + e]); }
+            gemm_epilogue(v[e], t, m + e, rxm, mxm, ep, Y, ldy);
+        }
     }
 }
 
@@ -285,20 +290,20 @@ int launch_cfg(int64_t T, int64_t N, int64_t M, const rwkv_half *A, int64_t lda,
     // workgroups per tile; partial sums go to fp32 slabs and a second pass reduces them in slab order.
     int ks = 1;
     const int nk = (int)(N / BK);
-    if (ep.splitk_ws && tiles <= 128 && lds <= 64 * 1024) {
-        for (int c = 8; c >= 2; c >>= 1) {
-            if (nk % c || nk / c < 8) continue;                                   // whole k-tiles, several per split
-            if (tiles * c > 512) continue;                                        // two workgroups per CU are enough
-            if ((size_t)c * T * M * sizeof(float) > ep.splitk_bytes) continue;    // slabs must fit
+    if (ep.splitk_ws && tiles <= 128 && lds <= 64 * 1024 && (M & 3) == 0) {
+        // the smallest split that gives every CU a workgroup (slab traffic grows with the split)
+        for (int c = 2; c <= 8; c <<= 1) {
+            if (nk % c || nk / c < 8) break;                                      // whole k-tiles, several per split
+            if ((size_t)c * T * M * sizeof(float) > ep.splitk_bytes) break;       // slabs must fit
             ks = c;
-            break;
+            if (tiles * c >= 256) break;
         }
     }
     if (ks > 1) {
         hipLaunchKernelGGL((gemm_kernel<W_U8, BT, BM, WT, WM, PF, true>), dim3((unsigned)tiles, (unsigned)ks), dim3(256), lds, st,
                            (int)T, (int)N, (int)M, (const h16 *)A, lda, W, ldw, Y, ldy, ep, nk / ks, ep.splitk_ws);
         const int64_t n = T * M;
-        const unsigned blocks = (unsigned)((n + 1023) / 1024 < 4096 ? (n + 1023) / 1024 : 4096);
+        const unsigned blocks = (unsigned)((n + 1023) / 1024 < 2048 ? (n + 1023) / 1024 : 2048);
         hipLaunchKernelGGL(splitk_epilogue_kernel, dim3(blocks), dim3(256), 0, st, (int)T, (int)M, ks, ep.splitk_ws, Y, ldy, ep);
     } else {
         hipLaunchKernelGGL((gemm_kernel<W_U8, BT, BM, WT, WM, PF, false>), dim3((unsigned)tiles), dim3(256), lds, st, (int)T,

@@ -79,29 +79,46 @@ struct Mix2Args {
     rwkv_half *out[5];               // [T, C] each
 };
 
-// grid (T, C/256, 5): m_j[c] = sum_i t1[t, jR + i] * w2[j][i][c]; out_j = xx + sxd * (maa_j + m_j).
-// One (channel, mix) per thread; the rank loop loads 16 coefficients before it adds them (in index order).
+// grid (ceil(T / 16), C/256, 5): m_j[c] = sum_i t1[t, jR + i] * w2[j][i][c]; out_j = xx + sxd * (maa_j + m_j).
+// One (channel, mix) per thread for a tile of 16 tokens: the R coefficients of the channel are loaded once
+// and reused for every token of the tile; the sum runs in index order.
+constexpr int MIX2_TT = 16;
 __global__ __launch_bounds__(256) void v6_mix2_kernel(Mix2Args a) {
-    __shared__ float st1[64];
-    const int t = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x, j = blockIdx.z, R = a.R, C = a.C;
-    for (int i = threadIdx.x; i < R; i += 256) st1[i] = h2f(a.t1[(size_t)t * 5 * R + j * R + i]);
+    __shared__ float st1[MIX2_TT][64];
+    const int t0 = blockIdx.x * MIX2_TT, c = blockIdx.y * 256 + threadIdx.x, j = blockIdx.z, R = a.R, C = a.C;
+    const int nt = min(MIX2_TT, a.T - t0);
+    for (int i = threadIdx.x; i < nt * R; i += 256) {
+        const int tt = i / R, r = i - tt * R;
+        st1[tt][r] = h2f(a.t1[(size_t)(t0 + tt) * 5 * R + j * R + r]);
+    }
     __syncthreads();
     if (c >= C) return;
-    const float xx = h2f(a.xx[(size_t)t * C + c]);
-    const float sd = a.sxd ? h2f(a.sxd[(size_t)t * C + c]) : round_h(h2f(a.prev[c]) - xx);
     const rwkv_half maa = a.maa[j][c];
     const rwkv_half *w = a.w2 + (size_t)j * R * C + c;
-    float m = 0.f;
+    float m[MIX2_TT];
+#pragma unroll
+    for (int tt = 0; tt < MIX2_TT; ++tt) m[tt] = 0.f;
     for (int i0 = 0; i0 < R; i0 += 16) {
         rwkv_half wv[16];
 #pragma unroll
         for (int i = 0; i < 16; ++i) wv[i] = w[(size_t)min(i0 + i, R - 1) * C];
 #pragma unroll
         for (int i = 0; i < 16; ++i)
-            if (i0 + i < R) m += st1[i0 + i] * h2f(wv[i]);
+            if (i0 + i < R) {
+                const float wf = h2f(wv[i]);
+#pragma unroll
+                for (int tt = 0; tt < MIX2_TT; ++tt) m[tt] += st1[tt][i0 + i] * wf;
+            }
     }
-    const float mm = round_h(h2f(maa) + round_h(m));
-    a.out[j][(size_t)t * C + c] = f2h(xx + round_h(sd * mm));
+#pragma unroll
+    for (int tt = 0; tt < MIX2_TT; ++tt) {
+        if (tt >= nt) break;
+        const int t = t0 + tt;
+        const float xx = h2f(a.xx[(size_t)t * C + c]);
+        const float sd = a.sxd ? h2f(a.sxd[(size_t)t * C + c]) : round_h(h2f(a.prev[c]) - xx);
+        const float mm = round_h(h2f(maa) + round_h(m[tt]));
+        a.out[j][(size_t)t * C + c] = f2h(xx + round_h(sd * mm));
+    }
 }
 
 MatDev to_dev56(const rwkv_mat &m) { return MatDev{m.w, m.ld, m.mx, m.rx, m.my, m.ry}; }
@@ -278,7 +295,7 @@ extern "C" int rwkv_v56_forward(const rwkv_v56_model *m, const rwkv_v56_layer_st
             }
             b.T = (int)T; b.C = C; b.R = lm; b.t1 = ws.t1; b.w2 = l.tm_w2;
             for (int j = 0; j < 5; ++j) { b.maa[j] = l.att_mix[1 + j]; b.out[j] = ws.mix[j]; }
-            hipLaunchKernelGGL(v6_mix2_kernel, dim3((unsigned)T, (unsigned)((C + 255) / 256), 5), dim3(256), 0, st, b);
+            hipLaunchKernelGGL(v6_mix2_kernel, dim3((unsigned)((T + MIX2_TT - 1) / MIX2_TT), (unsigned)((C + 255) / 256), 5), dim3(256), 0, st, b);
             wx = ws.mix[0]; kx = ws.mix[1]; vx = ws.mix[2]; rx = ws.mix[3]; gx = ws.mix[4];
             if ((rc = mm(c, lora_mat(l.td_w1, C, ld), false, wx, ACT_TANH, nullptr, nullptr, 1.f, ws.d1))) return rc;
             if (T > 1 && (rc = mm(c, lora_mat(l.td_w2, ld, C), false, ws.d1, ACT_NONE, nullptr, nullptr, 1.f, ws.d2))) return rc;
