@@ -35,7 +35,8 @@ size_t wkv4_scratch_bytes(int64_t T, int64_t C);
 int wkv56_fused_launch(bool v6, int T, int C, int H, float *state, const rwkv_half *r, const rwkv_half *k,
                        const rwkv_half *v, const void *w, const float *t_decay, const float *u, const float *lnx_w,
                        const float *lnx_b, const rwkv_half *gate, rwkv_half *out, hipStream_t st,
-                       const rwkv_half *dw2 = nullptr, int ld = 0);  // dw2: v6 with w = tanh(. @ D1), product with D2 in-kernel
+                       const rwkv_half *dw2 = nullptr, int ld = 0,  // dw2: v6 with w = tanh(. @ D1), product with D2 in-kernel
+                       float *y32 = nullptr);  // fp32 [T, C] scratch: calls of >= 32 tokens split each head over 4 workgroups
 // Row-wise LayerNorm + token shift + mixes for up to 4 consumers over a [T, C] activation (seq_v4.hip).
 struct SeqMixArgs {
     int T, C;

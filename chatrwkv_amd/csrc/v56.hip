@@ -179,7 +179,7 @@ size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
 struct Ws56 {
     rwkv_half *x, *xx, *sxd, *xxx, *t1, *mix[5], *d1, *d2, *r, *k, *v, *g, *att, *vx, *xs, *xx_att, *xx_ffn;
-    float *sums, *splitk;
+    float *sums, *splitk, *y32;
     size_t total;
 };
 
@@ -197,6 +197,7 @@ Ws56 carve56(void *base, int64_t T, int64_t C, int64_t F, int64_t lm, int64_t ld
     w.xx_att = take((size_t)C * 2); w.xx_ffn = take((size_t)C * 2);
     w.sums = (float *)take((size_t)T * 2 * sizeof(float));
     w.splitk = (float *)take(RWKV_SPLITK_WS_BYTES);
+    w.y32 = (float *)take(T >= 32 ? (size_t)T * C * 4 : 256);
     w.total = (size_t)(p - (unsigned char *)base);
     return w;
 }
@@ -330,7 +331,7 @@ extern "C" int rwkv_v56_forward(const rwkv_v56_model *m, const rwkv_v56_layer_st
         if ((rc = wkv56_fused_launch(v6, (int)T, C, H, s.att_kv, ws.r, ws.k, ws.v,
                                      v6 ? (const void *)(d2_fused ? ws.d1 : ws.d2) : (const void *)l.time_decay, l.time_decay,
                                      l.time_first, l.lnx_w, l.lnx_b, gated ? ws.g : nullptr, ws.att, st,
-                                     d2_fused ? l.td_w2 : nullptr, ld)))
+                                     d2_fused ? l.td_w2 : nullptr, ld, ws.y32)))
             return rc;
         if ((rc = mm(c, l.att_output, u8, ws.att, ACT_RESIDUAL, ws.x, nullptr, 1.f, ws.x))) return rc;
         // ---- channel mix

@@ -337,6 +337,95 @@ extern "C" int rwkv_wkv4_forward(int64_t B, int64_t T, int64_t C, const float *w
 }
 
 // fused variant used by the model path: k, v (fp16 or fp32) and fp16 r in; y = fp16(r * fp16(wkv)).
+// ---------------------------------------------------------------------------------------
+// RWKV-5 / RWKV-6 over a sequence, model path.  A head's 64 value columns never interact (y_i and the
+// column S[:, i] depend on v_i only), so a head is split over four workgroups of 16 value columns: 4 H
+// workgroups instead of H.  Thread (value i, key group g): lane & 15 = g owns keys 4g..4g+3 of column i,
+// lane >> 4 and the wave index give i.  The sum over the 16 key groups of a value is a DPP row sum in
+// registers, so the token loop has no barrier and no LDS partials; r, k, w of a slab of tokens are staged
+// in LDS once (two barriers per slab).  Raw y goes to an fp32 [T, C] scratch; GroupNorm and the gate need
+// the whole head and run in wkv56_gn_kernel.
+//   WMODE 0: w[C] fp32 constant decay (RWKV-5);  WMODE 2: fp16 LoRA output [T, C] + t_decay (RWKV-6)
+// ---------------------------------------------------------------------------------------
+constexpr int TS2 = 32;  // tokens per slab
+
+template <int WMODE>
+__global__ __launch_bounds__(256) void wkv56_split_kernel(Wkv56Args a) {
+    __shared__ __align__(16) float sr[TS2][HS], sk[TS2][HS], sw[TS2][HS];
+    __shared__ float sv[TS2][16];
+    const int T = a.T, C = a.C;
+    const int h = blockIdx.x >> 2, vb = blockIdx.x & 3;
+    const int lane = threadIdx.x & 63, g = lane & 15;
+    const int il = (threadIdx.x >> 6) * 4 + (lane >> 4);   // value column within the block of 16
+    const int i = vb * 16 + il;
+    float *S = a.state + (size_t)h * HS * HS;               // [key][value]
+    float s[4], u4[4], wc[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const int j = 4 * g + e;
+        s[e] = S[j * HS + i];
+        u4[e] = a.u[h * HS + j];
+        wc[e] = WMODE == 0 ? ((const float *)a.w)[h * HS + j] : 0.f;
+    }
+    const float tdec = WMODE == 2 ? a.t_decay[h * HS + (threadIdx.x & 63)] : 0.f;
+    for (int t0 = 0; t0 < T; t0 += TS2) {
+        const int nt = min(TS2, T - t0);
+        __syncthreads();  // previous slab fully consumed
+        for (int e = threadIdx.x; e < nt * HS; e += 256) {
+            const int tt = e >> 6, c = e & 63;               // c == threadIdx.x & 63
+            const size_t o = (size_t)(t0 + tt) * C + h * HS + c;
+            sr[tt][c] = h2f(((const rwkv_half *)a.r)[o]);
+            sk[tt][c] = h2f(((const rwkv_half *)a.k)[o]);
+            if (WMODE == 2) sw[tt][c] = expf(-expf(tdec + h2f(((const rwkv_half *)a.w)[o])));
+        }
+        for (int e = threadIdx.x; e < nt * 16; e += 256) {
+            const int tt = e >> 4, c = e & 15;
+            sv[tt][c] = h2f(((const rwkv_half *)a.v)[(size_t)(t0 + tt) * C + h * HS + vb * 16 + c]);
+        }
+        __syncthreads();
+        for (int tt = 0; tt < nt; ++tt) {
+            const float vi = sv[tt][il];
+            const f32x4 r4 = *(const f32x4 *)&sr[tt][4 * g];
+            const f32x4 k4 = *(const f32x4 *)&sk[tt][4 * g];
+            f32x4 w4;
+            if (WMODE == 2) w4 = *(const f32x4 *)&sw[tt][4 * g];
+            float y = 0.f;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const float x = k4[e] * vi;
+                y += r4[e] * (u4[e] * x + s[e]);
+                s[e] = s[e] * (WMODE == 2 ? w4[e] : wc[e]) + x;
+            }
+            y = row16_sum(y);
+            if (g == 0) a.y[(size_t)(t0 + tt) * C + h * HS + i] = y;
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) S[(4 * g + e) * HS + i] = s[e];
+}
+
+// GroupNorm over each head's 64 outputs (eps 64e-5), affine, fp16 rounding, gate: one wave per (token, head).
+__global__ __launch_bounds__(256) void wkv56_gn_kernel(int T, int C, const float *__restrict__ y,
+                                                       const float *__restrict__ lnx_w, const float *__restrict__ lnx_b,
+                                                       const rwkv_half *__restrict__ gate, rwkv_half *__restrict__ out) {
+    const int H = C / HS;
+    const int64_t wave = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (wave >= (int64_t)T * H) return;
+    const int c = threadIdx.x & 63;
+    const int64_t t = wave / H;
+    const int h = (int)(wave - t * H);
+    const size_t o = (size_t)t * C + h * HS + c;
+    const float v = y[o];
+    const float mean = wave_sum(v) * (1.f / HS);
+    const float d = v - mean;
+    const float var = wave_sum(d * d) * (1.f / HS);
+    float gq = d * rsqrtf(var + 64e-5f) * lnx_w[h * HS + c] + lnx_b[h * HS + c];
+    gq = round_h(gq);
+    if (gate) gq = gq * h2f(gate[o]);
+    out[o] = f2h(gq);
+}
+
+
 size_t wkv4_scratch_bytes(int64_t T, int64_t C) {
     if (T < 64) return 256;
     const int L = wkv4_chunk_len((int)T);
@@ -391,13 +480,21 @@ static int wkv56_launch(bool v6, int64_t B, int64_t T, int64_t C, int64_t H, flo
 int wkv56_fused_launch(bool v6, int T, int C, int H, float *state, const rwkv_half *r, const rwkv_half *k,
                        const rwkv_half *v, const void *w, const float *t_decay, const float *u, const float *lnx_w,
                        const float *lnx_b, const rwkv_half *gate, rwkv_half *out, hipStream_t st,
-                       const rwkv_half *dw2, int ld) {
+                       const rwkv_half *dw2, int ld, float *y32) {
     if (C != H * HS) return RWKV_E_SHAPE;
     Wkv56Args a{};
     a.T = T; a.C = C; a.state = state; a.state_layout = 1;
     a.r = r; a.k = k; a.v = v; a.w = w; a.u = u; a.t_decay = t_decay;
     a.lnx_w = lnx_w; a.lnx_b = lnx_b; a.gate = gate; a.out = out; a.dw2 = dw2; a.ld = ld;
-    if (v6 && dw2) {
+    if (T >= 32 && y32) {
+        // long call: four workgroups per head, raw y to the fp32 scratch, GroupNorm + gate in a second launch
+        a.y = y32;
+        if (v6) hipLaunchKernelGGL((wkv56_split_kernel<2>), dim3((unsigned)(4 * H)), dim3(256), 0, st, a);
+        else hipLaunchKernelGGL((wkv56_split_kernel<0>), dim3((unsigned)(4 * H)), dim3(256), 0, st, a);
+        const int64_t waves = (int64_t)T * H;
+        hipLaunchKernelGGL(wkv56_gn_kernel, dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, st, T, C, y32, lnx_w, lnx_b,
+                           gate, out);
+    } else if (v6 && dw2) {
         if (ld <= 0 || (ld & 7)) return RWKV_E_SHAPE;
         hipLaunchKernelGGL((wkv56_kernel<true, 3, true>), dim3((unsigned)H), dim3(256), 0, st, a);
     } else if (v6)

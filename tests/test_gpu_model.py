@@ -286,3 +286,26 @@ def test_v56_forward_parity(ver, tag, strat):
     for t in toks[1:4]:
         g_out, g_st = m.forward([t], g_st)
     assert torch.equal(r_out, g_out)
+
+
+@pytest.mark.parametrize("ver,tag", V56)
+@pytest.mark.parametrize("strat", ["cuda fp16i8", "cuda fp16"])
+def test_v56_long_prompt(ver, tag, strat):
+    """Calls of 32 tokens and more split every head over four workgroups and run GroupNorm in a second
+    launch (70 tokens = two full slabs and a ragged one); logits, state and a following call must match
+    the oracle's token-by-token recurrence."""
+    ck = synth.make_checkpoint(version=ver, seed=300 + int(ver * 10), **TINY)
+    m = _rwkv()(ck, strat, verbose=False)
+    o = OracleRWKV(ck, strat)
+    toks = synth.random_tokens(70 + 33, TINY["vocab"], seed=PROMPT_SEED + 1)
+    full, st = m.forward(toks[:70], None, full_output=True)
+    ofull, ost = o.forward(toks[:70], None, full_output=True)
+    d_full = float(np.abs(_np(full) - ofull).max())
+    assert d_full <= LOGIT_TOL, d_full
+    assert _argmax_agree(_np(full), ofull, d_full)
+    for i, (a, b) in enumerate(zip(st, ost)):
+        np.testing.assert_allclose(_np(a), b.astype(np.float32), rtol=2e-2, atol=2e-2, err_msg=f"state {i}")
+    out, st = m.forward(toks[70:], st)
+    oout, ost = o.forward(toks[70:], ost)
+    d = float(np.abs(_np(out) - oout).max())
+    assert d <= LOGIT_TOL, d
