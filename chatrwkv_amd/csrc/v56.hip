@@ -80,9 +80,9 @@ struct Mix2Args {
 };
 
 // grid (ceil(T / 16), C/256, 5): m_j[c] = sum_i t1[t, jR + i] * w2[j][i][c]; out_j = xx + sxd * (maa_j + m_j).
-// One (channel, mix) per thread for a tile of 16 tokens: the R coefficients of the channel are loaded once
+// One (channel, mix) per thread for a tile of MIX2_TT tokens (16, or 1 for a one-token call): the R coefficients of the channel are loaded once
 // and reused for every token of the tile; the sum runs in index order.
-constexpr int MIX2_TT = 16;
+template <int MIX2_TT>
 __global__ __launch_bounds__(256) void v6_mix2_kernel(Mix2Args a) {
     __shared__ float st1[MIX2_TT][64];
     const int t0 = blockIdx.x * MIX2_TT, c = blockIdx.y * 256 + threadIdx.x, j = blockIdx.z, R = a.R, C = a.C;
@@ -296,7 +296,8 @@ extern "C" int rwkv_v56_forward(const rwkv_v56_model *m, const rwkv_v56_layer_st
             }
             b.T = (int)T; b.C = C; b.R = lm; b.t1 = ws.t1; b.w2 = l.tm_w2;
             for (int j = 0; j < 5; ++j) { b.maa[j] = l.att_mix[1 + j]; b.out[j] = ws.mix[j]; }
-            hipLaunchKernelGGL(v6_mix2_kernel, dim3((unsigned)((T + MIX2_TT - 1) / MIX2_TT), (unsigned)((C + 255) / 256), 5), dim3(256), 0, st, b);
+            if (T == 1) hipLaunchKernelGGL(v6_mix2_kernel<1>, dim3(1, (unsigned)((C + 255) / 256), 5), dim3(256), 0, st, b);
+            else hipLaunchKernelGGL(v6_mix2_kernel<16>, dim3((unsigned)((T + 15) / 16), (unsigned)((C + 255) / 256), 5), dim3(256), 0, st, b);
             wx = ws.mix[0]; kx = ws.mix[1]; vx = ws.mix[2]; rx = ws.mix[3]; gx = ws.mix[4];
             if ((rc = mm(c, lora_mat(l.td_w1, C, ld), false, wx, ACT_TANH, nullptr, nullptr, 1.f, ws.d1))) return rc;
             if (T > 1 && (rc = mm(c, lora_mat(l.td_w2, ld, C), false, ws.d1, ACT_NONE, nullptr, nullptr, 1.f, ws.d2))) return rc;
