@@ -37,18 +37,18 @@ int wkv56_fused_launch(bool v6, int T, int C, int H, float *state, const rwkv_ha
                        const float *lnx_b, const rwkv_half *gate, rwkv_half *out, hipStream_t st,
                        const rwkv_half *dw2 = nullptr, int ld = 0,  // dw2: v6 with w = tanh(. @ D1), product with D2 in-kernel
                        float *y32 = nullptr);  // fp32 [T, C] scratch: calls of >= 32 tokens split each head over 4 workgroups
-// Row-wise LayerNorm + token shift + mixes for up to 4 consumers over a [T, C] activation (seq_v4.hip).
+// Row-wise LayerNorm + token shift + mixes for up to 6 consumers over a [T, C] activation (seq_v4.hip).
 struct SeqMixArgs {
     int T, C;
     const rwkv_half *x;        // [T, C]
     const rwkv_half *ln_w, *ln_b;
     const rwkv_half *sx;       // state (previous token's normalised activation), NULL = no token shift
     rwkv_half *xx_last;        // scratch [C]: normalised activation of the last row (new state)
-    const rwkv_half *mix[4];   // NULL entry = consumer sees LN(x)
-    const rwkv_half *ry[4], *my[4];  // NULL ry = no scaling / sums (fp16 weights)
-    rwkv_half *xs[4];          // [T, C] outputs
-    float *s0[4], *s2[4];      // [T] outputs
-    int maa_form;              // RWKV-6 mixing kx = xx + (prev - xx) * m
+    const rwkv_half *mix[6];   // NULL entry = consumer sees LN(x)
+    const rwkv_half *ry[6], *my[6];  // NULL ry = no scaling / sums (fp16 weights)
+    rwkv_half *xs[6];          // [T, C] outputs
+    float *s0[6], *s2[6];      // [T] outputs
+    int maa_form;              // RWKV-6 / RWKV-7 mixing kx = xx + (prev - xx) * m, rounded after every step
 };
 
 int lnmix_seq_launch(const SeqMixArgs &a, int nj, hipStream_t st);

@@ -86,7 +86,7 @@ __global__ __launch_bounds__(256) void lnmix_seq_kernel(SeqMixArgs a) {
 #pragma unroll
                 for (int e = 0; e < 8; ++e) {
                     const float m = (float)mv[e];
-                    kx[e] = a.maa_form ? (h16)((float)xx[e] + (float)(h16)((float)pv[e] - (float)xx[e]) * m)
+                    kx[e] = a.maa_form ? (h16)((float)xx[e] + (float)(h16)((float)(h16)((float)pv[e] - (float)xx[e]) * m))
                                        : (h16)((float)xx[e] * m + (float)pv[e] * (1.f - m));
                 }
             }
@@ -136,6 +136,7 @@ int lnmix_seq_launch(const SeqMixArgs &a, int nj, hipStream_t st) {
         case 2: hipLaunchKernelGGL(lnmix_seq_kernel<2>, grid, block, 0, st, a); break;
         case 3: hipLaunchKernelGGL(lnmix_seq_kernel<3>, grid, block, 0, st, a); break;
         case 4: hipLaunchKernelGGL(lnmix_seq_kernel<4>, grid, block, 0, st, a); break;
+        case 6: hipLaunchKernelGGL(lnmix_seq_kernel<6>, grid, block, 0, st, a); break;
         default: return RWKV_E_DTYPE;
     }
     RWKV_LAUNCH_CHECK();

@@ -87,7 +87,29 @@ class RwkvV56Model(ctypes.Structure):
                 ("layers", ctypes.POINTER(RwkvV56Layer))]
 
 
+class RwkvV7Layer(ctypes.Structure):
+    _fields_ = [("ln1_w", _vp), ("ln1_b", _vp), ("ln2_w", _vp), ("ln2_b", _vp),
+                ("x_mix", _vp * 6),
+                ("w0", _vp), ("a0", _vp), ("v0", _vp),
+                ("w1", _vp), ("w2", _vp), ("a1", _vp), ("a2", _vp), ("v1", _vp), ("v2", _vp), ("g1", _vp), ("g2", _vp),
+                ("k_k", _vp), ("k_a", _vp), ("r_k", _vp), ("lnx_w", _vp), ("lnx_b", _vp),
+                ("att_receptance", RwkvMat), ("att_key", RwkvMat), ("att_value", RwkvMat), ("att_output", RwkvMat),
+                ("ffn_x_k", _vp), ("ffn_key", RwkvMat), ("ffn_value", RwkvMat)]
+
+
+class RwkvV7Model(ctypes.Structure):
+    _fields_ = [("n_layer", ctypes.c_int32), ("n_embd", ctypes.c_int32), ("n_ffn", ctypes.c_int32),
+                ("vocab", ctypes.c_int32), ("n_head", ctypes.c_int32),
+                ("lora_w", ctypes.c_int32), ("lora_a", ctypes.c_int32), ("lora_v", ctypes.c_int32),
+                ("lora_g", ctypes.c_int32),
+                ("emb", _vp), ("ln_out_w", _vp), ("ln_out_b", _vp), ("head", RwkvMat),
+                ("layers", ctypes.POINTER(RwkvV7Layer))]
+
+
 SIGNATURES.update({
+    "rwkv_wkv7_forward": (_int, [_i64, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _vp]),
+    "rwkv_v7_workspace": (_sz, [ctypes.POINTER(RwkvV7Model), _i64]),
+    "rwkv_v7_forward": (_int, [ctypes.POINTER(RwkvV7Model), ctypes.POINTER(RwkvV56LayerState), _vp, _i64, _int, _vp, _vp, _sz, _vp]),
     "rwkv_v56_workspace": (_sz, [ctypes.POINTER(RwkvV56Model), _i64]),
     "rwkv_v56_forward": (_int, [ctypes.POINTER(RwkvV56Model), ctypes.POINTER(RwkvV56LayerState), _vp, _i64, _int, _vp, _vp, _sz, _vp]),
     "rwkv_layernorm_f32_f16": (_int, [_i64, _i64, _vp, _vp, _vp, _vp, _vp]),

@@ -29,20 +29,9 @@ import torch
 from . import lib as _lib
 from . import ops as _ops
 from . import strategy as _strategy
+from .state import StateList
 
 _MATRIX_KEYS = ('key.weight', 'value.weight', 'receptance.weight', 'gate.weight', 'output.weight', 'head.weight')
-
-
-class StateList(list):
-    """The state list returned by forward(): a plain list of tensors (model.py:1448-1471) that
-    also remembers the flat buffers its entries are views of, so that a one-token step on the
-    same state can replay a captured HIP graph."""
-    flat = None      # tuple of backing tensors
-    views = None     # the tensors as handed out, to detect replaced entries
-
-    def intact(self):
-        v = self.views
-        return v is not None and len(v) == len(self) and all(a is b for a, b in zip(self, v))
 
 
 def _ptr(t):
@@ -534,3 +523,8 @@ class RWKV:
             if len(tokens) == 1:
                 return self._forward_one(tokens[0], state)
             return self._forward_seq(tokens, state, full_output)
+
+
+if os.environ.get('RWKV_V7_ON') == '1':                               # model.py:1679-1680
+    from .model_v7 import RWKV_x070
+    RWKV = RWKV_x070

@@ -30,6 +30,7 @@ SHAPES = {
     "v4-7b": (4, 32, 4096, 16384, 50277),
     "v4-14b": (4, 40, 5120, 20480, 50277),
     "v6-7b": (6, 32, 4096, 14336, 65536),
+    "v7-7b": (7, 32, 4096, 16384, 65536),
 }
 
 
@@ -140,9 +141,71 @@ def make_checkpoint(version=4, n_layer=2, n_embd=64, n_ffn=None, vocab=97, seed=
     return w
 
 
+def v7_lora_dims(n_embd):
+    """LoRA ranks (decay, in-context rate, value residual, gate) that released RWKV-7 checkpoints of
+    width ``n_embd`` use: multiples of 32 growing with the width."""
+    c = float(n_embd)
+    r32 = lambda v: max(32, int(round(v / 32.0)) * 32)
+    return r32(1.8 * c ** 0.5), r32(1.8 * c ** 0.5), r32(1.3 * c ** 0.5), r32(0.6 * c ** 0.8)
+
+
+def make_checkpoint_v7(n_layer=2, n_embd=128, n_ffn=None, vocab=97, seed=0, head_size=64, lora=None, device=None):
+    """RWKV-7 checkpoint with the keys ``RWKV_x070.__init__`` reads (model.py:245-282) and the forward
+    passes use (model.py:349-358): per block ``att.x_{r,w,k,v,a,g}``, ``att.{w,a,v}{0,1,2}``,
+    ``att.g{1,2}``, ``att.k_k``, ``att.k_a``, ``att.r_k`` [H, N], the four square matrices, ``att.ln_x``,
+    ``ffn.x_k`` and the two channel-mix matrices.  LoRA matrices are stored [in, rank] / [rank, out]
+    and are not transposed by the loader.  ``lora`` = (decay, a, v, gate) ranks."""
+    C = int(n_embd)
+    F = int(n_ffn) if n_ffn is not None else 4 * C
+    V = int(vocab)
+    H = C // head_size
+    assert H * head_size == C
+    dw, da, dv, dg = lora if lora is not None else v7_lora_dims(C)
+    g = _NumpyGen(seed) if device is None else _TorchGen(seed, device)
+    w = OrderedDict()
+    w["emb.weight"] = g.normal("emb.weight", (V, C), 0.02)
+    for i in range(n_layer):
+        b = f"blocks.{i}."
+        for ln in (("ln1", "ln2", "ln0") if i == 0 else ("ln1", "ln2")):
+            w[b + ln + ".weight"] = g.uniform(b + ln + ".weight", (C,), 0.8, 1.2)
+            w[b + ln + ".bias"] = g.normal(b + ln + ".bias", (C,), 0.05)
+        a = b + "att."
+        for m in "rwkvag":
+            w[a + "x_" + m] = g.uniform(a + "x_" + m, (1, 1, C), 0.0, 1.0)
+        w[a + "w0"] = g.uniform(a + "w0", (1, 1, C), -3.0, 2.0)
+        w[a + "w1"] = g.normal(a + "w1", (C, dw), 0.1)
+        w[a + "w2"] = g.normal(a + "w2", (dw, C), 0.2)
+        w[a + "a0"] = g.uniform(a + "a0", (1, 1, C), -1.0, 1.0)
+        w[a + "a1"] = g.normal(a + "a1", (C, da), 0.1)
+        w[a + "a2"] = g.normal(a + "a2", (da, C), 0.2)
+        w[a + "v0"] = g.uniform(a + "v0", (1, 1, C), -1.0, 1.0)
+        w[a + "v1"] = g.normal(a + "v1", (C, dv), 0.1)
+        w[a + "v2"] = g.normal(a + "v2", (dv, C), 0.2)
+        w[a + "g1"] = g.normal(a + "g1", (C, dg), 0.1)
+        w[a + "g2"] = g.normal(a + "g2", (dg, C), 0.2)
+        w[a + "k_k"] = g.uniform(a + "k_k", (1, 1, C), 0.5, 1.5)
+        w[a + "k_a"] = g.uniform(a + "k_a", (1, 1, C), 0.0, 1.0)
+        w[a + "r_k"] = g.normal(a + "r_k", (H, head_size), 0.3)
+        for name in ("receptance", "key", "value", "output"):
+            w[a + name + ".weight"] = g.normal(a + name + ".weight", (C, C), 0.05)
+        w[a + "ln_x.weight"] = g.uniform(a + "ln_x.weight", (C,), 0.8, 1.2)
+        w[a + "ln_x.bias"] = g.normal(a + "ln_x.bias", (C,), 0.05)
+        f = b + "ffn."
+        w[f + "x_k"] = g.uniform(f + "x_k", (1, 1, C), 0.0, 1.0)
+        w[f + "key.weight"] = g.normal(f + "key.weight", (F, C), 0.05)
+        w[f + "value.weight"] = g.normal(f + "value.weight", (C, F), 0.05)
+    w["ln_out.weight"] = g.uniform("ln_out.weight", (C,), 0.8, 1.2)
+    w["ln_out.bias"] = g.normal("ln_out.bias", (C,), 0.05)
+    w["head.weight"] = g.normal("head.weight", (V, C), 0.05)
+    return w
+
+
 def make_named(name, seed=0, device=None, n_layer=None):
     """Checkpoint for one of the named shapes in ``SHAPES`` (optionally fewer layers)."""
     version, L, C, F, V = SHAPES[name]
+    if version == 7:
+        return make_checkpoint_v7(n_layer=L if n_layer is None else n_layer, n_embd=C, n_ffn=F, vocab=V,
+                                  seed=seed, device=device)
     return make_checkpoint(version=version, n_layer=L if n_layer is None else n_layer, n_embd=C,
                            n_ffn=F, vocab=V, seed=seed, device=device)
 

@@ -270,6 +270,56 @@ int rwkv_v56_forward(const rwkv_v56_model *m, const rwkv_v56_layer_state *states
                      int64_t T, int full_output, float *logits, void *workspace, size_t workspace_bytes,
                      void *stream);
 
+/* ---------------------------------------------------------------------------------------
+ * RWKV-7 state recurrence.  Replaces torch.ops.wkv7s.forward_fp16 / forward_fp32
+ * (cuda/rwkv7_op.cpp:15-26, cuda/rwkv7.cu:9-58): per head, with row i of the state held per value index,
+ *     sa_i = sum_j a_j S_ij ;  S_ij = S_ij * exp(-exp(w_j)) + k_j v_i + sa_i b_j ;  y_i = sum_j S_ij r_j
+ * r, w, k, v, a, b, y: [T, C] in `dtype` (RWKV_DT_F16 or RWKV_DT_F32), w is the log-decay the reference
+ * passes (model.py:537-538); state fp32 [H][value i][key j] (model.py:288), updated in place; head size
+ * C / H must be 64; B must be 1 (cuda/rwkv7.cu:17, 66).
+ */
+int rwkv_wkv7_forward(int64_t B, int64_t T, int64_t C, int64_t H, float *state, const void *r, const void *w,
+                      const void *k, const void *v, const void *a, const void *b, void *y, int dtype,
+                      void *stream);
+
+/* =======================================================================================
+ * RWKV-7 ("x070"): one entry point for both modes of RWKV_x070.forward (model.py:292-302), replacing
+ * forward_one / forward_seq (model.py:336-363, 457-487), RWKV_x070_TMix_one / _seq (model.py:492-572),
+ * RWKV_x070_CMix_one / _seq (model.py:597-608) and RWKV7_OP (model.py:198-219).  The reference runs RWKV-7
+ * in fp16, bf16 or fp32 without quantisation (model.py:236-243); this entry point is the fp16 one.  Head
+ * size must be 64.  LoRA matrices are fp16, input-contiguous like the model matrices: first stages
+ * [rank][C] (the checkpoint's [C, rank] transposed), second stages [C][rank]; every rank is padded with
+ * zeros to a multiple of 64.
+ */
+typedef struct {
+    const rwkv_half *ln1_w, *ln1_b, *ln2_w, *ln2_b;      /* [C] */
+    const rwkv_half *x_mix[6];                            /* att.x_r, x_w, x_k, x_v, x_a, x_g [C] */
+    const rwkv_half *w0, *a0, *v0;                        /* [C]; v0 unused in layer 0 */
+    const rwkv_half *w1, *w2, *a1, *a2, *v1, *v2, *g1, *g2; /* LoRA pairs; v1, v2 unused in layer 0 */
+    const rwkv_half *k_k, *k_a, *r_k;                     /* [C] */
+    const rwkv_half *lnx_w, *lnx_b;                       /* [C] GroupNorm affine */
+    rwkv_mat att_receptance, att_key, att_value, att_output;
+    const rwkv_half *ffn_x_k;                             /* [C] */
+    rwkv_mat ffn_key, ffn_value;
+} rwkv_v7_layer;
+
+typedef struct {
+    int32_t n_layer, n_embd, n_ffn, vocab, n_head;
+    int32_t lora_w, lora_a, lora_v, lora_g;   /* padded ranks (multiples of 64) */
+    const rwkv_half *emb, *ln_out_w, *ln_out_b;
+    rwkv_mat head;
+    const rwkv_v7_layer *layers;
+} rwkv_v7_model;
+
+size_t rwkv_v7_workspace(const rwkv_v7_model *m, int64_t T);
+/* tokens: device int32 [T]; states: rwkv_v56_layer_state per layer with att_kv laid out
+ * [H][value][key] (model.py:286-289); logits fp32 [vocab] or [T, vocab] holding fp16-rounded values (the
+ * reference returns them as fp16, model.py:362, 486).  All state tensors are updated in place.  Only
+ * launches kernels: capturable. */
+int rwkv_v7_forward(const rwkv_v7_model *m, const rwkv_v56_layer_state *states, const int32_t *tokens,
+                    int64_t T, int full_output, float *logits, void *workspace, size_t workspace_bytes,
+                    void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -13,6 +13,7 @@ Modules
   ops.py     LayerNorm/GroupNorm, mm8, WKV v4/v5/v6     (model.py:984-1340, cuda/*.cu)
   model.py   checkpoint conversion + forward            (model.py:613-903, 1443-1677)
   sampling.py  sampling step after the path           (utils.py:55-88, 103-123)
+  model_v7.py  RWKV-7 (RWKV_x070) loading + forward     (model.py:223-608, cuda/rwkv7.cu)
 
 How each function is pinned (what a wrong sign / index / dropped term would trip):
   sampling.*           the reference's own draws for seeded numpy generators
@@ -29,6 +30,11 @@ How each function is pinned (what a wrong sign / index / dropped term would trip
   layer_norm/group_norm  torch CPU library routines.
   forward (all versions) golden logits and final state from the reference's CPU
                        path ('cpu fp32i8', 'cpu fp32'); chunk invariance.
+  model_v7.*           golden logits and final states from the reference's RWKV_x070 on
+                       the CPU under 'cpu fp32' AND 'cpu fp16' (the latter pins the fp16
+                       rounding points, tests/golden/e2e_v7_*.npz); the two restatements
+                       of the recurrence against each other, against a scalar loop and
+                       against the closed form of the a = 0 special case.
 The fp16 rounding points of the reference's 'cuda fp16i8' path cannot be run
 anywhere in this build (needs nvcc + an NVIDIA GPU): for that emulation mode the
 placement of the roundings follows the reference text and is otherwise

@@ -1,0 +1,195 @@
+"""GPU parity of RWKV_x070(model, 'cuda fp16').forward and of the wkv7 operator against the oracle
+(same seeded synthetic checkpoints) and against the golden logits the reference produced under
+'cpu fp16'.
+
+Tolerance: max abs logit error <= 2e-2 and the same argmax wherever the oracle's top-2 gap exceeds
+twice the observed error."""
+import copy
+import ctypes
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from chatrwkv_amd import synth
+from oracle import model_v7
+from oracle.model_v7 import OracleRWKV7
+from tests.golden.make_goldens_v7 import TINY7, CKPT_SEED, CHUNKS
+
+pytestmark = pytest.mark.gpu
+
+G = os.path.join(os.path.dirname(__file__), "golden")
+LOGIT_TOL = 2e-2
+
+
+def _np(t):
+    return t.detach().float().cpu().numpy()
+
+
+def _argmax_agree(got, ref, err):
+    srt = np.sort(ref, axis=-1)
+    decisive = (srt[..., -1] - srt[..., -2]) > 2 * err
+    return bool((np.argmax(got, -1) == np.argmax(ref, -1))[decisive].all())
+
+
+def _x070():
+    from chatrwkv_amd.model_v7 import RWKV_x070
+    return RWKV_x070
+
+
+@pytest.fixture(scope="module")
+def tiny7():
+    ck = synth.make_checkpoint_v7(seed=CKPT_SEED, **TINY7)
+    return _x070()(ck, "cuda fp16"), OracleRWKV7(ck, "cuda fp16"), ck
+
+
+# ----------------------------------------------------------------------------- operator
+
+@pytest.mark.parametrize("dtype", ["fp32", "fp16"])
+def test_wkv7_operator(dtype):
+    """rwkv_wkv7_forward against the oracle's restatement of cuda/rwkv7.cu, state carried over three
+    calls of 1, 37 and 70 tokens (the last spans several staging slabs)."""
+    from chatrwkv_amd import lib as _lib
+    L = _lib.load()
+    rng = np.random.Generator(np.random.PCG64(17))
+    H, N = 3, 64
+    C = H * N
+    npdt = np.float32 if dtype == "fp32" else np.float16
+    tdt = torch.float32 if dtype == "fp32" else torch.float16
+    code = _lib.RWKV_DT_F32 if dtype == "fp32" else _lib.RWKV_DT_F16
+    S_ref = (rng.standard_normal((H, N, N)) * 0.1).astype(np.float32)
+    S = torch.from_numpy(S_ref.copy()).cuda()
+    for T in (1, 37, 70):
+        r, k, v = ((rng.standard_normal((T, C)) * 0.5).astype(npdt) for _ in range(3))
+        kk = rng.standard_normal((T, C))
+        kk /= np.linalg.norm(kk.reshape(T, H, N), axis=-1, keepdims=True).repeat(N, -1).reshape(T, C)
+        a = (-kk).astype(npdt)
+        b = (kk * rng.random((T, C))).astype(npdt)
+        w = rng.uniform(-4.0, -0.5, (T, C)).astype(npdt)
+        y_ref, S_ref = model_v7.wkv7_kernel(S_ref, r, w, k, v, a, b)
+        dev = [torch.from_numpy(x).cuda() for x in (r, w, k, v, a, b)]
+        y = torch.empty((T, C), dtype=tdt, device="cuda")
+        rc = L.rwkv_wkv7_forward(1, T, C, H, S.data_ptr(), *(x.data_ptr() for x in dev), y.data_ptr(), code,
+                                 torch.cuda.current_stream().cuda_stream)
+        _lib.check(rc, "rwkv_wkv7_forward")
+        torch.cuda.synchronize()
+        scale = float(np.abs(y_ref.astype(np.float32)).max())
+        tol = 2e-5 * max(scale, 1.0) if dtype == "fp32" else 2e-3 * max(scale, 1.0)
+        assert np.abs(_np(y) - y_ref.astype(np.float32)).max() <= tol, T
+        assert np.abs(_np(S) - S_ref).max() <= 2e-5 * max(float(np.abs(S_ref).max()), 1.0), T
+
+
+def test_wkv7_operator_rejects_bad_shapes():
+    from chatrwkv_amd import lib as _lib
+    L = _lib.load()
+    x = torch.zeros(64 * 64, device="cuda")
+    p = x.data_ptr()
+    assert L.rwkv_wkv7_forward(2, 1, 64, 1, p, p, p, p, p, p, p, p, _lib.RWKV_DT_F32, None) == -1   # B != 1
+    assert L.rwkv_wkv7_forward(1, 1, 96, 1, p, p, p, p, p, p, p, p, _lib.RWKV_DT_F32, None) == -1   # head size
+    assert L.rwkv_wkv7_forward(1, 1, 64, 1, p, p, p, p, p, p, p, p, 7, None) == -5
+    assert L.rwkv_wkv7_forward(1, 1, 64, 1, None, p, p, p, p, p, p, p, _lib.RWKV_DT_F32, None) == -3
+
+
+# ----------------------------------------------------------------------------- model
+
+def test_v7_forward_parity(tiny7):
+    m, o, _ = tiny7
+    g = dict(np.load(os.path.join(G, "e2e_v7_cpu_fp16.npz")))
+    toks = [int(t) for t in g["tokens"]]
+    full, st = m.forward(toks, None, full_output=True)
+    ofull, ost = o.forward(toks, None, full_output=True)
+    assert full.dtype == torch.float16 and tuple(full.shape) == ofull.shape
+    d = float(np.abs(_np(full) - ofull.astype(np.float32)).max())
+    assert d <= LOGIT_TOL, d
+    assert _argmax_agree(_np(full), ofull.astype(np.float32), d)
+    # the reference's own fp16 run on the CPU
+    dg = float(np.abs(_np(full) - g["full_logits"]).max())
+    assert dg <= LOGIT_TOL, dg
+    assert isinstance(st, list) and len(st) == 3 * TINY7["n_layer"]
+    H = TINY7["n_embd"] // 64
+    for i, (s, ref) in enumerate(zip(st, ost)):
+        assert s.dtype == (torch.float32 if i % 3 == 1 else torch.float16)
+        assert tuple(s.shape) == ref.shape == ((H, 64, 64) if i % 3 == 1 else (TINY7["n_embd"],))
+        scale = max(float(np.abs(ref.astype(np.float32)).max()), 1.0)
+        assert np.abs(_np(s) - ref.astype(np.float32)).max() <= 1e-2 * scale, i
+        assert np.abs(_np(s) - g[f"full_state_{i}"]).max() <= 1e-2 * scale, i
+
+
+def test_v7_chunked_and_one_token(tiny7):
+    """Sequence calls and one-token calls interleaved, state carried in place; int, [int] and GPU tensor
+    forms of a one-token call."""
+    m, o, _ = tiny7
+    g = dict(np.load(os.path.join(G, "e2e_v7_cpu_fp16.npz")))
+    toks = [int(t) for t in g["tokens"]]
+    st, ost = None, None
+    for j, (a, b) in enumerate(CHUNKS):
+        if b - a > 1:
+            idx = toks[a:b]
+        else:
+            idx = (toks[a], [toks[a]], torch.tensor([toks[a]], device="cuda"))[j % 3]
+        out, st2 = m.forward(idx, st)
+        assert st is None or st2 is st
+        st = st2
+        oo, ost = o.forward(toks[a:b], ost)
+        assert out.dtype == torch.float16 and tuple(out.shape) == (TINY7["vocab"],)
+        d = float(np.abs(_np(out) - oo.astype(np.float32)).max())
+        assert d <= LOGIT_TOL, (j, d)
+        assert np.abs(_np(out) - g["chunk_logits"][j]).max() <= LOGIT_TOL, j
+    for i, (s, ref) in enumerate(zip(st, ost)):
+        scale = max(float(np.abs(ref.astype(np.float32)).max()), 1.0)
+        assert np.abs(_np(s) - ref.astype(np.float32)).max() <= 1e-2 * scale, i
+
+
+def test_v7_graph_replay_and_snapshot(tiny7):
+    """Greedy one-token steps replay a captured graph: every replay equals the eager step from the
+    same state; a deep copy of the state is an independent snapshot."""
+    m, _, _ = tiny7
+    V = TINY7["vocab"]
+    toks = synth.random_tokens(12, V, seed=3)
+    _, st = m.forward(toks[:5], None)
+    for step, t in enumerate(toks[5:]):
+        snap = copy.deepcopy(st)
+        os.environ["RWKV_HIP_GRAPH"] = "0"
+        try:
+            eager, _ = m.forward([t], list(snap))
+        finally:
+            os.environ["RWKV_HIP_GRAPH"] = "1"
+        torch.cuda.synchronize()
+        out, st = m.forward([t], st)
+        assert torch.equal(out, eager), step
+        for a, b in zip(st, snap):
+            assert torch.equal(a, b)
+
+
+def test_v7_long_prompt_and_odd_lora_ranks():
+    """Two heads' worth more channels, LoRA ranks that need padding (32, 96, 160), a prompt longer than
+    two staging slabs followed by a shorter call."""
+    cfg = dict(n_layer=2, n_embd=256, n_ffn=1024, vocab=300, lora=(32, 96, 32, 160))
+    ck = synth.make_checkpoint_v7(seed=71, **cfg)
+    m, o = _x070()(ck, "cuda fp16"), OracleRWKV7(ck, "cuda fp16", kernel_form=True)
+    toks = synth.random_tokens(103, cfg["vocab"], seed=9)
+    st, ost = None, None
+    for a, b in ((0, 70), (70, 103)):
+        out, st = m.forward(toks[a:b], st, full_output=True)
+        oo, ost = o.forward(toks[a:b], ost, full_output=True)
+        d = float(np.abs(_np(out) - oo.astype(np.float32)).max())
+        assert d <= LOGIT_TOL, d
+        assert _argmax_agree(_np(out), oo.astype(np.float32), d)
+    for i, (s, ref) in enumerate(zip(st, ost)):
+        scale = max(float(np.abs(ref.astype(np.float32)).max()), 1.0)
+        assert np.abs(_np(s) - ref.astype(np.float32)).max() <= 1e-2 * scale, i
+
+
+def test_v7_api_errors(tiny7):
+    m, _, ck = tiny7
+    with pytest.raises(IndexError):
+        m.forward([TINY7["vocab"]], None)
+    with pytest.raises(IndexError):
+        m.forward([1, -1], None)
+    with pytest.raises(ValueError):
+        m.forward([1], [torch.zeros(1)])
+    with pytest.raises(NotImplementedError):
+        _x070()(ck, "cuda fp32")
+    with pytest.raises(AssertionError):
+        _x070()(ck, "cuda fp16i8")
