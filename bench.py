@@ -121,12 +121,19 @@ def main():
         L = args.layers
     dev = "cuda:0"
     torch.cuda.set_device(0)
-    ck = synth.make_checkpoint(version=version, n_layer=L, n_embd=C, n_ffn=F, vocab=V, seed=2, device=dev)
-    model = RWKV(ck, args.strategy, verbose=False)
+    u8 = args.strategy.endswith("i8")
+    if version == 7:
+        # RWKV-7 runs unquantised (the reference offers fp16 / bf16 / fp32 only)
+        from chatrwkv_amd.model_v7 import RWKV_x070
+        ck = synth.make_checkpoint_v7(n_layer=L, n_embd=C, n_ffn=F, vocab=V, seed=2, device=dev)
+        model = RWKV_x070(ck, args.strategy)
+        wbytes = 2 * (L * (4 * C * C + 2 * C * F + 2 * C * sum(synth.v7_lora_dims(C))) + C * V)
+    else:
+        ck = synth.make_checkpoint(version=version, n_layer=L, n_embd=C, n_ffn=F, vocab=V, seed=2, device=dev)
+        model = RWKV(ck, args.strategy, verbose=False)
+        wbytes = u8_weight_bytes(L, C, F, V, version) * (1 if u8 else 2)
     del ck
     torch.cuda.empty_cache()
-    u8 = args.strategy.endswith("i8")
-    wbytes = u8_weight_bytes(L, C, F, V, version) * (1 if u8 else 2)
 
     # ---- prefill: one call over `prefill` tokens (median of 3, after one warm-up call)
     ptoks = synth.random_tokens(args.prefill, V, seed=2)
@@ -216,7 +223,7 @@ def main():
         "ms_per_step": 1e3 * t_dev / args.steps, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "u8 weights, fp16 activations, fp32 accumulate" if u8 else "fp16",
         "data": "synthetic (random-init weights, random tokens)",
-        "config": {"workload": f"RWKV-4 {args.shape} ({L} layers, n_embd {C}, ffn {F}, vocab {V}) '{args.strategy}', "
+        "config": {"workload": f"RWKV-{int(version)} {args.shape} ({L} layers, n_embd {C}, ffn {F}, vocab {V}) '{args.strategy}', "
                                f"batch 1: prefill {args.prefill} tokens in {'one call' if chunk >= args.prefill else f'calls of {chunk}'}, "
                                f"then greedy decode" + (" (BASELINE.json configs[2])" if args.shape == "v4-7b" else ""),
                    "strategy": args.strategy, "prefill_tokens": args.prefill},
@@ -229,7 +236,7 @@ def main():
                     "flops": prefill_flops, "TFLOPs": prefill_flops / t_prefill / 1e12,
                     "frac_of_mfma_peak": prefill_flops / t_prefill / MFMA_F16_PEAK},
     }
-    if not args.no_cpu:
+    if not args.no_cpu and version != 7:
         res["cpu_baseline"] = cpu_baseline(args.shape)
     else:
         res["cpu_baseline"] = None

@@ -651,6 +651,13 @@ inline void lnmix1_small_launch(const LnMixArgs &a, hipStream_t st) {
     hipLaunchKernelGGL((lnmix_kernel<false, 1, 1>), dim3(grid), dim3(DTHREADS), (size_t)a.C * 2, st, a);
 }
 
+// LN + token shift + one mix + a GEMV over the rows of one large matrix.
+inline void lnmix1_launch(bool u8, const LnMixArgs &a, int grid, hipStream_t st) {
+    const size_t lds = (size_t)a.C * 2;
+    if (u8) hipLaunchKernelGGL((lnmix_kernel<true, 1, 4>), dim3(grid), dim3(DTHREADS), lds, st, a);
+    else hipLaunchKernelGGL((lnmix_kernel<false, 1, 4>), dim3(grid), dim3(DTHREADS), lds, st, a);
+}
+
 // LN_out(x) @ head -> fp32 logits (fp16-rounded values) in one launch.
 inline void lnhead_launch(bool u8, const rwkv_half *x, int C, const rwkv_half *ln_w, const rwkv_half *ln_b,
                           const MatDev &head, int vocab, float *logits, int grid, hipStream_t st) {

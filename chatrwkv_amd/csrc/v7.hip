@@ -10,6 +10,16 @@
 //   gn7     GroupNorm per head, + bonus * v, * g
 //   output matrix with the residual add in its epilogue
 // then the channel mix: LN2, one mix, relu(. @ K)^2 @ V with the residual add.
+//
+// One token (T == 1) runs five launches per layer instead:
+//   att7_kernel    LN1 + token shift + the six mixes -> rows (Wr[c], Wk[c], Wv[c]) per wave, then the rows of
+//                  the four first LoRA stages (tanh / none / none / sigmoid)
+//   tmix7_kernel   per head: second LoRA stages, the preparation above, one step of the recurrence,
+//                  GroupNorm, bonus and gate
+//   vec_kernel     rows of Wo, x += out
+//   lnmix_kernel   LN2 + token shift + mix -> rows of the channel-mix key matrix, relu^2
+//   vec_kernel     rows of the channel-mix value matrix, x += out
+#include <algorithm>
 #include "mm_dispatch.h"
 
 namespace {
@@ -69,61 +79,122 @@ struct Wkv7Args {
 
 // A head's value rows never interact (sa_i, y_i and row i of the state depend on v_i only), so a head is
 // split over four workgroups of 16 value rows.  Thread (value i, key group g): lane & 15 = g owns keys
-// 4g..4g+3 of row i.  The two sums over a row's 16 key groups are DPP row sums in registers, so the token
-// loop has no barrier; r, w, k, a, b of a slab of tokens are staged in LDS as fp32.
+// 4g..4g+3 of row i; sums over a row's 16 key groups are DPP row sums in registers, so the token loop has
+// no barrier.  r, w, k, a, b of a slab of tokens are staged in LDS as fp32.
+// The only loop-carried chain is state -> sa -> state.  The read-out is taken off it by expanding
+//     y_i = sum_j S'_ij r_j = sum_j S_ij (w_j r_j) + v_i (k . r) + sa_i (b . r)
+// so that both row sums of a token run on the OLD state side by side; k . r and b . r are per-token
+// scalars computed while staging.
 //   IN_F16: element type of r, k, v, a, b (and of w, y in the operator form)
 //   MODEL:  w is the fp32 decay itself and y an fp32 scratch; otherwise w is the log-decay
 //           (decay = exp(-exp(w))) and y has the input type
+// Staging: thread (token tid / 8, channels 8 (tid % 8) ..+7) loads its share of the NEXT slab into
+// registers before the token loop of the current one, so the loads' latency is hidden behind the loop.
+template <bool IN_F16>
+struct Stage7 {
+    float r[8], k[8], a[8], b[8], w[8], v[2];
+
+    DEV void load8(const void *p, size_t o, float (&d)[8]) {
+        if (IN_F16) {
+            const h16x8 x = *(const h16x8 *)((const rwkv_half *)p + o);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) d[e] = (float)x[e];
+        } else {
+            const f32x4 x0 = *(const f32x4 *)((const float *)p + o), x1 = *(const f32x4 *)((const float *)p + o + 4);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) { d[e] = x0[e]; d[4 + e] = x1[e]; }
+        }
+    }
+};
+
 template <bool IN_F16, bool MODEL>
 __global__ __launch_bounds__(256) void wkv7_kernel(Wkv7Args a) {
-    __shared__ __align__(16) float sr[TS7][HS7], sk[TS7][HS7], sw[TS7][HS7], sa[TS7][HS7], sb[TS7][HS7];
-    __shared__ float sv[TS7][16];
+    __shared__ __align__(16) float swr[TS7][HS7], sk[TS7][HS7], sw[TS7][HS7], sa[TS7][HS7], sb[TS7][HS7];
+    __shared__ float sv[TS7][16], skr[TS7], sbr[TS7];
     const int T = a.T, C = a.C;
     const int h = blockIdx.x >> 2, vb = blockIdx.x & 3;
     const int lane = threadIdx.x & 63, g = lane & 15;
     const int il = (threadIdx.x >> 6) * 4 + (lane >> 4);
     const int i = vb * 16 + il;
+    const int stt = threadIdx.x >> 3, sc = (threadIdx.x & 7) * 8;   // staging role
     float *S = a.state + (size_t)h * HS7 * HS7 + (size_t)i * HS7 + 4 * g;
     f32x4 s = *(const f32x4 *)S;
-    auto ld = [&](const void *p, size_t o) -> float {
-        return IN_F16 ? h2f(((const rwkv_half *)p)[o]) : ((const float *)p)[o];
+    Stage7<IN_F16> st;
+    auto fetch = [&](int t0) {
+        const size_t o = (size_t)min(t0 + stt, T - 1) * C + h * HS7;   // rows past the end re-read the last one
+        st.load8(a.r, o + sc, st.r);
+        st.load8(a.k, o + sc, st.k);
+        st.load8(a.a, o + sc, st.a);
+        st.load8(a.b, o + sc, st.b);
+        if (MODEL) {
+            const f32x4 x0 = *(const f32x4 *)((const float *)a.w + o + sc), x1 = *(const f32x4 *)((const float *)a.w + o + sc + 4);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) { st.w[e] = x0[e]; st.w[4 + e] = x1[e]; }
+        } else {
+            st.load8(a.w, o + sc, st.w);
+        }
+        const size_t ov = o + vb * 16 + 2 * (threadIdx.x & 7);
+        if (IN_F16) {
+            const h16x2 x = *(const h16x2 *)((const rwkv_half *)a.v + ov);
+            st.v[0] = (float)x[0]; st.v[1] = (float)x[1];
+        } else {
+            st.v[0] = ((const float *)a.v)[ov]; st.v[1] = ((const float *)a.v)[ov + 1];
+        }
     };
+    fetch(0);
     for (int t0 = 0; t0 < T; t0 += TS7) {
         const int nt = min(TS7, T - t0);
         __syncthreads();  // previous slab fully consumed
-        for (int e = threadIdx.x; e < nt * HS7; e += 256) {
-            const int tt = e >> 6, c = e & 63;
-            const size_t o = (size_t)(t0 + tt) * C + h * HS7 + c;
-            sr[tt][c] = ld(a.r, o);
-            sk[tt][c] = ld(a.k, o);
-            sa[tt][c] = ld(a.a, o);
-            sb[tt][c] = ld(a.b, o);
-            sw[tt][c] = MODEL ? ((const float *)a.w)[o] : __expf(-__expf(ld(a.w, o)));
-        }
-        for (int e = threadIdx.x; e < nt * 16; e += 256) {
-            const int tt = e >> 4, c = e & 15;
-            sv[tt][c] = ld(a.v, (size_t)(t0 + tt) * C + h * HS7 + vb * 16 + c);
+        {
+            float kr = 0.f, br = 0.f;
+            f32x4 o4[5][2];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float w = MODEL ? st.w[e] : __expf(-__expf(st.w[e]));
+                o4[0][e >> 2][e & 3] = w * st.r[e];
+                o4[1][e >> 2][e & 3] = st.k[e];
+                o4[2][e >> 2][e & 3] = w;
+                o4[3][e >> 2][e & 3] = st.a[e];
+                o4[4][e >> 2][e & 3] = st.b[e];
+                kr += st.k[e] * st.r[e];
+                br += st.b[e] * st.r[e];
+            }
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+                *(f32x4 *)&swr[stt][sc + 4 * u] = o4[0][u];
+                *(f32x4 *)&sk[stt][sc + 4 * u] = o4[1][u];
+                *(f32x4 *)&sw[stt][sc + 4 * u] = o4[2][u];
+                *(f32x4 *)&sa[stt][sc + 4 * u] = o4[3][u];
+                *(f32x4 *)&sb[stt][sc + 4 * u] = o4[4][u];
+            }
+            sv[stt][2 * (threadIdx.x & 7)] = st.v[0];
+            sv[stt][2 * (threadIdx.x & 7) + 1] = st.v[1];
+            // the 8 threads of a token are 8 consecutive lanes: three DPP steps
+            kr += dpp_mov<0xB1>(kr); br += dpp_mov<0xB1>(br);
+            kr += dpp_mov<0x4E>(kr); br += dpp_mov<0x4E>(br);
+            kr += dpp_mov<0x141>(kr); br += dpp_mov<0x141>(br);
+            if ((threadIdx.x & 7) == 0) { skr[stt] = kr; sbr[stt] = br; }
         }
         __syncthreads();
+        fetch(t0 + TS7);
         for (int tt = 0; tt < nt; ++tt) {
-            const float vi = sv[tt][il];
-            const f32x4 r4 = *(const f32x4 *)&sr[tt][4 * g];
+            const float vi = sv[tt][il], kr = skr[tt], br = sbr[tt];
+            const f32x4 wr4 = *(const f32x4 *)&swr[tt][4 * g];
             const f32x4 k4 = *(const f32x4 *)&sk[tt][4 * g];
             const f32x4 w4 = *(const f32x4 *)&sw[tt][4 * g];
             const f32x4 a4 = *(const f32x4 *)&sa[tt][4 * g];
             const f32x4 b4 = *(const f32x4 *)&sb[tt][4 * g];
-            float p = 0.f;
+            float p = (a4[0] * s[0] + a4[1] * s[1]) + (a4[2] * s[2] + a4[3] * s[3]);
+            float yw = (wr4[0] * s[0] + wr4[1] * s[1]) + (wr4[2] * s[2] + wr4[3] * s[3]);
+            f32x4 kv;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) p += a4[e] * s[e];
-            const float sav = row16_sum(p);
-            float y = 0.f;
+            for (int e = 0; e < 4; ++e) kv[e] = s[e] * w4[e] + k4[e] * vi;
+            p = row16_sum(p);
+            yw = row16_sum(yw);
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                s[e] = s[e] * w4[e] + k4[e] * vi + sav * b4[e];
-                y += s[e] * r4[e];
-            }
-            y = row16_sum(y);
+            for (int e = 0; e < 4; ++e) s[e] = kv[e] + p * b4[e];
             if (g == 0) {
+                const float y = yw + vi * kr + p * br;
                 const size_t o = (size_t)(t0 + tt) * C + h * HS7 + i;
                 if (MODEL || !IN_F16) ((float *)a.y)[o] = y;
                 else ((rwkv_half *)a.y)[o] = f2h(y);
@@ -157,8 +228,177 @@ __global__ __launch_bounds__(256) void gn7_kernel(int T, int C, const float *__r
     out[o] = f2h(q * h2f(gate[o]));
 }
 
+// ---- one-token kernels ---------------------------------------------------------------------
+struct Att7Args {
+    const rwkv_half *x;
+    int C;
+    const rwkv_half *ln_w, *ln_b, *sx;
+    rwkv_half *xx_tmp;
+    const rwkv_half *mix[6];   // r, w, k, v, a, g
+    MatDev mat[3];             // receptance, key, value
+    rwkv_half *out[3];         // r, k, v  [C]
+    const rwkv_half *lora1;    // [rtot][C]
+    int rtot, o_a, o_v, o_g;   // rows, first row of the a / v / g blocks
+    rwkv_half *l1;             // [rtot] activated first-stage outputs
+};
+
+struct NoEpi {};
+
+__global__ __launch_bounds__(DTHREADS) void att7_kernel(Att7Args a) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    __shared__ float red[(2 + 3 * 6) * DWAVES];
+    const int C = a.C;
+    h16 *xs[6];
+    const rwkv_half *mix[6];
+    MatDev nomat[6] = {};
+#pragma unroll
+    for (int j = 0; j < 6; ++j) { xs[j] = (h16 *)smem + j * C; mix[j] = a.mix[j]; }
+    VecSums S[6];
+    LnMixPro<false, 6> pro;
+    auto pro_load = [&]() { pro.load(a.x, C, a.ln_w, a.ln_b, a.sx, mix, nomat); };
+    auto pro_compute = [&]() { pro.compute(C, true, mix, xs, S, a.xx_tmp, red, true); };
+    auto rowf = [&](int c, int k, const uint8_t *&row, const h16 *&xv) {
+        row = row_ptr<false>(a.mat[k], c);
+        xv = xs[k == 0 ? 0 : (k == 1 ? 2 : 3)];
+    };
+    auto epi_load = [&](int) { return NoEpi{}; };
+    auto epi = [&](int c, const float (&d)[3], const NoEpi &) {
+#pragma unroll
+        for (int k = 0; k < 3; ++k) a.out[k][c] = f2h(d[k]);
+    };
+    const int nseg = (C * 2) >> 4;
+    stream_rows<false, 1, 3, 2, NoEpi>(C, nseg, pro_owner_wave(C >> 3), pro_load, pro_compute, rowf, epi_load, epi);
+    // first LoRA stages: row g of the stacked matrix belongs to block j = w, a, v, g
+    auto block_of = [&](int g) { return (g >= a.o_a ? 1 : 0) + (g >= a.o_v ? 1 : 0) + (g >= a.o_g ? 1 : 0); };
+    auto rowf2 = [&](int g, int, const uint8_t *&row, const h16 *&xv) {
+        row = (const uint8_t *)(a.lora1 + (size_t)g * C);
+        const int j = block_of(g);
+        const int mi = j == 0 ? 1 : (j == 1 ? 4 : (j == 2 ? 3 : 5));   // xw, xa, xv, xg
+        xv = (const h16 *)smem + mi * C;
+    };
+    auto epi2 = [&](int g, const float (&d)[1], const NoEpi &) {
+        const int j = block_of(g);
+        float v = round_h(d[0]);
+        v = j == 0 ? tanhf(v) : (j == 3 ? sigmoidf_(v) : v);
+        a.l1[g] = f2h(v);
+    };
+    stream_rows<false, 1, 1, 2, NoEpi>(a.rtot, nseg, false, [] {}, [] {}, rowf2, epi_load, epi2);
+}
+
+struct Tmix7Args {
+    int C, rtot, o_a, o_v, o_g, d_w, d_a, d_v, d_g;
+    int first_layer;
+    const rwkv_half *l1;       // [rtot]
+    const rwkv_half *lora2;    // [C][rtot]
+    const rwkv_half *r, *k, *v, *v_first;   // [C]; v_first unused in layer 0 (there v is the layer-0 value itself)
+    const rwkv_half *w0, *a0, *v0, *k_k, *k_a, *r_k, *lnx_w, *lnx_b;
+    float *state;              // [H][64][64]
+    rwkv_half *out;            // [C]
+    const rwkv_half *commit_src;   // scratch xx -> token-shift state, done by workgroup 0
+    rwkv_half *commit_dst;
+};
+
+// One workgroup of 16 waves per head.  All operands are requested in the first instructions (one memory
+// round trip): wave w takes 16 (channel, product) rows of the second LoRA stages -- product w / 4, lane =
+// 16-byte segment of the row, so a row is one coalesced request -- the first four waves also the head's
+// state, wave 0 also the head's vectors.  Then: row sums -> LDS; wave 0 prepares the step; threads 0..255
+// (value rows il + 16 m, key group g = lane & 15, holding S[i][4g..4g+3] of their four rows) advance the
+// state, the sums over a row's key groups being DPP row sums; wave 0 normalises and gates.
+__global__ __launch_bounds__(1024) void tmix7_kernel(Tmix7Args a) {
+    __shared__ float lo[4][HS7];
+    __shared__ __align__(16) float sr[HS7], sk[HS7], sw[HS7], sa[HS7], sb[HS7];
+    __shared__ float sv[HS7], sy[HS7], srk;
+    const int h = blockIdx.x, tid = threadIdx.x, lane = tid & 63;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int il = (tid >> 4) & 15, g = tid & 15;
+    const int c = h * HS7 + lane;
+    float *S = a.state + (size_t)h * HS7 * HS7;
+    // ---- loads
+    const int q = w >> 2;
+    const int off = q == 0 ? 0 : (q == 1 ? a.o_a : (q == 2 ? a.o_v : a.o_g));
+    const int d8 = (q == 0 ? a.d_w : (q == 1 ? a.d_a : (q == 2 ? (a.first_layer ? 0 : a.d_v) : a.d_g))) >> 3;
+    const int seg = lane < d8 ? lane : 0;
+    const h16x8 xv = *(const h16x8 *)(a.l1 + off + 8 * seg);
+    u32x4 wv[16];
+#pragma unroll
+    for (int jj = 0; jj < 16; ++jj)
+        wv[jj] = *(const u32x4 *)(a.lora2 + (size_t)(h * HS7 + (w & 3) * 16 + jj) * a.rtot + off + 8 * seg);
+    f32x4 s[4] = {};
+    if (w < 4)
+#pragma unroll
+        for (int m = 0; m < 4; ++m) s[m] = *(const f32x4 *)(S + (size_t)(il + 16 * m) * HS7 + 4 * g);
+    float r = 0.f, k = 0.f, v = 0.f, vf = 0.f, a0 = 0.f, w0 = 0.f, v0 = 0.f, k_k = 0.f, k_a = 0.f, r_k = 0.f, lw = 0.f, lb = 0.f;
+    if (w == 0) {
+        r = h2f(a.r[c]); k = h2f(a.k[c]); v = h2f(a.v[c]);
+        a0 = h2f(a.a0[c]); w0 = h2f(a.w0[c]); k_k = h2f(a.k_k[c]); k_a = h2f(a.k_a[c]); r_k = h2f(a.r_k[c]);
+        lw = h2f(a.lnx_w[c]); lb = h2f(a.lnx_b[c]);
+        if (!a.first_layer) { vf = h2f(a.v_first[c]); v0 = h2f(a.v0[c]); }
+    }
+    // ---- second LoRA stages
+#pragma unroll
+    for (int jj = 0; jj < 16; ++jj) {
+        const float p = wave_sum(lane < d8 ? dot8_f16(wv[jj], xv, 0.f) : 0.f);
+        if (lane == 0) lo[q][(w & 3) * 16 + jj] = round_h(p);
+    }
+    __syncthreads();
+    if (w == 0) {
+        const float av = round_h(sigmoidf_(round_h(a0 + lo[1][lane])));
+        const float kku = round_h(k * k_k);
+        const float nrm = fmaxf(round_h(sqrtf(wave_sum(kku * kku))), 1e-12f);
+        const float kk = round_h(kku / nrm);
+        const float k2 = round_h(k * round_h(1.f + round_h(round_h(av - 1.f) * k_a)));
+        if (!a.first_layer) {
+            const float sg = round_h(sigmoidf_(round_h(v0 + lo[2][lane])));
+            v = round_h(v + round_h(round_h(vf - v) * sg));
+        }
+        const float z = round_h(w0 + lo[0][lane]);
+        sr[lane] = r; sk[lane] = k2; sv[lane] = v;
+        sw[lane] = __expf(-0.606531f * sigmoidf_(z));
+        sa[lane] = -kk;
+        sb[lane] = round_h(kk * av);
+        const float rk = wave_sum(round_h(round_h(r * k2) * r_k));
+        if (lane == 0) srk = round_h(rk);
+    }
+    __syncthreads();
+    if (w < 4) {
+        const f32x4 r4 = *(const f32x4 *)&sr[4 * g], k4 = *(const f32x4 *)&sk[4 * g], w4 = *(const f32x4 *)&sw[4 * g];
+        const f32x4 a4 = *(const f32x4 *)&sa[4 * g], b4 = *(const f32x4 *)&sb[4 * g];
+#pragma unroll
+        for (int m = 0; m < 4; ++m) {
+            const int i = il + 16 * m;
+            const float vi = sv[i];
+            float p = 0.f;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) p += a4[e] * s[m][e];
+            const float sav = row16_sum(p);
+            float y = 0.f;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                s[m][e] = s[m][e] * w4[e] + k4[e] * vi + sav * b4[e];
+                y += s[m][e] * r4[e];
+            }
+            y = row16_sum(y);
+            if (g == 0) sy[i] = y;
+            *(f32x4 *)(S + (size_t)i * HS7 + 4 * g) = s[m];
+        }
+    }
+    __syncthreads();
+    if (w == 0) {
+        const float yv = round_h(sy[lane]);
+        const float mean = wave_sum(yv) * (1.f / HS7);
+        const float dv = yv - mean;
+        const float var = wave_sum(dv * dv) * (1.f / HS7);
+        float o = round_h(dv * rsqrtf(var + 64e-5f) * lw + lb);
+        o = round_h(o + round_h(srk * sv[lane]));
+        a.out[c] = f2h(o * lo[3][lane]);
+    }
+    if (blockIdx.x == 0 && a.commit_dst)
+        for (int j8 = tid; j8 < (a.C >> 3); j8 += 1024)
+            *(u32x4 *)(a.commit_dst + 8 * j8) = *(const u32x4 *)(a.commit_src + 8 * j8);
+}
+
 struct Ws7 {
-    rwkv_half *x, *mix[6], *lw, *la, *lv, *lg, *w_raw, *a_raw, *vg_raw, *g, *r, *k, *v, *v_first, *an, *b, *att, *vx,
+    rwkv_half *x, *mix[6], *l1, *lw, *la, *lv, *lg, *w_raw, *a_raw, *vg_raw, *g, *r, *k, *v, *v_first, *an, *b, *att, *vx,
         *xx_att, *xx_ffn;
     float *dec, *rk, *y32, *splitk;
     size_t total;
@@ -172,6 +412,7 @@ Ws7 carve7(void *base, int64_t T, const rwkv_v7_model *m) {
     const size_t tc = (size_t)T * C * 2;
     w.x = take(tc);
     for (int j = 0; j < 6; ++j) w.mix[j] = take(tc);
+    w.l1 = take((size_t)(m->lora_w + m->lora_a + m->lora_v + m->lora_g) * 2);
     w.lw = take((size_t)T * m->lora_w * 2); w.la = take((size_t)T * m->lora_a * 2);
     w.lv = take((size_t)T * m->lora_v * 2); w.lg = take((size_t)T * m->lora_g * 2);
     w.w_raw = take(tc); w.a_raw = take(tc); w.vg_raw = take(tc); w.g = take(tc);
@@ -205,7 +446,9 @@ extern "C" int rwkv_wkv7_forward(int64_t B, int64_t T, int64_t C, int64_t H, flo
     int rc = wkv7_check(B, T, C, H);
     if (rc) return rc;
     if (dtype != RWKV_DT_F16 && dtype != RWKV_DT_F32) return RWKV_E_DTYPE;
-    if (!aligned16(state)) return RWKV_E_LAYOUT;
+    if (!aligned16(state) || !aligned16(r) || !aligned16(w) || !aligned16(k) || !aligned16(a) || !aligned16(b) ||
+        (((uintptr_t)v) & 3))
+        return RWKV_E_LAYOUT;
     Wkv7Args q{(int)T, (int)C, state, r, w, k, v, a, b, y};
     const dim3 grid((unsigned)(4 * H)), block(256);
     if (dtype == RWKV_DT_F16) hipLaunchKernelGGL((wkv7_kernel<true, false>), grid, block, 0, (hipStream_t)stream, q);
@@ -225,10 +468,11 @@ static int v7_check(const rwkv_v7_model *m) {
         if (ranks[j] <= 0 || (ranks[j] & 63) || ranks[j] > 8 * DTHREADS) return RWKV_E_SHAPE;
     for (int i = 0; i < m->n_layer; ++i) {
         const rwkv_v7_layer &l = m->layers[i];
-        if (!l.ln1_w || !l.ln1_b || !l.ln2_w || !l.ln2_b || !l.w0 || !l.a0 || !l.w1 || !l.w2 || !l.a1 || !l.a2 ||
-            !l.g1 || !l.g2 || !l.k_k || !l.k_a || !l.r_k || !l.lnx_w || !l.lnx_b || !l.ffn_x_k)
+        if (!l.ln1_w || !l.ln1_b || !l.ln2_w || !l.ln2_b || !l.w0 || !l.a0 || !l.lora1 || !l.lora2 || !l.k_k ||
+            !l.k_a || !l.r_k || !l.lnx_w || !l.lnx_b || !l.ffn_x_k)
             return RWKV_E_NULL;
-        if (i > 0 && (!l.v0 || !l.v1 || !l.v2)) return RWKV_E_NULL;
+        if (i > 0 && !l.v0) return RWKV_E_NULL;
+        if (!aligned16(l.lora1) || !aligned16(l.lora2)) return RWKV_E_LAYOUT;
         for (int j = 0; j < 6; ++j)
             if (!l.x_mix[j]) return RWKV_E_NULL;
         if (!mat_ok7(l.att_receptance, C, C) || !mat_ok7(l.att_key, C, C) || !mat_ok7(l.att_value, C, C) ||
@@ -264,10 +508,55 @@ extern "C" int rwkv_v7_forward(const rwkv_v7_model *m, const rwkv_v56_layer_stat
     Ctx c{st, false, T, num_cu(), nullptr, nullptr, nullptr, ws.splitk};
     const unsigned head_waves = (unsigned)(((int64_t)T * H + 3) / 4);
 
+    const int max_rank = std::max(std::max(m->lora_w, m->lora_a), std::max(m->lora_v, m->lora_g));
+    const int o_a = m->lora_w, o_v = o_a + m->lora_a, o_g = o_v + m->lora_v, rtot = o_g + m->lora_g;
+    // block j of the stacked LoRA matrices as matrices of their own
+    auto lora_first = [&](const rwkv_v7_layer &l, int off, int d) { return lora_mat(l.lora1 + (size_t)off * C, C, d); };
+    auto lora_second = [&](const rwkv_v7_layer &l, int off, int d) {
+        rwkv_mat q{};
+        q.w = l.lora2 + off; q.ld = rtot; q.N = d; q.M = C;
+        return q;
+    };
+
     if ((rc = gather_emb_launch(T, C, tokens, m->emb, ws.x, st))) return rc;
     for (int i = 0; i < m->n_layer; ++i) {
         const rwkv_v7_layer &l = m->layers[i];
         const rwkv_v56_layer_state &s = states[i];
+        // one token: the six mixed activation vectors must fit the default LDS window, a LoRA row one request per wave
+        if (T == 1 && C <= 5120 && max_rank <= 512) {
+            rwkv_half *v1 = i == 0 ? ws.v_first : ws.v;
+            {
+                Att7Args a{};
+                a.x = ws.x; a.C = C; a.ln_w = l.ln1_w; a.ln_b = l.ln1_b; a.sx = s.att_xx; a.xx_tmp = ws.xx_att;
+                for (int j = 0; j < 6; ++j) a.mix[j] = l.x_mix[j];
+                a.mat[0] = to_dev56(l.att_receptance); a.mat[1] = to_dev56(l.att_key); a.mat[2] = to_dev56(l.att_value);
+                a.out[0] = ws.r; a.out[1] = ws.k; a.out[2] = v1;
+                a.lora1 = l.lora1; a.rtot = rtot; a.o_a = o_a; a.o_v = o_v; a.o_g = o_g; a.l1 = ws.l1;
+                hipLaunchKernelGGL(att7_kernel, dim3(c.grid), dim3(DTHREADS), 6 * (size_t)C * 2, st, a);
+            }
+            {
+                Tmix7Args a{};
+                a.C = C; a.rtot = rtot; a.o_a = o_a; a.o_v = o_v; a.o_g = o_g;
+                a.d_w = m->lora_w; a.d_a = m->lora_a; a.d_v = m->lora_v; a.d_g = m->lora_g;
+                a.first_layer = i == 0; a.l1 = ws.l1; a.lora2 = l.lora2;
+                a.r = ws.r; a.k = ws.k; a.v = v1; a.v_first = ws.v_first;
+                a.w0 = l.w0; a.a0 = l.a0; a.v0 = l.v0; a.k_k = l.k_k; a.k_a = l.k_a; a.r_k = l.r_k;
+                a.lnx_w = l.lnx_w; a.lnx_b = l.lnx_b; a.state = s.att_kv; a.out = ws.att;
+                a.commit_src = ws.xx_att; a.commit_dst = s.att_xx;
+                hipLaunchKernelGGL(tmix7_kernel, dim3((unsigned)H), dim3(1024), 0, st, a);
+            }
+            if ((rc = mm(c, l.att_output, false, ws.att, ACT_RESIDUAL, ws.x, nullptr, 1.f, ws.x))) return rc;
+            {
+                LnMixArgs a{};
+                a.x = ws.x; a.C = C; a.ln_w = l.ln2_w; a.ln_b = l.ln2_b; a.sx = s.ffn_xx; a.xx_tmp = ws.xx_ffn;
+                a.mix[0] = l.ffn_x_k; a.mat[0] = to_dev56(l.ffn_key); a.M[0] = (int)l.ffn_key.M; a.epi[0] = EPI_RELU_SQ;
+                a.out[0] = ws.vx; a.maa_form = 1;
+                lnmix1_launch(false, a, c.grid, st);
+            }
+            if ((rc = mm(c, l.ffn_value, false, ws.vx, ACT_RESIDUAL, ws.x, nullptr, 1.f, ws.x, ws.xx_ffn, s.ffn_xx, C))) return rc;
+            RWKV_LAUNCH_CHECK();
+            continue;
+        }
         {
             SeqMixArgs a{};
             a.T = (int)T; a.C = C; a.x = ws.x; a.ln_w = l.ln1_w; a.ln_b = l.ln1_b; a.sx = s.att_xx;
@@ -282,16 +571,16 @@ extern "C" int rwkv_v7_forward(const rwkv_v7_model *m, const rwkv_v56_layer_stat
         if ((rc = mm(c, l.att_receptance, false, xr, ACT_NONE, nullptr, nullptr, 1.f, ws.r, ws.xx_att, s.att_xx, C))) return rc;
         if ((rc = mm(c, l.att_key, false, xk, ACT_NONE, nullptr, nullptr, 1.f, ws.k))) return rc;
         if ((rc = mm(c, l.att_value, false, xv, ACT_NONE, nullptr, nullptr, 1.f, v))) return rc;
-        if ((rc = mm(c, lora_mat(l.w1, C, m->lora_w), false, xw, ACT_TANH, nullptr, nullptr, 1.f, ws.lw))) return rc;
-        if ((rc = mm(c, lora_mat(l.w2, m->lora_w, C), false, ws.lw, ACT_NONE, nullptr, nullptr, 1.f, ws.w_raw))) return rc;
-        if ((rc = mm(c, lora_mat(l.a1, C, m->lora_a), false, xa, ACT_NONE, nullptr, nullptr, 1.f, ws.la))) return rc;
-        if ((rc = mm(c, lora_mat(l.a2, m->lora_a, C), false, ws.la, ACT_NONE, nullptr, nullptr, 1.f, ws.a_raw))) return rc;
+        if ((rc = mm(c, lora_first(l, 0, m->lora_w), false, xw, ACT_TANH, nullptr, nullptr, 1.f, ws.lw))) return rc;
+        if ((rc = mm(c, lora_second(l, 0, m->lora_w), false, ws.lw, ACT_NONE, nullptr, nullptr, 1.f, ws.w_raw))) return rc;
+        if ((rc = mm(c, lora_first(l, o_a, m->lora_a), false, xa, ACT_NONE, nullptr, nullptr, 1.f, ws.la))) return rc;
+        if ((rc = mm(c, lora_second(l, o_a, m->lora_a), false, ws.la, ACT_NONE, nullptr, nullptr, 1.f, ws.a_raw))) return rc;
         if (i > 0) {
-            if ((rc = mm(c, lora_mat(l.v1, C, m->lora_v), false, xv, ACT_NONE, nullptr, nullptr, 1.f, ws.lv))) return rc;
-            if ((rc = mm(c, lora_mat(l.v2, m->lora_v, C), false, ws.lv, ACT_NONE, nullptr, nullptr, 1.f, ws.vg_raw))) return rc;
+            if ((rc = mm(c, lora_first(l, o_v, m->lora_v), false, xv, ACT_NONE, nullptr, nullptr, 1.f, ws.lv))) return rc;
+            if ((rc = mm(c, lora_second(l, o_v, m->lora_v), false, ws.lv, ACT_NONE, nullptr, nullptr, 1.f, ws.vg_raw))) return rc;
         }
-        if ((rc = mm(c, lora_mat(l.g1, C, m->lora_g), false, xg, ACT_SIGMOID, nullptr, nullptr, 1.f, ws.lg))) return rc;
-        if ((rc = mm(c, lora_mat(l.g2, m->lora_g, C), false, ws.lg, ACT_NONE, nullptr, nullptr, 1.f, ws.g))) return rc;
+        if ((rc = mm(c, lora_first(l, o_g, m->lora_g), false, xg, ACT_SIGMOID, nullptr, nullptr, 1.f, ws.lg))) return rc;
+        if ((rc = mm(c, lora_second(l, o_g, m->lora_g), false, ws.lg, ACT_NONE, nullptr, nullptr, 1.f, ws.g))) return rc;
         {
             Prep7Args a{};
             a.T = (int)T; a.C = C; a.H = H; a.r = ws.r; a.k = ws.k; a.v = v; a.w_raw = ws.w_raw; a.a_raw = ws.a_raw;

@@ -91,7 +91,7 @@ class RwkvV7Layer(ctypes.Structure):
     _fields_ = [("ln1_w", _vp), ("ln1_b", _vp), ("ln2_w", _vp), ("ln2_b", _vp),
                 ("x_mix", _vp * 6),
                 ("w0", _vp), ("a0", _vp), ("v0", _vp),
-                ("w1", _vp), ("w2", _vp), ("a1", _vp), ("a2", _vp), ("v1", _vp), ("v2", _vp), ("g1", _vp), ("g2", _vp),
+                ("lora1", _vp), ("lora2", _vp),
                 ("k_k", _vp), ("k_a", _vp), ("r_k", _vp), ("lnx_w", _vp), ("lnx_b", _vp),
                 ("att_receptance", RwkvMat), ("att_key", RwkvMat), ("att_value", RwkvMat), ("att_output", RwkvMat),
                 ("ffn_x_k", _vp), ("ffn_key", RwkvMat), ("ffn_value", RwkvMat)]

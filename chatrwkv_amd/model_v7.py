@@ -102,25 +102,12 @@ class RWKV_x070:
         return m
 
     def _build_descriptors(self):
-        """LoRA matrices are laid out input-contiguous with the rank padded with zeros to a multiple of
-        64: first stages [rank][C] (the checkpoint's [C, rank] transposed), second stages [C][rank]."""
+        """The four LoRA pairs of a layer are concatenated, every rank padded with zeros to a multiple of
+        64: first stages as row blocks of one [R][C] matrix (the checkpoint's [C, rank] transposed),
+        second stages as column blocks of one [C][R] matrix."""
         a, z, dev = self.args, self.z, self.device
         C = a.n_embd
         keep = self._keep = []
-
-        def first(name, rank):
-            t = z[name]                                               # [C, r]
-            p = torch.zeros((rank, C), dtype=torch.float16, device=dev)
-            p[:t.shape[1]] = t.t()
-            keep.append(p)
-            return p.data_ptr()
-
-        def second(name, rank):
-            t = z[name]                                               # [r, C]
-            p = torch.zeros((C, rank), dtype=torch.float16, device=dev)
-            p[:, :t.shape[0]] = t.t()
-            keep.append(p)
-            return p.data_ptr()
 
         ranks = [_pad64(z['blocks.0.att.' + n + '1'].shape[1]) for n in 'wa'] + \
                 [_pad64(z['blocks.1.att.v1'].shape[1]) if a.n_layer > 1 else 64,
@@ -134,12 +121,19 @@ class RWKV_x070:
             for j, c in enumerate('rwkvag'):
                 l.x_mix[j] = z[at + 'x_' + c].data_ptr()
             l.w0, l.a0 = z[at + 'w0'].data_ptr(), z[at + 'a0'].data_ptr()
-            l.w1, l.w2 = first(at + 'w1', ranks[0]), second(at + 'w2', ranks[0])
-            l.a1, l.a2 = first(at + 'a1', ranks[1]), second(at + 'a2', ranks[1])
-            if i > 0:                                                 # layer 0 ignores them (model.py:279-281, 505)
+            l1 = torch.zeros((sum(ranks), C), dtype=torch.float16, device=dev)
+            l2 = torch.zeros((C, sum(ranks)), dtype=torch.float16, device=dev)
+            off = 0
+            for n, rank in zip('wavg', ranks):
+                if not (n == 'v' and i == 0):                         # layer 0 ignores v0, v1, v2 (model.py:279-281, 505)
+                    t1, t2 = z[at + n + '1'], z[at + n + '2']         # [C, r], [r, C]
+                    l1[off:off + t1.shape[1]] = t1.t()
+                    l2[:, off:off + t2.shape[0]] = t2.t()
+                off += rank
+            keep += [l1, l2]
+            l.lora1, l.lora2 = l1.data_ptr(), l2.data_ptr()
+            if i > 0:
                 l.v0 = z[at + 'v0'].data_ptr()
-                l.v1, l.v2 = first(at + 'v1', ranks[2]), second(at + 'v2', ranks[2])
-            l.g1, l.g2 = first(at + 'g1', ranks[3]), second(at + 'g2', ranks[3])
             l.k_k, l.k_a, l.r_k = z[at + 'k_k'].data_ptr(), z[at + 'k_a'].data_ptr(), z[at + 'r_k'].data_ptr()
             l.lnx_w, l.lnx_b = z[at + 'ln_x.weight'].data_ptr(), z[at + 'ln_x.bias'].data_ptr()
             l.att_receptance, l.att_key = self._mat(at + 'receptance.weight'), self._mat(at + 'key.weight')

@@ -287,15 +287,18 @@ int rwkv_wkv7_forward(int64_t B, int64_t T, int64_t C, int64_t H, float *state, 
  * forward_one / forward_seq (model.py:336-363, 457-487), RWKV_x070_TMix_one / _seq (model.py:492-572),
  * RWKV_x070_CMix_one / _seq (model.py:597-608) and RWKV7_OP (model.py:198-219).  The reference runs RWKV-7
  * in fp16, bf16 or fp32 without quantisation (model.py:236-243); this entry point is the fp16 one.  Head
- * size must be 64.  LoRA matrices are fp16, input-contiguous like the model matrices: first stages
- * [rank][C] (the checkpoint's [C, rank] transposed), second stages [C][rank]; every rank is padded with
- * zeros to a multiple of 64.
+ * size must be 64.  The four LoRA pairs (decay w, in-context rate a, value residual v, gate g) are fp16
+ * and input-contiguous like the model matrices, every rank padded with zeros to a multiple of 64 and the
+ * four concatenated in the order w, a, v, g (R = lora_w + lora_a + lora_v + lora_g):
+ *   lora1 [R][C]   first stages: the checkpoint's w1, a1, v1, g1 ([C, rank]) transposed, row blocks stacked
+ *   lora2 [C][R]   second stages: w2, a2, v2, g2 ([rank, C]) transposed, column blocks side by side
+ * Layer 0 has no value residual (model.py:279-281, 505): its v blocks are ignored.
  */
 typedef struct {
     const rwkv_half *ln1_w, *ln1_b, *ln2_w, *ln2_b;      /* [C] */
     const rwkv_half *x_mix[6];                            /* att.x_r, x_w, x_k, x_v, x_a, x_g [C] */
     const rwkv_half *w0, *a0, *v0;                        /* [C]; v0 unused in layer 0 */
-    const rwkv_half *w1, *w2, *a1, *a2, *v1, *v2, *g1, *g2; /* LoRA pairs; v1, v2 unused in layer 0 */
+    const rwkv_half *lora1, *lora2;                       /* [R][C], [C][R] */
     const rwkv_half *k_k, *k_a, *r_k;                     /* [C] */
     const rwkv_half *lnx_w, *lnx_b;                       /* [C] GroupNorm affine */
     rwkv_mat att_receptance, att_key, att_value, att_output;

@@ -176,6 +176,12 @@ def test_v7_long_prompt_and_odd_lora_ranks():
         d = float(np.abs(_np(out) - oo.astype(np.float32)).max())
         assert d <= LOGIT_TOL, d
         assert _argmax_agree(_np(out), oo.astype(np.float32), d)
+    # one-token steps (the fused one-token kernels) continue from the same state
+    for t in synth.random_tokens(4, cfg["vocab"], seed=10):
+        out, st = m.forward([t], st)
+        oo, ost = o.forward([t], ost)
+        d = float(np.abs(_np(out) - oo.astype(np.float32)).max())
+        assert d <= LOGIT_TOL, d
     for i, (s, ref) in enumerate(zip(st, ost)):
         scale = max(float(np.abs(ref.astype(np.float32)).max()), 1.0)
         assert np.abs(_np(s) - ref.astype(np.float32)).max() <= 1e-2 * scale, i
