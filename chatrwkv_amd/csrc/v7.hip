@@ -177,28 +177,41 @@ __global__ __launch_bounds__(256) void wkv7_kernel(Wkv7Args a) {
         }
         __syncthreads();
         fetch(t0 + TS7);
-        for (int tt = 0; tt < nt; ++tt) {
-            const float vi = sv[tt][il], kr = skr[tt], br = sbr[tt];
-            const f32x4 wr4 = *(const f32x4 *)&swr[tt][4 * g];
-            const f32x4 k4 = *(const f32x4 *)&sk[tt][4 * g];
-            const f32x4 w4 = *(const f32x4 *)&sw[tt][4 * g];
-            const f32x4 a4 = *(const f32x4 *)&sa[tt][4 * g];
-            const f32x4 b4 = *(const f32x4 *)&sb[tt][4 * g];
-            float p = (a4[0] * s[0] + a4[1] * s[1]) + (a4[2] * s[2] + a4[3] * s[3]);
-            float yw = (wr4[0] * s[0] + wr4[1] * s[1]) + (wr4[2] * s[2] + wr4[3] * s[3]);
+        struct Tok { float vi, kr, br; f32x4 wr4, k4, w4, a4, b4; };
+        auto ldtok = [&](int tt) {
+            Tok q;
+            q.vi = sv[tt][il]; q.kr = skr[tt]; q.br = sbr[tt];
+            q.wr4 = *(const f32x4 *)&swr[tt][4 * g];
+            q.k4 = *(const f32x4 *)&sk[tt][4 * g];
+            q.w4 = *(const f32x4 *)&sw[tt][4 * g];
+            q.a4 = *(const f32x4 *)&sa[tt][4 * g];
+            q.b4 = *(const f32x4 *)&sb[tt][4 * g];
+            return q;
+        };
+        auto step = [&](const Tok &q, int tt) {
+            float p = (q.a4[0] * s[0] + q.a4[1] * s[1]) + (q.a4[2] * s[2] + q.a4[3] * s[3]);
+            float yw = (q.wr4[0] * s[0] + q.wr4[1] * s[1]) + (q.wr4[2] * s[2] + q.wr4[3] * s[3]);
             f32x4 kv;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) kv[e] = s[e] * w4[e] + k4[e] * vi;
+            for (int e = 0; e < 4; ++e) kv[e] = s[e] * q.w4[e] + q.k4[e] * q.vi;
             p = row16_sum(p);
             yw = row16_sum(yw);
 #pragma unroll
-            for (int e = 0; e < 4; ++e) s[e] = kv[e] + p * b4[e];
+            for (int e = 0; e < 4; ++e) s[e] = kv[e] + p * q.b4[e];
             if (g == 0) {
-                const float y = yw + vi * kr + p * br;
+                const float y = yw + q.vi * q.kr + p * q.br;
                 const size_t o = (size_t)(t0 + tt) * C + h * HS7 + i;
                 if (MODEL || !IN_F16) ((float *)a.y)[o] = y;
                 else ((rwkv_half *)a.y)[o] = f2h(y);
             }
+        };
+        // four tokens per pass: their LDS reads are issued together, so the read latency is paid once per four
+        for (int tt = 0; tt < nt; tt += 4) {
+            const Tok q0 = ldtok(tt), q1 = ldtok(tt + 1), q2 = ldtok(tt + 2), q3 = ldtok(tt + 3);
+            step(q0, tt);
+            if (tt + 1 < nt) step(q1, tt + 1);
+            if (tt + 2 < nt) step(q2, tt + 2);
+            if (tt + 3 < nt) step(q3, tt + 3);
         }
     }
     *(f32x4 *)S = s;

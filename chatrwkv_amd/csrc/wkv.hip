@@ -358,6 +358,9 @@ __global__ __launch_bounds__(256) void wkv56_split_kernel(Wkv56Args a) {
     const int lane = threadIdx.x & 63, g = lane & 15;
     const int il = (threadIdx.x >> 6) * 4 + (lane >> 4);   // value column within the block of 16
     const int i = vb * 16 + il;
+    // staging role: token threadIdx.x / 8 of the slab, channels 8 (threadIdx.x % 8) .. + 7 of the head.  The
+    // NEXT slab is fetched into registers before the token loop of the current one, which hides the loads.
+    const int stt = threadIdx.x >> 3, sp = threadIdx.x & 7, sc = sp * 8;
     float *S = a.state + (size_t)h * HS * HS;               // [key][value]
     float s[4], u4[4], wc[4];
 #pragma unroll
@@ -367,37 +370,66 @@ __global__ __launch_bounds__(256) void wkv56_split_kernel(Wkv56Args a) {
         u4[e] = a.u[h * HS + j];
         wc[e] = WMODE == 0 ? ((const float *)a.w)[h * HS + j] : 0.f;
     }
-    const float tdec = WMODE == 2 ? a.t_decay[h * HS + (threadIdx.x & 63)] : 0.f;
+    float tdec[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) tdec[e] = WMODE == 2 ? a.t_decay[h * HS + sc + e] : 0.f;
+    h16x8 pr, pk, pw = {};
+    h16x2 pv;
+    auto fetch = [&](int t0) {
+        const size_t o = (size_t)min(t0 + stt, T - 1) * C + h * HS;   // rows past the end re-read the last one
+        pr = *(const h16x8 *)((const rwkv_half *)a.r + o + sc);
+        pk = *(const h16x8 *)((const rwkv_half *)a.k + o + sc);
+        if (WMODE == 2) pw = *(const h16x8 *)((const rwkv_half *)a.w + o + sc);
+        pv = *(const h16x2 *)((const rwkv_half *)a.v + o + vb * 16 + 2 * sp);
+    };
+    fetch(0);
     for (int t0 = 0; t0 < T; t0 += TS2) {
         const int nt = min(TS2, T - t0);
         __syncthreads();  // previous slab fully consumed
-        for (int e = threadIdx.x; e < nt * HS; e += 256) {
-            const int tt = e >> 6, c = e & 63;               // c == threadIdx.x & 63
-            const size_t o = (size_t)(t0 + tt) * C + h * HS + c;
-            sr[tt][c] = h2f(((const rwkv_half *)a.r)[o]);
-            sk[tt][c] = h2f(((const rwkv_half *)a.k)[o]);
-            if (WMODE == 2) sw[tt][c] = expf(-expf(tdec + h2f(((const rwkv_half *)a.w)[o])));
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            f32x4 r4, k4, w4;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                r4[e] = (float)pr[4 * u + e];
+                k4[e] = (float)pk[4 * u + e];
+                w4[e] = WMODE == 2 ? expf(-expf(tdec[4 * u + e] + (float)pw[4 * u + e])) : 0.f;
+            }
+            *(f32x4 *)&sr[stt][sc + 4 * u] = r4;
+            *(f32x4 *)&sk[stt][sc + 4 * u] = k4;
+            if (WMODE == 2) *(f32x4 *)&sw[stt][sc + 4 * u] = w4;
         }
-        for (int e = threadIdx.x; e < nt * 16; e += 256) {
-            const int tt = e >> 4, c = e & 15;
-            sv[tt][c] = h2f(((const rwkv_half *)a.v)[(size_t)(t0 + tt) * C + h * HS + vb * 16 + c]);
-        }
+        sv[stt][2 * sp] = (float)pv[0];
+        sv[stt][2 * sp + 1] = (float)pv[1];
         __syncthreads();
-        for (int tt = 0; tt < nt; ++tt) {
-            const float vi = sv[tt][il];
-            const f32x4 r4 = *(const f32x4 *)&sr[tt][4 * g];
-            const f32x4 k4 = *(const f32x4 *)&sk[tt][4 * g];
-            f32x4 w4;
-            if (WMODE == 2) w4 = *(const f32x4 *)&sw[tt][4 * g];
+        fetch(t0 + TS2);
+        struct Tok { float vi; f32x4 r4, k4, w4; };
+        auto ldtok = [&](int tt) {
+            Tok q;
+            q.vi = sv[tt][il];
+            q.r4 = *(const f32x4 *)&sr[tt][4 * g];
+            q.k4 = *(const f32x4 *)&sk[tt][4 * g];
+            q.w4 = WMODE == 2 ? *(const f32x4 *)&sw[tt][4 * g] : f32x4{};
+            return q;
+        };
+        auto step = [&](const Tok &q, int tt) {
             float y = 0.f;
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                const float x = k4[e] * vi;
-                y += r4[e] * (u4[e] * x + s[e]);
-                s[e] = s[e] * (WMODE == 2 ? w4[e] : wc[e]) + x;
+                const float x = q.k4[e] * q.vi;
+                y += q.r4[e] * (u4[e] * x + s[e]);
+                s[e] = s[e] * (WMODE == 2 ? q.w4[e] : wc[e]) + x;
             }
             y = row16_sum(y);
             if (g == 0) a.y[(size_t)(t0 + tt) * C + h * HS + i] = y;
+        };
+        // four tokens per pass: their LDS reads are issued together, so the read latency is paid once per four
+        for (int tt = 0; tt < nt; tt += 4) {
+            const Tok q0 = ldtok(tt), q1 = ldtok(tt + 1), q2 = ldtok(tt + 2), q3 = ldtok(tt + 3);
+            step(q0, tt);
+            if (tt + 1 < nt) step(q1, tt + 1);
+            if (tt + 2 < nt) step(q2, tt + 2);
+            if (tt + 3 < nt) step(q3, tt + 3);
         }
     }
 #pragma unroll
