@@ -9,7 +9,8 @@ rebuild the same model from a seed instead of shipping weights.
 Distributions: 2-D matrices (emb, head, key/value/receptance/gate/output)
 N(0, 0.02); time_decay U[-6,-1]; time_first / time_faaaa U[-1,1];
 time_mix_* / time_maa_* U[0,1]; LayerNorm / GroupNorm weight 1, bias 0;
-RWKV-6 LoRA matrices N(0, 0.01).
+RWKV-6 LoRA matrices N(0, 0.01).  ``make_checkpoint_v7`` writes RWKV-7 checkpoints (its own key set,
+non-trivial LayerNorm / GroupNorm affines and LoRA matrices large enough to matter).
 
 Two generators:
   * ``numpy`` (default): PCG64 streams keyed by (seed, crc32(tensor name)).
