@@ -529,7 +529,14 @@ struct MultiVecArgs {
     const rwkv_half *commit_src; // scratch xx -> token-shift state, done by workgroup 0
     rwkv_half *commit_dst;
     int commit_n;
+    // optional extra product after the NM matrices: tanh(xin @ X) for a small fp16 matrix X of xm rows [xm][N]
+    // (RWKV-6: the first decay-LoRA stage), NULL = none
+    const rwkv_half *xin, *xmat;
+    int xm;
+    rwkv_half *xout;             // [xm]
 };
+
+struct NoEpi {};
 
 // NM input vectors of N <= 4096 elements (one 8-element group per thread of the first 8 waves).
 template <bool U8, int NM>
@@ -540,13 +547,15 @@ __global__ __launch_bounds__(DTHREADS) void multi_vec_kernel(MultiVecArgs a) {
     h16 *xs[NM];
 #pragma unroll
     for (int j = 0; j < NM; ++j) xs[j] = (h16 *)smem + (size_t)j * N;
+    h16 *xs_x = (h16 *)smem + (size_t)NM * N;   // input of the extra product, plain layout
     VecSums S[NM];
-    h16x8 pv[NM], pr[NM], pm[NM];
+    h16x8 pv[NM], pr[NM], pm[NM], px = {};
     const bool own = (int)threadIdx.x < (N >> 3);
     auto pro_load = [&]() {
 #pragma unroll
         for (int j = 0; j < NM; ++j) pv[j] = pr[j] = pm[j] = h16x8{};
         if (!own) return;
+        px = *(const h16x8 *)((a.xin ? a.xin : a.vin[0]) + 8 * threadIdx.x);
 #pragma unroll
         for (int j = 0; j < NM; ++j) {
             pv[j] = *(const h16x8 *)(a.vin[j] + 8 * threadIdx.x);
@@ -577,6 +586,7 @@ __global__ __launch_bounds__(DTHREADS) void multi_vec_kernel(MultiVecArgs a) {
             }
             if (own) ((h16x8 *)xs[j])[xs_item<U8>(threadIdx.x, nseg)] = o;
         }
+        if (own) ((h16x8 *)xs_x)[threadIdx.x] = px;
         block_sum_1b<3 * NM>(acc, red);  // the barrier also publishes xs
         if (U8)
 #pragma unroll
@@ -611,13 +621,22 @@ __global__ __launch_bounds__(DTHREADS) void multi_vec_kernel(MultiVecArgs a) {
         }
     };
     stream_rows<U8, 1, NM, 2, Epi>(M, (N * (U8 ? 1 : 2)) >> 4, pro_owner_wave(N >> 3), pro_load, pro_compute, rowf, epi_load, epi);
+    if (a.xmat) {
+        auto rowf2 = [&](int g, int, const uint8_t *&row, const h16 *&xv) {
+            row = (const uint8_t *)(a.xmat + (size_t)g * N);
+            xv = xs_x;
+        };
+        auto epi_load2 = [&](int) { return NoEpi{}; };
+        auto epi2 = [&](int g, const float (&d)[1], const NoEpi &) { a.xout[g] = f2h(tanhf(round_h(d[0]))); };
+        stream_rows<false, 1, 1, 2, NoEpi>(a.xm, (N * 2) >> 4, false, [] {}, [] {}, rowf2, epi_load2, epi2);
+    }
     if (blockIdx.x == 0 && a.commit_dst)
         for (int j8 = threadIdx.x; j8 < (a.commit_n >> 3); j8 += blockDim.x)
             *(u32x4 *)(a.commit_dst + 8 * j8) = *(const u32x4 *)(a.commit_src + 8 * j8);
 }
 
 inline void multi_vec_launch(bool u8, const MultiVecArgs &a, int grid, hipStream_t st) {
-    const size_t lds = (size_t)a.nm * a.N * 2;
+    const size_t lds = (size_t)(a.nm + 1) * a.N * 2;
     if (a.nm == 4) {
         if (u8) hipLaunchKernelGGL((multi_vec_kernel<true, 4>), dim3(grid), dim3(DTHREADS), lds, st, a);
         else hipLaunchKernelGGL((multi_vec_kernel<false, 4>), dim3(grid), dim3(DTHREADS), lds, st, a);

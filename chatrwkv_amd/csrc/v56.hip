@@ -216,6 +216,7 @@ extern "C" int rwkv_v56_forward(const rwkv_v56_model *m, const rwkv_v56_layer_st
         const rwkv_v56_layer &l = m->layers[i];
         const rwkv_v56_layer_state &s = states[i];
         const rwkv_half *kx, *vx, *rx, *gx = nullptr, *wx = nullptr;
+        bool fuse_d1 = false;
         if (v6) {
             Mix2Args b{};
             if (T == 1) {
@@ -237,7 +238,9 @@ extern "C" int rwkv_v56_forward(const rwkv_v56_model *m, const rwkv_v56_layer_st
             if (T == 1) hipLaunchKernelGGL(v6_mix2_kernel<1>, dim3(1, (unsigned)((C + 255) / 256), 5), dim3(256), 0, st, b);
             else hipLaunchKernelGGL(v6_mix2_kernel<16>, dim3((unsigned)((T + 15) / 16), (unsigned)((C + 255) / 256), 5), dim3(256), 0, st, b);
             wx = ws.mix[0]; kx = ws.mix[1]; vx = ws.mix[2]; rx = ws.mix[3]; gx = ws.mix[4];
-            if ((rc = mm(c, lora_mat(l.td_w1, C, ld), false, wx, ACT_TANH, nullptr, nullptr, 1.f, ws.d1))) return rc;
+            // one token: the first decay-LoRA stage rides at the end of the receptance / key / value / gate launch
+            fuse_d1 = T == 1 && C <= 8 * 512;
+            if (!fuse_d1 && (rc = mm(c, lora_mat(l.td_w1, C, ld), false, wx, ACT_TANH, nullptr, nullptr, 1.f, ws.d1))) return rc;
             if (T > 1 && (rc = mm(c, lora_mat(l.td_w2, ld, C), false, ws.d1, ACT_NONE, nullptr, nullptr, 1.f, ws.d2))) return rc;
         } else {
             SeqMixArgs a{};
@@ -258,6 +261,7 @@ extern "C" int rwkv_v56_forward(const rwkv_v56_model *m, const rwkv_v56_layer_st
             a.vin[2] = vx; a.mat[2] = to_dev56(l.att_value); a.act[2] = VACT_F16; a.out[2] = ws.v;
             if (gated) { a.vin[3] = gx; a.mat[3] = to_dev56(l.att_gate); a.act[3] = VACT_SILU; a.out[3] = ws.g; }
             a.commit_src = ws.xx_att; a.commit_dst = s.att_xx; a.commit_n = C;
+            if (fuse_d1) { a.xin = wx; a.xmat = l.td_w1; a.xm = ld; a.xout = ws.d1; }
             multi_vec_launch(u8, a, c.grid, st);
         } else {
             if ((rc = mm(c, l.att_receptance, u8, rx, ACT_NONE, nullptr, nullptr, 1.f, ws.r, ws.xx_att, s.att_xx, C))) return rc;

@@ -255,8 +255,6 @@ struct Att7Args {
     rwkv_half *l1;             // [rtot] activated first-stage outputs
 };
 
-struct NoEpi {};
-
 __global__ __launch_bounds__(DTHREADS) void att7_kernel(Att7Args a) {
     extern __shared__ __align__(16) unsigned char smem[];
     __shared__ float red[(2 + 3 * 6) * DWAVES];
