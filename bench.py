@@ -16,6 +16,8 @@ One JSON line is printed:
                         the 8 TB/s HBM peak
   decode_hbm            whole-step figure: uint8 weight bytes per token x tokens/s / 8 TB/s
   prefill               prefill tokens/s and the MFMA fraction of the whole prefill
+  prefill_roofline      the prefill contraction alone on the model's largest matrix shape: 2 T N M flops /
+                        mean launch duration (HIP events), against the 2.5 PFLOP/s dense fp16 MFMA peak
   cpu_baseline          the oracle's 'cpu fp32i8' path (numpy port of the reference's CPU arithmetic)
                         timed on this host: a bounded sample at the 7B shape, extrapolated per token
 """
@@ -89,6 +91,53 @@ def cpu_baseline(shape, budget_s=25.0):
                    f"t_layer {t_layer * 1e3:.0f} ms, t_head {t_head * 1e3:.0f} ms, "
                    f"per token = {L} x t_layer + t_head = {per_token:.2f} s; setup {setup:.0f} s"),
     }
+
+
+def gemm_roofline(T, N, M, u8, reps=10):
+    """The prefill contraction alone on the model's largest matrix shape (channel-mix key, [T, N] x [N, M]),
+    through the C ABI (rwkv_mm8_seq_f16 incl. its activation-scaling pass, or rwkv_gemm_f16), timed with two
+    events on the stream it is launched on: algorithmic flops 2 T N M over the mean launch time against the
+    dense fp16 MFMA peak."""
+    import torch
+    from chatrwkv_amd import lib
+    L = lib.load()
+    dev = "cuda:0"
+    x = torch.randn(T, N, device=dev).half()
+    y = torch.empty(T, M, device=dev, dtype=torch.float16)
+    st = torch.cuda.current_stream().cuda_stream
+    if u8:
+        w = torch.randint(0, 256, (M, N), dtype=torch.uint8, device=dev)
+        mx = torch.randn(M, device=dev).half(); rx = (torch.rand(M, device=dev) * 0.01).half()
+        my = torch.randn(N, device=dev).half(); ry = (torch.rand(N, device=dev) * 0.06).half()
+        nbytes = L.rwkv_mm8_seq_workspace(T, N)
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+
+        def run():
+            lib.check(L.rwkv_mm8_seq_f16(T, N, M, x.data_ptr(), N, w.data_ptr(), 1, N, mx.data_ptr(), rx.data_ptr(),
+                                         my.data_ptr(), ry.data_ptr(), y.data_ptr(), M, ws.data_ptr(), nbytes, st),
+                      "rwkv_mm8_seq_f16")
+        name = "gemm_kernel<uint8 weights, 128x128 tile> + mm8_prepare_kernel"
+    else:
+        w = torch.randn(M, N, device=dev).half()
+
+        def run():
+            lib.check(L.rwkv_gemm_f16(T, N, M, x.data_ptr(), N, w.data_ptr(), 1, N, y.data_ptr(), M, lib.RWKV_DT_F16, st),
+                      "rwkv_gemm_f16")
+        name = "gemm_kernel<fp16 weights, 128x128 tile>"
+    for _ in range(3):
+        run()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    e0.record()
+    for _ in range(reps):
+        run()
+    e1.record()
+    torch.cuda.synchronize()
+    t = e0.elapsed_time(e1) * 1e-3 / reps
+    flops = 2.0 * T * N * M
+    return {"bound": "mfma", "kernel": f"{name}, [{T} x {N}] x [{N} x {M}]", "achieved": flops / t / 1e12,
+            "peak": MFMA_F16_PEAK / 1e12, "unit": "TFLOP/s", "frac": flops / t / MFMA_F16_PEAK, "traffic": None,
+            "flops_per_launch": flops, "ms_per_launch": t * 1e3}
 
 
 def main():
@@ -235,6 +284,7 @@ def main():
         "prefill": {"tokens": args.prefill, "tok_s": args.prefill / t_prefill, "ms": 1e3 * t_prefill,
                     "flops": prefill_flops, "TFLOPs": prefill_flops / t_prefill / 1e12,
                     "frac_of_mfma_peak": prefill_flops / t_prefill / MFMA_F16_PEAK},
+        "prefill_roofline": gemm_roofline(min(chunk, args.prefill), C, F, u8),
     }
     if not args.no_cpu and version != 7:
         res["cpu_baseline"] = cpu_baseline(args.shape)
