@@ -2,7 +2,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--shape v4-7b] [--no-cpu]
 
-Workload (BASELINE.json configs[2]): random-init 32-layer / n_embd 4096 / ffn 16384 / vocab
+Workload (the headline configuration): random-init 32-layer / n_embd 4096 / ffn 16384 / vocab
 50277 model, prefill of 1024 uniform-random tokens in one call, then greedy decode.  A "step"
 is one decoded token (one pass of forward([token], state)); W untimed steps, then exactly K
 timed steps with the next token taken on the device (argmax) so the loop has no host
