@@ -35,8 +35,15 @@ How each function is pinned (what a wrong sign / index / dropped term would trip
                        rounding points, tests/golden/e2e_v7_*.npz); the two restatements
                        of the recurrence against each other, against a scalar loop and
                        against the closed form of the a = 0 special case.
-The fp16 rounding points of the reference's 'cuda fp16i8' path cannot be run
-anywhere in this build (needs nvcc + an NVIDIA GPU): for that emulation mode the
-placement of the roundings follows the reference text and is otherwise
-"parity unpinned"; its arithmetic is the same code the goldens pin in fp32.
+Where the half-precision path rounds is pinned by the reference itself: its pure-torch
+functions run on the CPU under 'cpu fp16' (tests/golden/e2e_*_cpu_fp16.npz, RWKV-4 to 6 and
+RWKV-7, incl. 8-layer models where the rescale acts); the oracle's 'cpu fp16' mode restates
+that run and its 'cuda fp16' emulation stays within one half-precision ulp of it.  What
+cannot be executed anywhere in this build (it needs nvcc and an NVIDIA GPU) and is therefore
+restated from the reference text only -- "parity unpinned" -- is the arithmetic specific to
+the reference's native CUDA library: the fp32 evaluation order inside kernel_mm_seq_fp16i8 /
+kernel_mm_one_fp16i8 with their fp16 outputs (cuda/operators.cu:116-246, model.py:63-86) and
+gemm_fp16_cublas writing fp32 without an intermediate fp16 rounding
+(cuda/gemm_fp16_cublas.cpp:31-33); the values they compute are pinned in fp32 by the
+'cpu fp32i8' goldens.
 """

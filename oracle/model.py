@@ -11,6 +11,11 @@ single-segment ones:
                               RESCALE_LAYER = 0 (model.py:634).  'cpu fp32i8' is the CPU
                               baseline path: every matmul dequantises the whole matrix
                               per call (model.py:91-97).
+  'cpu fp16'                  the reference's pure-torch functions on half tensors (what it runs
+                              with RWKV_CUDA_ON=0): the same rounding points as 'cuda fp16' except
+                              that a float product is rounded to fp16 before any widening
+                              (model.py:163); RESCALE_LAYER = 6.  Exists so that the reference
+                              itself, run on the CPU, pins where the fp16 path rounds.
   'cuda fp16', 'cuda fp16i8'  emulation of the GPU path: fp16 activations, fp32 WKV, fp32
                               accumulation in every contraction, roundings where the
                               reference's CUDA path rounds, RESCALE_LAYER = 6.
@@ -181,7 +186,9 @@ class OracleRWKV:
         return m
 
     def _mm(self, a, name, output_dtype=None):
-        return ops.matmul(a, self.mat(name), self.atype, output_dtype, cache=self.cache)
+        # on 'cpu' the reference has no native GEMM: a float product is rounded to the activation dtype first
+        return ops.matmul(a, self.mat(name), self.atype, output_dtype, cache=self.cache,
+                          via_atype=self.device == 'cpu')
 
     # ------------------------------------------------------------------ state
     def init_state(self):

@@ -85,19 +85,21 @@ class Mat:
         return d
 
 
-def matmul(a, m, atype, output_dtype=None, cache=False):
+def matmul(a, m, atype, output_dtype=None, cache=False, via_atype=False):
     """The reference's ``matmul`` (model.py:127-140).
 
     uint8 weights: contraction with fp32 accumulation, result rounded to the activation
     dtype (fp16 on the GPU path: model.py:86, operators.cu:138), then cast to
     ``output_dtype`` (model.py:138).
     float weights: fp32 accumulation, result written directly in ``output_dtype``
-    (model.py:150-161, gemm_fp16_cublas.cpp:31-33; on CPU ``(a @ b).to(output_dtype)``).
+    (model.py:150-161, gemm_fp16_cublas.cpp:31-33).  ``via_atype``: the plain-torch form
+    ``(a @ b).to(output_dtype)`` (model.py:163, 167) that runs without the native library, whose
+    product is first rounded to the activation dtype.
     """
     if output_dtype is None:
         output_dtype = atype
     acc = a.astype(f32) @ m.dense_f32(cache)
-    if m.quantized:
+    if m.quantized or via_atype:
         return acc.astype(atype).astype(output_dtype)
     return acc.astype(output_dtype)
 

@@ -14,6 +14,10 @@ RWKV_CUDA_ON=0 (no native build), feeds it synthetic checkpoints from
   e2e_<ver>_<strategy>.npz  logits (full_output over a 9-token prompt, then chunked calls
                             and one-token calls) and the final state, tiny models of
                             RWKV-4 / 5.0 / 5.1 / 5.2 / 6.0 under 'cpu fp32i8' and 'cpu fp32'
+  e2e_<ver>_cpu_fp16.npz    the same runs under 'cpu fp16' (the reference's pure-torch functions on half
+                            tensors, RESCALE_LAYER = 6): pins where the fp16 path rounds; and
+  e2e_<ver>_l8_cpu_fp16.npz 8-layer RWKV-4 / RWKV-6 models (n_embd 64) under 'cpu fp16', deep enough for
+                            the rescale (x / 2 after layer 6, matrices of layers >= 6 halved) to act
   planner.json              the per-slot plan the reference prints for a list of strategy strings
   e2e_v4_169m_cpu_fp32i8.npz  the 169M-shape model: 128-token prefill + 32 greedy steps;
                             argmax per position, 256 fixed logits per position, state sums
@@ -91,17 +95,41 @@ def quant_cuda_convert(tmp):
 
 
 def _state_np(state):
-    return {f"state_{i}": s.detach().cpu().contiguous().numpy() for i, s in enumerate(state)}
+    return {f"state_{i}": s.detach().float().cpu().contiguous().numpy() for i, s in enumerate(state)}
 
 
-def e2e_tiny(tmp):
+def e2e_deep_fp16(tmp):
+    RWKV = _ref()
+    for ver, tag in ((4, "v4"), (6, "v6_0")):
+        ck = synth.make_checkpoint(version=ver, seed=300 + int(ver * 10), **TINY8)
+        p = os.path.join(tmp, f"deep_{tag}.pth")
+        _save_ckpt(ck, p)
+        toks = synth.random_tokens(9, TINY8["vocab"], seed=PROMPT_SEED)
+        m = RWKV(p, "cpu fp16", verbose=False)
+        assert m.RESCALE_LAYER == 6
+        full, st_full = m.forward(toks, None, full_output=True)
+        outs, st = [], None
+        for a, b in ((0, 2), (2, 3), (3, 7), (7, 8), (8, 9)):
+            o, st = m.forward(toks[a:b], st)
+            outs.append(o.detach().float().cpu().numpy())
+        d = {"tokens": np.array(toks), "full_logits": full.detach().float().cpu().numpy(), "chunk_logits": np.stack(outs)}
+        d.update({"full_" + k: v for k, v in _state_np(st_full).items()})
+        d.update({"chunk_" + k: v for k, v in _state_np(st).items()})
+        name = f"e2e_{tag}_l8_cpu_fp16.npz"
+        np.savez_compressed(os.path.join(HERE, name), **d)
+        print("wrote", name)
+
+
+def e2e_tiny(tmp, which_strats=None):
     RWKV = _ref()
     for ver, tag in ((4, "v4"), (5, "v5_0"), (5.1, "v5_1"), (5.2, "v5_2"), (6, "v6_0")):
         ck = synth.make_checkpoint(version=ver, seed=200 + int(ver * 10), **TINY)
         p = os.path.join(tmp, f"tiny_{tag}.pth")
         _save_ckpt(ck, p)
         toks = synth.random_tokens(9, TINY["vocab"], seed=PROMPT_SEED)
-        for strat in ("cpu fp32i8", "cpu fp32"):
+        for strat in ("cpu fp32i8", "cpu fp32", "cpu fp16"):
+            if which_strats and strat not in which_strats:
+                continue
             m = RWKV(p, strat, verbose=False)
             full, st_full = m.forward(toks, None, full_output=True)
             # chunked: [0:2] seq, [2:3] one, [3:7] seq, [7:8] one, [8:9] one
@@ -109,8 +137,8 @@ def e2e_tiny(tmp):
             st = None
             for a, b in ((0, 2), (2, 3), (3, 7), (7, 8), (8, 9)):
                 o, st = m.forward(toks[a:b], st)
-                outs.append(o.detach().cpu().numpy())
-            d = {"tokens": np.array(toks), "full_logits": full.detach().cpu().numpy(),
+                outs.append(o.detach().float().cpu().numpy())
+            d = {"tokens": np.array(toks), "full_logits": full.detach().float().cpu().numpy(),
                  "chunk_logits": np.stack(outs)}
             d.update({"full_" + k: v for k, v in _state_np(st_full).items()})
             d.update({"chunk_" + k: v for k, v in _state_np(st).items()})
@@ -193,9 +221,13 @@ def planner(tmp):
 if __name__ == "__main__":
     torch.manual_seed(0)
     with tempfile.TemporaryDirectory() as tmp:
-        which = sys.argv[1:] or ["quant_cpu", "quant_cuda", "tiny", "169m", "planner"]
+        which = sys.argv[1:] or ["quant_cpu", "quant_cuda", "tiny", "fp16", "169m", "planner"]
         if "planner" in which:
             planner(tmp)
+        if "fp16" in which and "tiny" not in which:
+            e2e_tiny(tmp, which_strats=("cpu fp16",))   # only the half-precision files
+        if "fp16" in which:
+            e2e_deep_fp16(tmp)
         if "quant_cpu" in which:
             quant_cpu(tmp)
         if "quant_cuda" in which:

@@ -309,3 +309,47 @@ def test_v56_long_prompt(ver, tag, strat):
     oout, ost = o.forward(toks[70:], ost)
     d = float(np.abs(_np(out) - oout).max())
     assert d <= LOGIT_TOL, d
+
+
+@pytest.mark.parametrize("ver,tag", [(4, "v4"), (5, "v5_0"), (5.1, "v5_1"), (5.2, "v5_2"), (6, "v6_0")])
+def test_fp16_strategy_against_reference_half_run(ver, tag):
+    """'cuda fp16' on the GPU against the logits and states the reference itself produced under 'cpu fp16'
+    (its pure-torch functions on half tensors; tests/golden/make_goldens.py): full_output over the prompt,
+    then the chunked sequence / one-token calls."""
+    ref = dict(np.load(os.path.join(G, f"e2e_{tag}_cpu_fp16.npz")))
+    ck = synth.make_checkpoint(version=ver, seed=200 + int(ver * 10), **TINY)
+    m = _rwkv()(ck, "cuda fp16", verbose=False)
+    toks = [int(t) for t in ref["tokens"]]
+    full, st_full = m.forward(toks, None, full_output=True)
+    d = float(np.abs(_np(full) - ref["full_logits"]).max())
+    assert d <= LOGIT_TOL, d
+    assert _argmax_agree(_np(full), ref["full_logits"], d)
+    st, outs = None, []
+    for a, b in ((0, 2), (2, 3), (3, 7), (7, 8), (8, 9)):
+        out, st = m.forward(toks[a:b], st)
+        outs.append(_np(out))
+    assert np.abs(np.stack(outs) - ref["chunk_logits"]).max() <= LOGIT_TOL
+    for prefix, state in (("full_", st_full), ("chunk_", st)):
+        for i, s in enumerate(state):
+            r = ref[f"{prefix}state_{i}"]
+            assert tuple(s.shape) == r.shape, (prefix, i)
+            big = max(float(np.abs(r).max()), 1.0)
+            assert np.abs(_np(s) - r).max() <= 1e-2 * big, (prefix, i)
+
+
+@pytest.mark.parametrize("ver,tag", [(4, "v4"), (6, "v6_0")])
+def test_fp16_rescale_against_reference_half_run(ver, tag):
+    """Eight layers, so the rescale (x / 2 after layer 6, halved matrices from layer 6 on) acts."""
+    from tests.golden.make_goldens import TINY8
+    ref = dict(np.load(os.path.join(G, f"e2e_{tag}_l8_cpu_fp16.npz")))
+    ck = synth.make_checkpoint(version=ver, seed=300 + int(ver * 10), **TINY8)
+    m = _rwkv()(ck, "cuda fp16", verbose=False)
+    assert m.RESCALE_LAYER == 6
+    toks = [int(t) for t in ref["tokens"]]
+    full, _ = m.forward(toks, None, full_output=True)
+    assert np.abs(_np(full) - ref["full_logits"]).max() <= LOGIT_TOL
+    st, outs = None, []
+    for a, b in ((0, 2), (2, 3), (3, 7), (7, 8), (8, 9)):
+        out, st = m.forward(toks[a:b], st)
+        outs.append(_np(out))
+    assert np.abs(np.stack(outs) - ref["chunk_logits"]).max() <= LOGIT_TOL

@@ -92,3 +92,55 @@ def test_forward_matches_reference_cpu(ver, tag, strat):
             r = ref[f"{prefix}state_{i}"]
             assert s.shape == r.shape and s.dtype == r.dtype, (prefix, i)
             np.testing.assert_allclose(s, r, rtol=2e-4, atol=2e-5, err_msg=f"{prefix}{i}")
+
+
+def _check_fp16(o, ref, vocab):
+    """Within a few half-precision roundings of the reference's own half-precision run (the CPU half
+    kernels and numpy round the same operations but sum in different orders)."""
+    toks = [int(t) for t in ref["tokens"]]
+    scale = float(np.abs(ref["full_logits"]).max())
+    tol = 1.5e-3 * max(scale, 1.0)                  # three half-precision ulps of a logit near 1 (observed: one)
+    full, st_full = o.forward(toks, None, full_output=True)
+    assert np.abs(full - ref["full_logits"]).max() <= tol
+    st, outs = None, []
+    for a, b in ((0, 2), (2, 3), (3, 7), (7, 8), (8, 9)):
+        out, st = o.forward(toks[a:b], st)
+        assert out.shape == (vocab,)
+        outs.append(out)
+    assert np.abs(np.stack(outs) - ref["chunk_logits"]).max() <= tol
+    for prefix, state in (("full_", st_full), ("chunk_", st)):
+        for i, s in enumerate(state):
+            r = ref[f"{prefix}state_{i}"]
+            assert s.shape == r.shape, (prefix, i)
+            big = max(float(np.abs(r).max()), 1.0)
+            assert np.abs(s.astype(np.float32) - r).max() <= 4e-3 * big, (prefix, i)
+    return float(np.abs(full - ref["full_logits"]).max())
+
+
+@pytest.mark.parametrize("ver,tag", VERS)
+def test_fp16_rounding_points_match_reference(ver, tag):
+    """The reference run under 'cpu fp16' (its pure-torch functions on half tensors) pins where the
+    half-precision path rounds: the oracle's 'cpu fp16' mode restates exactly that path, and its 'cuda
+    fp16' emulation (which differs only in not rounding a float product before widening it) stays as
+    close."""
+    ref = _load(f"e2e_{tag}_cpu_fp16.npz")
+    ck = synth.make_checkpoint(version=ver, seed=200 + int(ver * 10), **TINY)
+    for strat in ("cpu fp16", "cuda fp16"):
+        o = OracleRWKV(ck, strat)
+        assert o.rescale_layer == 6
+        _check_fp16(o, ref, TINY["vocab"])
+
+
+@pytest.mark.parametrize("ver,tag", [(4, "v4"), (6, "v6_0")])
+def test_fp16_rescale_matches_reference(ver, tag):
+    """Eight layers: the halving of x after layer 6 and of the output / value matrices of layers >= 6
+    (model.py:785-789, 1660-1662) acts; without it the logits would differ by a factor of two."""
+    ref = _load(f"e2e_{tag}_l8_cpu_fp16.npz")
+    ck = synth.make_checkpoint(version=ver, seed=300 + int(ver * 10), **TINY8)
+    for strat in ("cpu fp16", "cuda fp16"):
+        _check_fp16(OracleRWKV(ck, strat), ref, TINY8["vocab"])
+    wrong = OracleRWKV(ck, "cuda fp16", rescale_layer=0)
+    toks = [int(t) for t in ref["tokens"]]
+    full, _ = wrong.forward(toks, None, full_output=True)
+    # mathematically invisible (LayerNorm follows), so still close: the check above is what pins the placement
+    assert np.abs(full - ref["full_logits"]).max() < 0.05
