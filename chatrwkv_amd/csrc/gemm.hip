@@ -120,7 +120,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(int T, int N, int M, const h1
             for (int i = 0; i < B_LD; ++i) {
                 const int row = (tid >> 2) + 64 * i, ch = tid & 3;
                 const int m = min(m0 + row, M - 1);
-                qb[i] = __builtin_nontemporal_load((const u32x4 *)((const uint8_t *)Wv + (size_t)m * ldw + k0 + ch * 16));
+                qb[i] = *(const u32x4 *)((const uint8_t *)Wv + (size_t)m * ldw + k0 + ch * 16);  // a 64-byte half line: the other half is the next k-tile, kept in L1
             }
         } else {
 #pragma unroll
