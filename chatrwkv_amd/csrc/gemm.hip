@@ -8,7 +8,7 @@
 // rank-1 corrections enter in the epilogue:
 //     y[t, m] = rx[m] * acc[t, m] + mx[m] * S0[t] + S2[t],   S0 = sum_j x[t, j],  S2 = sum_j x[t, j] my[j].
 //
-// Tiling: BT x BM outputs per workgroup of 256 threads (WT x WM waves, each owning a
+// Tiling: BT x BM outputs per workgroup of 64 WT WM threads (WT x WM waves, each owning a
 // (BT/WT) x (BM/WM) block built from 32x32 MFMA tiles), K step 64, LDS double buffered; both LDS
 // tiles are [row][64 halves] with the eight 16-byte chunks of a row XOR-swizzled by (row & 7) so
 // that the ds_read_b128 of 32 consecutive rows spreads over all banks.  A wave block of
@@ -78,10 +78,12 @@ __global__ __launch_bounds__(256) void splitk_epilogue_kernel(int T, int M, int 
 }
 
 template <bool W_U8, int BT, int BM, int WT, int WM, int PF, bool SPLIT>
-__global__ __launch_bounds__(256) void gemm_kernel(int T, int N, int M, const h16 *__restrict__ A, int64_t lda,
+__global__ __launch_bounds__(64 * WT * WM) void gemm_kernel(int T, int N, int M, const h16 *__restrict__ A, int64_t lda,
                                                    const void *__restrict__ Wv, int64_t ldw, void *__restrict__ Y,
                                                    int64_t ldy, GemmEpi ep, int nk_split, float *__restrict__ part) {
-    static_assert(WT * WM == 4 && BT % (32 * WT) == 0 && BM % (32 * WM) == 0 && BM % 64 == 0, "tile");
+    constexpr int NT = 64 * WT * WM;                 // threads per workgroup
+    constexpr int RA = NT / 8, RB8 = NT / 4;         // tile rows one pass of 16-byte loads covers (fp16 / uint8 rows)
+    static_assert(BT % (32 * WT) == 0 && BM % (32 * WM) == 0 && BT % RA == 0 && BM % RB8 == 0, "tile");
     constexpr int MI = BT / (32 * WT), NI = BM / (32 * WM);  // 32x32 blocks per wave in each direction
     extern __shared__ __align__(16) unsigned char smem[];
     h16 *lA[2], *lB[2];
@@ -99,8 +101,8 @@ __global__ __launch_bounds__(256) void gemm_kernel(int T, int N, int M, const h1
     if ((gridDim.x & 7) == 0) bid = (bid & 7) * (gridDim.x >> 3) + (bid >> 3);
     const int t0 = (bid % tiles_t) * BT, m0 = (bid / tiles_t) * BM;
 
-    constexpr int A_LD = BT / 32;                    // 16-byte loads per thread for the A tile
-    constexpr int B_LD = W_U8 ? BM / 64 : BM / 32;   // 16-byte loads per thread for the W tile
+    constexpr int A_LD = BT / RA;                    // 16-byte loads per thread for the A tile
+    constexpr int B_LD = W_U8 ? BM / RB8 : BM / RA;  // 16-byte loads per thread for the W tile
     // PF k-tiles are in flight in registers (global latency under load is several k-tile times);
     // the LDS holds the tile being multiplied and the next one.
     u32x4 ra[PF][A_LD], rb[PF][B_LD];
@@ -111,21 +113,21 @@ __global__ __launch_bounds__(256) void gemm_kernel(int T, int N, int M, const h1
         const int k0 = (kbase + kt) * BK;
 #pragma unroll
         for (int i = 0; i < A_LD; ++i) {
-            const int row = (tid >> 3) + 32 * i, ch = tid & 7;
+            const int row = (tid >> 3) + RA * i, ch = tid & 7;
             const int t = min(t0 + row, T - 1);
             qa[i] = *(const u32x4 *)(A + (size_t)t * lda + k0 + ch * 8);
         }
         if (W_U8) {
 #pragma unroll
             for (int i = 0; i < B_LD; ++i) {
-                const int row = (tid >> 2) + 64 * i, ch = tid & 3;
+                const int row = (tid >> 2) + RB8 * i, ch = tid & 3;
                 const int m = min(m0 + row, M - 1);
                 qb[i] = *(const u32x4 *)((const uint8_t *)Wv + (size_t)m * ldw + k0 + ch * 16);  // a 64-byte half line: the other half is the next k-tile, kept in L1
             }
         } else {
 #pragma unroll
             for (int i = 0; i < B_LD; ++i) {
-                const int row = (tid >> 3) + 32 * i, ch = tid & 7;
+                const int row = (tid >> 3) + RA * i, ch = tid & 7;
                 const int m = min(m0 + row, M - 1);
                 qb[i] = *(const u32x4 *)((const h16 *)Wv + (size_t)m * ldw + k0 + ch * 8);
             }
@@ -134,14 +136,14 @@ __global__ __launch_bounds__(256) void gemm_kernel(int T, int N, int M, const h1
     auto store_tiles = [&](const u32x4 (&qa)[A_LD], const u32x4 (&qb)[B_LD], int buf) {
 #pragma unroll
         for (int i = 0; i < A_LD; ++i) {
-            const int row = (tid >> 3) + 32 * i, ch = tid & 7;
+            const int row = (tid >> 3) + RA * i, ch = tid & 7;
             *(u32x4 *)(lA[buf] + swz(row, ch)) = qa[i];
         }
         if (W_U8) {
             const h16x2 off = {(h16)1023.5f, (h16)1023.5f};
 #pragma unroll
             for (int i = 0; i < B_LD; ++i) {
-                const int row = (tid >> 2) + 64 * i, ch = tid & 3;
+                const int row = (tid >> 2) + RB8 * i, ch = tid & 3;
                 u32x4 lo, hi;
                 const uint32_t d[4] = {qb[i].x, qb[i].y, qb[i].z, qb[i].w};
                 uint32_t o[8];
@@ -161,7 +163,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(int T, int N, int M, const h1
         } else {
 #pragma unroll
             for (int i = 0; i < B_LD; ++i) {
-                const int row = (tid >> 3) + 32 * i, ch = tid & 7;
+                const int row = (tid >> 3) + RA * i, ch = tid & 7;
                 *(u32x4 *)(lB[buf] + swz(row, ch)) = qb[i];
             }
         }
@@ -300,13 +302,13 @@ int launch_cfg(int64_t T, int64_t N, int64_t M, const rwkv_half *A, int64_t lda,
         }
     }
     if (ks > 1) {
-        hipLaunchKernelGGL((gemm_kernel<W_U8, BT, BM, WT, WM, PF, true>), dim3((unsigned)tiles, (unsigned)ks), dim3(256), lds, st,
+        hipLaunchKernelGGL((gemm_kernel<W_U8, BT, BM, WT, WM, PF, true>), dim3((unsigned)tiles, (unsigned)ks), dim3(64 * WT * WM), lds, st,
                            (int)T, (int)N, (int)M, (const h16 *)A, lda, W, ldw, Y, ldy, ep, nk / ks, ep.splitk_ws);
         const int64_t n = T * M;
         const unsigned blocks = (unsigned)((n + 1023) / 1024 < 2048 ? (n + 1023) / 1024 : 2048);
         hipLaunchKernelGGL(splitk_epilogue_kernel, dim3(blocks), dim3(256), 0, st, (int)T, (int)M, ks, ep.splitk_ws, Y, ldy, ep);
     } else {
-        hipLaunchKernelGGL((gemm_kernel<W_U8, BT, BM, WT, WM, PF, false>), dim3((unsigned)tiles), dim3(256), lds, st, (int)T,
+        hipLaunchKernelGGL((gemm_kernel<W_U8, BT, BM, WT, WM, PF, false>), dim3((unsigned)tiles), dim3(64 * WT * WM), lds, st, (int)T,
                            (int)N, (int)M, (const h16 *)A, lda, W, ldw, Y, ldy, ep, nk, (float *)nullptr);
     }
     RWKV_LAUNCH_CHECK();
@@ -317,13 +319,10 @@ template <bool W_U8>
 int launch_pick(int cfg, int64_t T, int64_t N, int64_t M, const rwkv_half *A, int64_t lda, const void *W, int64_t ldw,
                 void *Y, int64_t ldy, const GemmEpi &ep, hipStream_t st) {
     switch (cfg) {
-        case 0: return launch_cfg<W_U8, 128, 128, 2, 2, 1>(T, N, M, A, lda, W, ldw, Y, ldy, ep, st);
-        case 1: return launch_cfg<W_U8, 128, 128, 2, 2, 2>(T, N, M, A, lda, W, ldw, Y, ldy, ep, st);
-        case 2: return launch_cfg<W_U8, 128, 128, 2, 2, 3>(T, N, M, A, lda, W, ldw, Y, ldy, ep, st);
         case 3: return launch_cfg<W_U8, 128, 128, 2, 2, 4>(T, N, M, A, lda, W, ldw, Y, ldy, ep, st);
-        case 4: return launch_cfg<W_U8, 256, 128, 2, 2, 2>(T, N, M, A, lda, W, ldw, Y, ldy, ep, st);
-        case 5: return launch_cfg<W_U8, 128, 256, 2, 2, 2>(T, N, M, A, lda, W, ldw, Y, ldy, ep, st);
-        case 6: return launch_cfg<W_U8, 256, 256, 2, 2, 2>(T, N, M, A, lda, W, ldw, Y, ldy, ep, st);
+        case 9:
+            if constexpr (W_U8) return launch_cfg<true, 256, 256, 4, 4, 2>(T, N, M, A, lda, W, ldw, Y, ldy, ep, st);
+            return RWKV_E_DTYPE;
         default: return RWKV_E_DTYPE;
     }
 }
@@ -332,15 +331,21 @@ int launch_pick(int cfg, int64_t T, int64_t N, int64_t M, const rwkv_half *A, in
 int pick_cfg(int64_t T, int64_t M) {
     const char *e = getenv("RWKV_GEMM_CFG");  // tuning override
     if (e && *e) return atoi(e);
-    (void)T; (void)M;
-    return 3;  // 128 x 128 tile, 4 k-tiles of prefetch: the best of the sweep for every shape measured
+    // The kernel is bound by how fast a CU's L1 can be filled, and a 256 x 256 tile (16 waves) fetches half the
+    // operand bytes per flop of a 128 x 128 one: +30 % on [1024 x 4096] x [4096 x 16384].  Only where such tiles
+    // fill the chip: one per CU and round, the last round at least 70 % full.
+    const int64_t big = ((T + 255) / 256) * ((M + 255) / 256), rounds = (big + 255) / 256;
+    if (big * 10 >= rounds * 256 * 7) return 9;
+    return 3;  // 128 x 128 tile, 4 k-tiles of prefetch
 }
 
 }  // namespace
 
 int gemm_launch(bool w_u8, int64_t T, int64_t N, int64_t M, const rwkv_half *A, int64_t lda, const void *W,
                 int64_t ldw, void *Y, int64_t ldy, const GemmEpi &ep, hipStream_t st) {
-    const int cfg = pick_cfg(T, M);
+    int cfg = pick_cfg(T, M);
+    // the large tile pays with uint8 weights only: fp16 weight tiles are twice the bytes and its registers spill
+    if ((ep.small_tiles || !w_u8) && cfg == 9) cfg = 3;
     return w_u8 ? launch_pick<true>(cfg, T, N, M, A, lda, W, ldw, Y, ldy, ep, st)
                 : launch_pick<false>(cfg, T, N, M, A, lda, W, ldw, Y, ldy, ep, st);
 }

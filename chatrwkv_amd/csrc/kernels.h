@@ -16,6 +16,8 @@ struct GemmEpi {
     int raw_f32;                   // 1: store the fp32 accumulator unrounded (out_dtype must be F32)
     float *splitk_ws;              // scratch for split-K partial sums (NULL: never split)
     size_t splitk_bytes;
+    int small_tiles;               // 1: keep the 128 x 128 tile (the caller runs another contraction beside this one, and a
+                                   // 256 x 256 tile's 128 KB of LDS would leave no room for it on the CU)
 };
 
 // Size of the split-K scratch the model-level entry points reserve in their workspaces.

@@ -346,7 +346,9 @@ extern "C" int rwkv_v4_forward_seq(const rwkv_v4_model *m, const rwkv_v4_layer_s
         const bool par2 = ss && (T / 128) * (C / 128) > 128 && fork_streams(ss, st, 1);
         if ((rc = run_gemm(l.ffn_receptance, u8, T, ws.xs[0], s0[0], s2[0], ws.r, C, e, par2 ? ss->s[0] : st, ws.splitk))) return rc;
         e.act = ACT_RELU_SQ;
+        e.small_tiles = par2 ? 1 : 0;   // the receptance product runs beside this one
         if ((rc = run_gemm(l.ffn_key, u8, T, ws.xs[1], s0[1], s2[1], ws.vx, F, e, st, ws.splitk))) return rc;
+        e.small_tiles = 0;
         if (par2 && !join_streams(ss, st, 1)) return (int)hipErrorUnknown;
         const rwkv_half *a_v = ws.vx;
         if (u8) {
