@@ -59,3 +59,14 @@ int copy_h16_launch(int n, const rwkv_half *src, rwkv_half *dst, hipStream_t st)
 int v4_model_check(const rwkv_v4_model *m);
 int v4_head_launch(const rwkv_v4_model *m, const rwkv_half *x, float *logits, hipStream_t st);
 int num_cu();
+
+// Two extra streams (default priority, created once per process) for contractions that are independent and each
+// too small to fill the chip; fork / join by events around them (seq_v4.hip).
+struct SideStreams {
+    hipStream_t s[2];
+    hipEvent_t fork, join[2];
+    bool ok;
+};
+SideStreams *side_streams();                                   // NULL when the streams could not be created
+bool fork_streams(SideStreams *ss, hipStream_t st, int n);     // side stream j < n then sees everything queued on st so far
+bool join_streams(SideStreams *ss, hipStream_t st, int n);     // st then sees everything queued on the side streams

@@ -204,11 +204,7 @@ int run_gemm(const rwkv_mat &m, bool u8, int64_t T, const rwkv_half *A, const fl
 
 // Two side streams (default priority) for contractions that are independent of each other and too small
 // to fill the chip alone: k / v / r of the time mix and r / k of the channel mix run side by side.
-struct SideStreams {
-    hipStream_t s[2];
-    hipEvent_t fork, join[2];
-    bool ok;
-};
+}  // namespace
 
 SideStreams *side_streams() {
     static SideStreams ss{};
@@ -240,8 +236,6 @@ bool join_streams(SideStreams *ss, hipStream_t st, int n) {
     }
     return true;
 }
-
-}  // namespace
 
 extern "C" int rwkv_layernorm_f32_f16(int64_t T, int64_t C, const float *x, const float *w, const float *b,
                                       rwkv_half *y, void *stream) {

@@ -529,6 +529,8 @@ extern "C" int rwkv_v7_forward(const rwkv_v7_model *m, const rwkv_v56_layer_stat
         return q;
     };
 
+    SideStreams *ss = T >= 256 ? side_streams() : nullptr;
+
     if ((rc = gather_emb_launch(T, C, tokens, m->emb, ws.x, st))) return rc;
     for (int i = 0; i < m->n_layer; ++i) {
         const rwkv_v7_layer &l = m->layers[i];
@@ -578,20 +580,27 @@ extern "C" int rwkv_v7_forward(const rwkv_v7_model *m, const rwkv_v56_layer_stat
         const rwkv_half *xr = ws.mix[0], *xw = ws.mix[1], *xk = ws.mix[2], *xv = ws.mix[3], *xa = ws.mix[4],
                         *xg = ws.mix[5];
         rwkv_half *v = i == 0 ? ws.v_first : ws.v;
+        // The three C x C products and the LoRA chain are independent of each other.  Long calls run them on three
+        // streams: receptance and key on the caller's, value on the first side stream, the eight small LoRA
+        // products (the only ones that split K: they share the split-K scratch) on the second.
+        const bool par = ss && fork_streams(ss, st, 2);
+        Ctx cm = c, cv = c, cl = c;
+        if (par) { cm.splitk = nullptr; cv.splitk = nullptr; cv.st = ss->s[0]; cl.st = ss->s[1]; }
         // the first matrix call also commits the new token-shift state (all readers of the old one are done)
-        if ((rc = mm(c, l.att_receptance, false, xr, ACT_NONE, nullptr, nullptr, 1.f, ws.r, ws.xx_att, s.att_xx, C))) return rc;
-        if ((rc = mm(c, l.att_key, false, xk, ACT_NONE, nullptr, nullptr, 1.f, ws.k))) return rc;
-        if ((rc = mm(c, l.att_value, false, xv, ACT_NONE, nullptr, nullptr, 1.f, v))) return rc;
-        if ((rc = mm(c, lora_first(l, 0, m->lora_w), false, xw, ACT_TANH, nullptr, nullptr, 1.f, ws.lw))) return rc;
-        if ((rc = mm(c, lora_second(l, 0, m->lora_w), false, ws.lw, ACT_NONE, nullptr, nullptr, 1.f, ws.w_raw))) return rc;
-        if ((rc = mm(c, lora_first(l, o_a, m->lora_a), false, xa, ACT_NONE, nullptr, nullptr, 1.f, ws.la))) return rc;
-        if ((rc = mm(c, lora_second(l, o_a, m->lora_a), false, ws.la, ACT_NONE, nullptr, nullptr, 1.f, ws.a_raw))) return rc;
+        if ((rc = mm(cm, l.att_receptance, false, xr, ACT_NONE, nullptr, nullptr, 1.f, ws.r, ws.xx_att, s.att_xx, C))) return rc;
+        if ((rc = mm(cm, l.att_key, false, xk, ACT_NONE, nullptr, nullptr, 1.f, ws.k))) return rc;
+        if ((rc = mm(cv, l.att_value, false, xv, ACT_NONE, nullptr, nullptr, 1.f, v))) return rc;
+        if ((rc = mm(cl, lora_first(l, 0, m->lora_w), false, xw, ACT_TANH, nullptr, nullptr, 1.f, ws.lw))) return rc;
+        if ((rc = mm(cl, lora_second(l, 0, m->lora_w), false, ws.lw, ACT_NONE, nullptr, nullptr, 1.f, ws.w_raw))) return rc;
+        if ((rc = mm(cl, lora_first(l, o_a, m->lora_a), false, xa, ACT_NONE, nullptr, nullptr, 1.f, ws.la))) return rc;
+        if ((rc = mm(cl, lora_second(l, o_a, m->lora_a), false, ws.la, ACT_NONE, nullptr, nullptr, 1.f, ws.a_raw))) return rc;
         if (i > 0) {
-            if ((rc = mm(c, lora_first(l, o_v, m->lora_v), false, xv, ACT_NONE, nullptr, nullptr, 1.f, ws.lv))) return rc;
-            if ((rc = mm(c, lora_second(l, o_v, m->lora_v), false, ws.lv, ACT_NONE, nullptr, nullptr, 1.f, ws.vg_raw))) return rc;
+            if ((rc = mm(cl, lora_first(l, o_v, m->lora_v), false, xv, ACT_NONE, nullptr, nullptr, 1.f, ws.lv))) return rc;
+            if ((rc = mm(cl, lora_second(l, o_v, m->lora_v), false, ws.lv, ACT_NONE, nullptr, nullptr, 1.f, ws.vg_raw))) return rc;
         }
-        if ((rc = mm(c, lora_first(l, o_g, m->lora_g), false, xg, ACT_SIGMOID, nullptr, nullptr, 1.f, ws.lg))) return rc;
-        if ((rc = mm(c, lora_second(l, o_g, m->lora_g), false, ws.lg, ACT_NONE, nullptr, nullptr, 1.f, ws.g))) return rc;
+        if ((rc = mm(cl, lora_first(l, o_g, m->lora_g), false, xg, ACT_SIGMOID, nullptr, nullptr, 1.f, ws.lg))) return rc;
+        if ((rc = mm(cl, lora_second(l, o_g, m->lora_g), false, ws.lg, ACT_NONE, nullptr, nullptr, 1.f, ws.g))) return rc;
+        if (par && !join_streams(ss, st, 2)) return (int)hipErrorUnknown;
         {
             Prep7Args a{};
             a.T = (int)T; a.C = C; a.H = H; a.r = ws.r; a.k = ws.k; a.v = v; a.w_raw = ws.w_raw; a.a_raw = ws.a_raw;

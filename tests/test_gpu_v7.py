@@ -187,6 +187,27 @@ def test_v7_long_prompt_and_odd_lora_ranks():
         assert np.abs(_np(s) - ref.astype(np.float32)).max() <= 1e-2 * scale, i
 
 
+def test_v7_side_stream_path(tiny7):
+    """A call of 256 tokens or more runs the independent products of a layer on three streams; its logits and
+    states must match the oracle and the same prompt fed in shorter calls (which stay on one stream)."""
+    m, o, _ = tiny7
+    toks = synth.random_tokens(300, TINY7["vocab"], seed=21)
+    out, st = m.forward(toks, None, full_output=True)
+    torch.cuda.synchronize()
+    oo, ost = o.forward(toks, None, full_output=True)
+    d = float(np.abs(_np(out) - oo.astype(np.float32)).max())
+    assert d <= LOGIT_TOL, d
+    assert _argmax_agree(_np(out), oo.astype(np.float32), d)
+    st2 = None
+    for a in range(0, 300, 100):
+        out2, st2 = m.forward(toks[a:a + 100], st2)
+    assert np.abs(_np(out2) - _np(out[-1])).max() <= LOGIT_TOL
+    for i, (s, s2, ref) in enumerate(zip(st, st2, ost)):
+        scale = max(float(np.abs(ref.astype(np.float32)).max()), 1.0)
+        assert np.abs(_np(s) - ref.astype(np.float32)).max() <= 1e-2 * scale, i
+        assert np.abs(_np(s) - _np(s2)).max() <= 1e-2 * scale, i
+
+
 def test_v7_api_errors(tiny7):
     m, _, ck = tiny7
     with pytest.raises(IndexError):
