@@ -13,7 +13,8 @@ struct Ctx {
     int grid;
     rwkv_half *xs;       // scaled-activation scratch [T, max(C, F)]
     float *s0, *s2;      // [T]
-    float *splitk;       // RWKV_SPLITK_WS_BYTES of split-K scratch
+    float *splitk;       // RWKV_SPLITK_WS_BYTES of split-K scratch (NULL: never split)
+    int small_tiles;     // 1: another contraction runs beside the ones launched through this context
 };
 
 // y = act(x @ W) for a model matrix (uint8 or fp16 per strategy) or an fp16 LoRA matrix.
@@ -49,6 +50,7 @@ inline int mm(const Ctx &c, const rwkv_mat &m, bool mat_u8, const rwkv_half *x, 
     GemmEpi e{};
     e.act = act; e.res = res; e.ldres = M; e.gate = gate; e.ldgate = M; e.out_scale = out_scale;
     e.out_dtype = RWKV_DT_F16; e.splitk_ws = c.splitk; e.splitk_bytes = RWKV_SPLITK_WS_BYTES;
+    e.small_tiles = c.small_tiles;
     if (mat_u8) {
         int rc = mm8_prepare_launch(c.T, N, x, N, m.ry, m.my, c.xs, c.s0, c.s2, c.st);
         if (rc) return rc;

@@ -124,6 +124,8 @@ __global__ __launch_bounds__(256) void v6_mix2_kernel(Mix2Args a) {
 struct Ws56 {
     rwkv_half *x, *xx, *sxd, *xxx, *t1, *mix[5], *d1, *d2, *r, *k, *v, *g, *att, *vx, *xs, *xx_att, *xx_ffn;
     float *sums, *splitk, *y32;
+    rwkv_half *xs_side[2];   // scaled-activation scratch of the products that run on side streams [T, C]
+    float *sums_side[2];
     size_t total;
 };
 
@@ -140,6 +142,10 @@ Ws56 carve56(void *base, int64_t T, int64_t C, int64_t F, int64_t lm, int64_t ld
     w.vx = take(tf); w.xs = take(tf > tc ? tf : tc);
     w.xx_att = take((size_t)C * 2); w.xx_ffn = take((size_t)C * 2);
     w.sums = (float *)take((size_t)T * 2 * sizeof(float));
+    for (int j = 0; j < 2; ++j) {
+        w.xs_side[j] = take(T >= 256 ? tc : 256);
+        w.sums_side[j] = (float *)take((size_t)T * 2 * sizeof(float));
+    }
     w.splitk = (float *)take(RWKV_SPLITK_WS_BYTES);
     w.y32 = (float *)take(T >= 32 ? (size_t)T * C * 4 : 256);
     w.total = (size_t)(p - (unsigned char *)base);
@@ -209,7 +215,17 @@ extern "C" int rwkv_v56_forward(const rwkv_v56_model *m, const rwkv_v56_layer_st
     const bool u8 = m->weights_u8 != 0, v6 = ver == 60, gated = ver != 50;
     const int lm = m->lora_maa, ld = m->lora_decay;
     Ws56 ws = carve56(workspace, T, C, F, v6 ? lm : 32, v6 ? ld : 64);
-    Ctx c{st, u8, T, num_cu(), ws.xs, ws.sums, ws.sums + T, ws.splitk};
+    Ctx c{st, u8, T, num_cu(), ws.xs, ws.sums, ws.sums + T, ws.splitk, 0};
+    // Sequence calls whose square products have more than 128 output tiles (none of them would split K) run
+    // independent products side by side on two extra streams, each with its own activation scratch.  Shorter
+    // calls are faster one product after the other with split-K (measured at 256 tokens, n_embd 4096).
+    SideStreams *ss = (T / 128) * (C / 128) > 128 ? side_streams() : nullptr;
+    Ctx cs[2] = {c, c};
+    if (ss)
+        for (int j = 0; j < 2; ++j) {
+            cs[j].st = ss->s[j]; cs[j].xs = ws.xs_side[j]; cs[j].s0 = ws.sums_side[j]; cs[j].s2 = ws.sums_side[j] + T;
+            cs[j].splitk = nullptr;
+        }
 
     if ((rc = gather_emb_launch(T, C, tokens, m->emb, ws.x, st))) return rc;
     for (int i = 0; i < m->n_layer; ++i) {
@@ -264,10 +280,15 @@ extern "C" int rwkv_v56_forward(const rwkv_v56_model *m, const rwkv_v56_layer_st
             if (fuse_d1) { a.xin = wx; a.xmat = l.td_w1; a.xm = ld; a.xout = ws.d1; }
             multi_vec_launch(u8, a, c.grid, st);
         } else {
-            if ((rc = mm(c, l.att_receptance, u8, rx, ACT_NONE, nullptr, nullptr, 1.f, ws.r, ws.xx_att, s.att_xx, C))) return rc;
-            if ((rc = mm(c, l.att_key, u8, kx, ACT_NONE, nullptr, nullptr, 1.f, ws.k))) return rc;
-            if ((rc = mm(c, l.att_value, u8, vx, ACT_NONE, nullptr, nullptr, 1.f, ws.v))) return rc;
+            // receptance (then gate) on the caller's stream, key and value on the side streams
+            const bool par = ss && fork_streams(ss, st, 2);
+            Ctx cr = c;
+            if (par) cr.splitk = nullptr;
+            if ((rc = mm(cr, l.att_receptance, u8, rx, ACT_NONE, nullptr, nullptr, 1.f, ws.r, ws.xx_att, s.att_xx, C))) return rc;
+            if ((rc = mm(par ? cs[0] : c, l.att_key, u8, kx, ACT_NONE, nullptr, nullptr, 1.f, ws.k))) return rc;
+            if ((rc = mm(par ? cs[1] : c, l.att_value, u8, vx, ACT_NONE, nullptr, nullptr, 1.f, ws.v))) return rc;
             if (gated && (rc = mm(c, l.att_gate, u8, gx, ACT_SILU, nullptr, nullptr, 1.f, ws.g))) return rc;
+            if (par && !join_streams(ss, st, 2)) return (int)hipErrorUnknown;
         }
         // one token of v6: the second decay LoRA product is done inside the WKV kernel
         const bool d2_fused = v6 && T == 1;
@@ -299,8 +320,20 @@ extern "C" int rwkv_v56_forward(const rwkv_v56_model *m, const rwkv_v56_layer_st
             for (int j = 0; j < 2; ++j) { a.ry[j] = nullptr; a.my[j] = nullptr; a.xs[j] = ws.mix[j]; }
             if ((rc = lnmix_seq_launch(a, 2, st))) return rc;
         }
-        if ((rc = mm(c, l.ffn_receptance, u8, ws.mix[0], ACT_SIGMOID, nullptr, nullptr, 1.f, ws.r, ws.xx_ffn, s.ffn_xx, C))) return rc;
-        if ((rc = mm(c, l.ffn_key, u8, ws.mix[1], ACT_RELU_SQ, nullptr, nullptr, 1.f, ws.vx))) return rc;
+        {
+            // channel-mix receptance beside the key product
+            const bool par = ss && fork_streams(ss, st, 1);
+            if (par && (rc = copy_h16_launch(C, ws.xx_ffn, s.ffn_xx, st))) return rc;
+            if (par) {
+                if ((rc = mm(cs[0], l.ffn_receptance, u8, ws.mix[0], ACT_SIGMOID, nullptr, nullptr, 1.f, ws.r))) return rc;
+            } else if ((rc = mm(c, l.ffn_receptance, u8, ws.mix[0], ACT_SIGMOID, nullptr, nullptr, 1.f, ws.r, ws.xx_ffn, s.ffn_xx, C))) {
+                return rc;
+            }
+            Ctx ck = c;
+            ck.small_tiles = par ? 1 : 0;
+            if ((rc = mm(ck, l.ffn_key, u8, ws.mix[1], ACT_RELU_SQ, nullptr, nullptr, 1.f, ws.vx))) return rc;
+            if (par && !join_streams(ss, st, 1)) return (int)hipErrorUnknown;
+        }
         if ((rc = mm(c, l.ffn_value, u8, ws.vx, ACT_GATED_RESIDUAL, ws.x, ws.r, scale, ws.x))) return rc;
         RWKV_LAUNCH_CHECK();
     }

@@ -516,7 +516,7 @@ extern "C" int rwkv_v7_forward(const rwkv_v7_model *m, const rwkv_v56_layer_stat
     const int C = m->n_embd, H = m->n_head;
     Ws7 ws = carve7(workspace, T, m);
     // the fp16 path needs no scaled-activation scratch or row sums
-    Ctx c{st, false, T, num_cu(), nullptr, nullptr, nullptr, ws.splitk};
+    Ctx c{st, false, T, num_cu(), nullptr, nullptr, nullptr, ws.splitk, 0};
     const unsigned head_waves = (unsigned)(((int64_t)T * H + 3) / 4);
 
     const int max_rank = std::max(std::max(m->lora_w, m->lora_a), std::max(m->lora_v, m->lora_g));

@@ -376,3 +376,28 @@ def test_v4_side_stream_path():
         scale = max(float(np.abs(ref.astype(np.float32)).max()), 1.0)
         assert np.abs(_np(s) - ref.astype(np.float32)).max() <= 1e-2 * scale, i
         assert np.abs(_np(s) - _np(s2)).max() <= 1e-2 * scale, i
+
+
+@pytest.mark.parametrize("ver", [5.1, 6])
+def test_v56_side_stream_path(ver):
+    """RWKV-5/6 sequence calls with more than 128 output tiles per square product run receptance (+ gate), key
+    and value, and the channel-mix receptance / key products side by side: two layers at n_embd 1024 (the head
+    count is only detected from the second layer on, as in the reference), 2176 tokens, against the oracle and
+    against the same prompt in shorter calls."""
+    cfg = dict(n_layer=2, n_embd=1024, n_ffn=3584, vocab=500)
+    ck = synth.make_checkpoint(version=ver, seed=88, **cfg)
+    m, o = _rwkv()(ck, "cuda fp16i8", verbose=False), OracleRWKV(ck, "cuda fp16i8")
+    toks = synth.random_tokens(2176, cfg["vocab"], seed=6)
+    out, st = m.forward(toks, None)
+    torch.cuda.synchronize()
+    oo, ost = o.forward(toks, None)
+    d = float(np.abs(_np(out) - oo).max())
+    assert d <= LOGIT_TOL, d
+    st2 = None
+    for a in range(0, 2176, 128):
+        out2, st2 = m.forward(toks[a:a + 128], st2)
+    assert np.abs(_np(out2) - _np(out)).max() <= LOGIT_TOL
+    for i, (s, s2, ref) in enumerate(zip(st, st2, ost)):
+        scale = max(float(np.abs(ref.astype(np.float32)).max()), 1.0)
+        assert np.abs(_np(s) - ref.astype(np.float32)).max() <= 1e-2 * scale, i
+        assert np.abs(_np(s) - _np(s2)).max() <= 1e-2 * scale, i
