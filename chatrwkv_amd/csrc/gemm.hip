@@ -292,13 +292,17 @@ int launch_cfg(int64_t T, int64_t N, int64_t M, const rwkv_half *A, int64_t lda,
     // workgroups per tile; partial sums go to fp32 slabs and a second pass reduces them in slab order.
     int ks = 1;
     const int nk = (int)(N / BK);
-    if (ep.splitk_ws && tiles <= 128 && lds <= 64 * 1024 && (M & 3) == 0) {
-        // the smallest split that gives every CU a workgroup (slab traffic grows with the split)
+    // up to 128 tiles: split until every CU has a workgroup; up to 256 tiles (at most one workgroup per CU, which
+    // leaves a CU's four waves waiting on their own loads): split in two, +12-18 % on 1024 x 4096 x 4096,
+    // 1024 x 16384 x 4096 and 256 x 4096 x 16384
+    const int want = tiles <= 128 ? 256 : 512;
+    if (ep.splitk_ws && tiles <= 256 && lds <= 64 * 1024 && (M & 3) == 0) {
+        // the smallest split that reaches that many workgroups (slab traffic grows with the split)
         for (int c = 2; c <= 8; c <<= 1) {
             if (nk % c || nk / c < 8) break;                                      // whole k-tiles, several per split
             if ((size_t)c * T * M * sizeof(float) > ep.splitk_bytes) break;       // slabs must fit
             ks = c;
-            if (tiles * c >= 256) break;
+            if (tiles * c >= want) break;
         }
     }
     if (ks > 1) {

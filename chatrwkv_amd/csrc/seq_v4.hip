@@ -303,10 +303,11 @@ extern "C" int rwkv_v4_forward_seq(const rwkv_v4_model *m, const rwkv_v4_layer_s
         // side by side when none of them would split K (the split-K scratch is shared)
         const bool par = ss && (T / 128) * (C / 128) > 128 && fork_streams(ss, st, 2);
         hipStream_t sv = par ? ss->s[0] : st, sr = par ? ss->s[1] : st;
-        if ((rc = run_gemm(l.att_key, u8, T, ws.xs[0], s0[0], s2[0], ws.k, C, e, st, ws.splitk))) return rc;
-        if ((rc = run_gemm(l.att_value, u8, T, ws.xs[1], s0[1], s2[1], ws.v, C, e, sv, ws.splitk))) return rc;
+        float *sk = par ? nullptr : ws.splitk;   // products that run side by side do not split K
+        if ((rc = run_gemm(l.att_key, u8, T, ws.xs[0], s0[0], s2[0], ws.k, C, e, st, sk))) return rc;
+        if ((rc = run_gemm(l.att_value, u8, T, ws.xs[1], s0[1], s2[1], ws.v, C, e, sv, sk))) return rc;
         e.act = ACT_SIGMOID; e.out_dtype = RWKV_DT_F16; e.raw_f32 = 0;
-        if ((rc = run_gemm(l.att_receptance, u8, T, ws.xs[2], s0[2], s2[2], ws.r, C, e, sr, ws.splitk))) return rc;
+        if ((rc = run_gemm(l.att_receptance, u8, T, ws.xs[2], s0[2], s2[2], ws.r, C, e, sr, sk))) return rc;
         if (par && !join_streams(ss, st, 2)) return (int)hipErrorUnknown;
         if ((rc = wkv4_fused_launch((int)T, C, l.time_decay, l.time_first, ws.k, ws.v, u8 ? 0 : 1, ws.r, ws.rwkv, s.aa,
                                     s.bb, s.pp, st, ws.wkv)))
@@ -338,10 +339,11 @@ extern "C" int rwkv_v4_forward_seq(const rwkv_v4_model *m, const rwkv_v4_layer_s
         e.out_scale = 1.f; e.out_dtype = RWKV_DT_F16;
         e.act = ACT_SIGMOID;
         const bool par2 = ss && (T / 128) * (C / 128) > 128 && fork_streams(ss, st, 1);
-        if ((rc = run_gemm(l.ffn_receptance, u8, T, ws.xs[0], s0[0], s2[0], ws.r, C, e, par2 ? ss->s[0] : st, ws.splitk))) return rc;
+        float *sk2 = par2 ? nullptr : ws.splitk;
+        if ((rc = run_gemm(l.ffn_receptance, u8, T, ws.xs[0], s0[0], s2[0], ws.r, C, e, par2 ? ss->s[0] : st, sk2))) return rc;
         e.act = ACT_RELU_SQ;
         e.small_tiles = par2 ? 1 : 0;   // the receptance product runs beside this one
-        if ((rc = run_gemm(l.ffn_key, u8, T, ws.xs[1], s0[1], s2[1], ws.vx, F, e, st, ws.splitk))) return rc;
+        if ((rc = run_gemm(l.ffn_key, u8, T, ws.xs[1], s0[1], s2[1], ws.vx, F, e, st, sk2))) return rc;
         e.small_tiles = 0;
         if (par2 && !join_streams(ss, st, 1)) return (int)hipErrorUnknown;
         const rwkv_half *a_v = ws.vx;
