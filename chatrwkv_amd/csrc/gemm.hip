@@ -309,7 +309,7 @@ int launch_cfg(int64_t T, int64_t N, int64_t M, const rwkv_half *A, int64_t lda,
         hipLaunchKernelGGL((gemm_kernel<W_U8, BT, BM, WT, WM, PF, true>), dim3((unsigned)tiles, (unsigned)ks), dim3(64 * WT * WM), lds, st,
                            (int)T, (int)N, (int)M, (const h16 *)A, lda, W, ldw, Y, ldy, ep, nk / ks, ep.splitk_ws);
         const int64_t n = T * M;
-        const unsigned blocks = (unsigned)((n + 1023) / 1024 < 2048 ? (n + 1023) / 1024 : 2048);
+        const unsigned blocks = (unsigned)((n + 1023) / 1024 < 16384 ? (n + 1023) / 1024 : 16384);
         hipLaunchKernelGGL(splitk_epilogue_kernel, dim3(blocks), dim3(256), 0, st, (int)T, (int)M, ks, ep.splitk_ws, Y, ldy, ep);
     } else {
         hipLaunchKernelGGL((gemm_kernel<W_U8, BT, BM, WT, WM, PF, false>), dim3((unsigned)tiles), dim3(64 * WT * WM), lds, st, (int)T,
