@@ -64,9 +64,10 @@ int v4_model_check(const rwkv_v4_model *m) {
     const int64_t C = m->n_embd, F = m->n_ffn, V = m->vocab;
     if (m->n_layer <= 0 || C <= 0 || F <= 0 || V <= 0 || (C & 63) || (F & 63) || C > 8 * DTHREADS || F > 8 * VP * DTHREADS)
         return RWKV_E_SHAPE;
-    const bool u8 = m->weights_u8 != 0;
+    if (m->weights_u8 < 0 || m->weights_u8 > 2) return RWKV_E_DTYPE;
     for (int i = 0; i < m->n_layer; ++i) {
         const rwkv_v4_layer &l = m->layers[i];
+        const bool u8 = mat_is_u8(m->weights_u8, l.att_key);   // one weight type per layer
         if (!l.ln1_w || !l.ln1_b || !l.ln2_w || !l.ln2_b || !l.att_mix_k || !l.att_mix_v || !l.att_mix_r ||
             !l.time_decay || !l.time_first || !l.ffn_mix_k || !l.ffn_mix_r)
             return RWKV_E_NULL;
@@ -75,7 +76,7 @@ int v4_model_check(const rwkv_v4_model *m) {
             !mat_ok(l.ffn_value, u8, F, C))
             return RWKV_E_LAYOUT;
     }
-    if (!mat_ok(m->head, u8, C, V)) return RWKV_E_LAYOUT;
+    if (!mat_ok(m->head, mat_is_u8(m->weights_u8, m->head), C, V)) return RWKV_E_LAYOUT;
     return RWKV_OK;
 }
 
@@ -87,7 +88,7 @@ extern "C" size_t rwkv_v4_one_workspace(const rwkv_v4_model *m) {
 // Head: LN_out(x) @ head -> fp32 logits (fp16-rounded).  Shared by the one-token and the
 // sequence entry points (last token only).
 int v4_head_launch(const rwkv_v4_model *m, const rwkv_half *x, float *logits, hipStream_t st) {
-    lnhead_launch(m->weights_u8 != 0, x, m->n_embd, m->ln_out_w, m->ln_out_b, to_dev(m->head), m->vocab, logits, num_cu(), st);
+    lnhead_launch(mat_is_u8(m->weights_u8, m->head), x, m->n_embd, m->ln_out_w, m->ln_out_b, to_dev(m->head), m->vocab, logits, num_cu(), st);
     RWKV_LAUNCH_CHECK();
     return RWKV_OK;
 }
@@ -110,7 +111,6 @@ static int v4_one_impl(const rwkv_v4_model *m, const rwkv_v4_layer_state *states
     }
     hipStream_t st = (hipStream_t)stream;
     const int C = m->n_embd, F = m->n_ffn;
-    const bool u8 = m->weights_u8 != 0;
     unsigned char *p = (unsigned char *)workspace;
     OneWs ws;
     const size_t cb = align256((size_t)C * 2);
@@ -129,6 +129,7 @@ static int v4_one_impl(const rwkv_v4_model *m, const rwkv_v4_layer_state *states
         const rwkv_v4_layer &l = m->layers[i];
         const rwkv_v4_layer_state &s = states[i];
         const int32_t *tok = (i == 0) ? token : nullptr;
+        const bool u8 = mat_is_u8(m->weights_u8, l.att_key);
         if (only_phase < 0 || only_phase == 0) {
             AttArgs a{};
             a.x = ws.x; a.emb = m->emb; a.token = tok; a.C = C;

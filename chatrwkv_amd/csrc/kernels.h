@@ -60,6 +60,10 @@ int v4_model_check(const rwkv_v4_model *m);
 int v4_head_launch(const rwkv_v4_model *m, const rwkv_half *x, float *logits, hipStream_t st);
 int num_cu();
 
+// Is this matrix uint8?  weights_u8 0: no matrix is, 1: every matrix is, 2: decided per layer (and for the head) by
+// the presence of the scale vectors -- a strategy such as 'cuda fp16i8 *20 -> cuda fp16'.
+inline bool mat_is_u8(int weights_u8, const rwkv_mat &m) { return weights_u8 == 2 ? m.mx != nullptr : weights_u8 != 0; }
+
 // Two extra streams (default priority, created once per process) for contractions that are independent and each
 // too small to fill the chip; fork / join by events around them (seq_v4.hip).
 struct SideStreams {

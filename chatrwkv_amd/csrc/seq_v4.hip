@@ -268,7 +268,6 @@ extern "C" int rwkv_v4_forward_seq(const rwkv_v4_model *m, const rwkv_v4_layer_s
     }
     hipStream_t st = (hipStream_t)stream;
     const int C = m->n_embd, F = m->n_ffn;
-    const bool u8 = m->weights_u8 != 0;
     SeqWs ws = carve(workspace, T, C, F);
     float *s0[3] = {ws.sums, ws.sums + 2 * T, ws.sums + 4 * T};
     float *s2[3] = {ws.sums + T, ws.sums + 3 * T, ws.sums + 5 * T};
@@ -281,6 +280,7 @@ extern "C" int rwkv_v4_forward_seq(const rwkv_v4_model *m, const rwkv_v4_layer_s
     for (int i = 0; i < m->n_layer; ++i) {
         const rwkv_v4_layer &l = m->layers[i];
         const rwkv_v4_layer_state &s = states[i];
+        const bool u8 = mat_is_u8(m->weights_u8, l.att_key);
         // ---- time mix
         {
             SeqMixArgs a{};
@@ -357,6 +357,7 @@ extern "C" int rwkv_v4_forward_seq(const rwkv_v4_model *m, const rwkv_v4_layer_s
         RWKV_LAUNCH_CHECK();
     }
     if (!full_output) return v4_head_launch(m, ws.x + (size_t)(T - 1) * C, logits, st);
+    const bool u8 = mat_is_u8(m->weights_u8, m->head);
     {
         SeqMixArgs a{};
         a.T = (int)T; a.C = C; a.x = ws.x; a.ln_w = m->ln_out_w; a.ln_b = m->ln_out_b; a.sx = nullptr;

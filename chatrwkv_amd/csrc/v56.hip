@@ -171,9 +171,10 @@ static int v56_check(const rwkv_v56_model *m) {
     if (ver == 60 && (m->lora_maa <= 0 || m->lora_maa > 64 || (m->lora_maa * 5) % 8 || m->lora_decay % 64 ||
                       m->lora_decay <= 0))
         return RWKV_E_SHAPE;
-    const bool u8 = m->weights_u8 != 0;
+    if (m->weights_u8 < 0 || m->weights_u8 > 2) return RWKV_E_DTYPE;
     for (int i = 0; i < m->n_layer; ++i) {
         const rwkv_v56_layer &l = m->layers[i];
+        const bool u8 = mat_is_u8(m->weights_u8, l.att_key);   // one weight type per layer
         if (!l.ln1_w || !l.ln1_b || !l.ln2_w || !l.ln2_b || !l.time_decay || !l.time_first || !l.lnx_w || !l.lnx_b ||
             !l.ffn_mix_k || !l.ffn_mix_r)
             return RWKV_E_NULL;
@@ -187,7 +188,7 @@ static int v56_check(const rwkv_v56_model *m) {
             !mat_ok56(l.ffn_receptance, u8, C, C) || !mat_ok56(l.ffn_value, u8, F, C))
             return RWKV_E_LAYOUT;
     }
-    if (!mat_ok56(m->head, u8, C, V)) return RWKV_E_LAYOUT;
+    if (!mat_ok56(m->head, mat_is_u8(m->weights_u8, m->head), C, V)) return RWKV_E_LAYOUT;
     return RWKV_OK;
 }
 
@@ -212,10 +213,10 @@ extern "C" int rwkv_v56_forward(const rwkv_v56_model *m, const rwkv_v56_layer_st
     }
     hipStream_t st = (hipStream_t)stream;
     const int C = m->n_embd, F = m->n_ffn, H = m->n_head, ver = m->version_x10;
-    const bool u8 = m->weights_u8 != 0, v6 = ver == 60, gated = ver != 50;
+    const bool v6 = ver == 60, gated = ver != 50;
     const int lm = m->lora_maa, ld = m->lora_decay;
     Ws56 ws = carve56(workspace, T, C, F, v6 ? lm : 32, v6 ? ld : 64);
-    Ctx c{st, u8, T, num_cu(), ws.xs, ws.sums, ws.sums + T, ws.splitk, 0};
+    Ctx c{st, false, T, num_cu(), ws.xs, ws.sums, ws.sums + T, ws.splitk, 0};
     // Sequence calls whose square products have more than 128 output tiles (none of them would split K) run
     // independent products side by side on two extra streams, each with its own activation scratch.  Shorter
     // calls are faster one product after the other with split-K (measured at 256 tokens, n_embd 4096).
@@ -231,6 +232,7 @@ extern "C" int rwkv_v56_forward(const rwkv_v56_model *m, const rwkv_v56_layer_st
     for (int i = 0; i < m->n_layer; ++i) {
         const rwkv_v56_layer &l = m->layers[i];
         const rwkv_v56_layer_state &s = states[i];
+        const bool u8 = mat_is_u8(m->weights_u8, l.att_key);
         const rwkv_half *kx, *vx, *rx, *gx = nullptr, *wx = nullptr;
         bool fuse_d1 = false;
         if (v6) {
@@ -338,6 +340,7 @@ extern "C" int rwkv_v56_forward(const rwkv_v56_model *m, const rwkv_v56_layer_st
         RWKV_LAUNCH_CHECK();
     }
     // ---- head
+    const bool u8 = mat_is_u8(m->weights_u8, m->head);
     const bool all_rows = full_output && T > 1;
     const int64_t TH = all_rows ? T : 1;
     const rwkv_half *xh = all_rows ? ws.x : ws.x + (size_t)(T - 1) * C;

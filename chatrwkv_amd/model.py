@@ -1,7 +1,8 @@
 """``RWKV(model, strategy)`` / ``model.forward(tokens, state)`` on one MI355X.
 
 Drop-in for the class of the same name in rwkv_pip_package/src/rwkv/model.py:612-1677 for
-the strategies 'cuda fp16i8' and 'cuda fp16': same constructor and forward signatures, same
+the strategies 'cuda fp16i8', 'cuda fp16' and chains of the two on one GPU ('cuda fp16i8 *20 -> cuda
+fp16'): same constructor and forward signatures, same
 state-list layout, dtypes and initial values (model.py:1448-1471), same chunked-prefill
 behaviour (len(tokens) == 1 -> one-token mode, > 1 -> sequence mode, state carried
 between calls).  Everything numeric runs in librwkv_hip.so; PyTorch provides device
@@ -131,7 +132,6 @@ class RWKV:
         args, dev, R = self.args, self.device, self.RESCALE_LAYER
         L = _lib.load()
         st = torch.cuda.current_stream().cuda_stream
-        u8 = self._wkind == 'u8'
         out = {}
         real_time_first = any('.time_faaaa' in k for k in w)          # model.py:764-771
         if real_time_first:
@@ -165,6 +165,9 @@ class RWKV:
                     out[x] = t.to(dev).contiguous()
                 continue
             if is_matrix:
+                # the slot of the tensor's layer decides its type; ln_out and head sit in the last slot (model.py:776-778)
+                slot = self.strategy[layer_id if 'blocks.' in x else args.n_layer]
+                u8 = slot.wtype == torch.uint8
                 t = t.to(device=dev, dtype=torch.float32)
                 if R > 0 and ('att.output.weight' in x or 'ffn.value.weight' in x):
                     t = t / (2 ** int(layer_id // R))                 # model.py:785-789 (exact scaling)
@@ -252,7 +255,7 @@ class RWKV:
         m.n_layer, m.n_embd, m.n_ffn = a.n_layer, a.n_embd, a.n_ffn
         m.vocab = w['emb.weight'].shape[0]
         m.rescale_layer = self.RESCALE_LAYER
-        m.weights_u8 = 1 if self._wkind == 'u8' else 0
+        m.weights_u8 = {'f16': 0, 'u8': 1, 'mixed': 2}[self._wkind]
         m.emb = w['emb.weight'].data_ptr()
         m.ln_out_w, m.ln_out_b = w['ln_out.weight'].data_ptr(), w['ln_out.bias'].data_ptr()
         m.head = self._mat('head.weight')
@@ -319,7 +322,7 @@ class RWKV:
             m.lora_maa = w['blocks.0.att.time_maa_w2'].shape[1]
             m.lora_decay = w['blocks.0.att.time_decay_w1'].shape[1]
         m.rescale_layer = self.RESCALE_LAYER
-        m.weights_u8 = 1 if self._wkind == 'u8' else 0
+        m.weights_u8 = {'f16': 0, 'u8': 1, 'mixed': 2}[self._wkind]
         m.emb = w['emb.weight'].data_ptr()
         m.ln_out_w, m.ln_out_b = w['ln_out.weight'].data_ptr(), w['ln_out.bias'].data_ptr()
         m.head = self._mat('head.weight')

@@ -4,9 +4,10 @@ Restates the planner of RWKV.__init__ (rwkv_pip_package/src/rwkv/model.py:620-75
 strategy is a chain of segments ``device dtype[i8] [*N | *N+]`` joined by ``->``; the
 n_layer + 1 slots (the last one holds ln_out + head, model.py:776-778) are dealt to the
 segments in order.  This package then runs only plans that put every slot on one ROCm
-GPU with fp16 activations and uint8 or fp16 weights ('cuda fp16i8', 'cuda fp16'); any other
-valid strategy raises NotImplementedError, an invalid string raises ValueError as the
-reference does (model.py:621-622).
+GPU with fp16 activations and uint8 or fp16 weights: 'cuda fp16i8', 'cuda fp16', and chains of the
+two on the same GPU such as 'cuda fp16i8 *20 -> cuda fp16' (uint8 weights for the first 20 layers,
+fp16 for the rest and the head).  Any other valid strategy raises NotImplementedError, an invalid
+string raises ValueError as the reference does (model.py:621-622).
 """
 import re
 import types
@@ -87,19 +88,19 @@ def plan(strategy, n_layer):
 
 
 def require_single_gpu(slots):
-    """Check that a plan is one this package runs; return 'u8' or 'f16' (the weight type)."""
-    first = slots[0]
+    """Check that a plan is one this package runs; return the weight type: 'u8', 'f16', or 'mixed' when
+    the slots differ (then each layer, and the head, has the type of its own slot)."""
+    kinds = set()
     for s in slots:
         if s is None:
             raise NotImplementedError("strategy leaves layers unassigned")
         if not str(s.device).startswith("cuda") or s.stream:
             raise NotImplementedError(
-                "chatrwkv_amd runs single-GPU strategies only ('cuda fp16i8' or 'cuda fp16'); "
+                "chatrwkv_amd runs single-GPU strategies only ('cuda fp16i8', 'cuda fp16' and chains of the two); "
                 f"got device {s.device!r}{' with streaming' if s.stream else ''}")
-        if s.device != first.device or s.atype != first.atype or s.wtype != first.wtype:
-            raise NotImplementedError("chatrwkv_amd does not split a model across devices or dtypes")
-    if first.device not in ("cuda", "cuda:0"):
-        raise NotImplementedError("chatrwkv_amd uses GPU 0 only")
-    if first.atype != torch.float16 or first.wtype not in (torch.uint8, torch.float16):
-        raise NotImplementedError("supported strategies: 'cuda fp16i8' and 'cuda fp16'")
-    return "u8" if first.wtype == torch.uint8 else "f16"
+        if s.device not in ("cuda", "cuda:0"):
+            raise NotImplementedError("chatrwkv_amd uses GPU 0 only")
+        if s.atype != torch.float16 or s.wtype not in (torch.uint8, torch.float16):
+            raise NotImplementedError("supported strategies: 'cuda fp16i8', 'cuda fp16' and chains of the two")
+        kinds.add("u8" if s.wtype == torch.uint8 else "f16")
+    return kinds.pop() if len(kinds) == 1 else "mixed"

@@ -181,7 +181,9 @@ typedef struct {
 typedef struct {
     int32_t n_layer, n_embd, n_ffn, vocab;
     int32_t rescale_layer;  /* x /= 2 after every rescale_layer-th layer; 0 = never (model.py:1660-1662) */
-    int32_t weights_u8;     /* 1: uint8 matrices ('cuda fp16i8'); 0: fp16 matrices ('cuda fp16') */
+    int32_t weights_u8;     /* 1: uint8 matrices ('cuda fp16i8'); 0: fp16 matrices ('cuda fp16'); 2: per layer and for
+                             * the head, uint8 where the scale vectors are non-NULL ('cuda fp16i8 *20 -> cuda fp16';
+                             * all matrices of one layer have one type, model.py:776-778) */
     const rwkv_half *emb;   /* [vocab, C] fp16, ln0 already applied (model.py:756) */
     const rwkv_half *ln_out_w, *ln_out_b;
     rwkv_mat head;          /* [C -> vocab] */
@@ -257,7 +259,7 @@ typedef struct {
     int32_t version_x10;    /* 50, 51, 52 or 60 */
     int32_t n_layer, n_embd, n_ffn, vocab, n_head;
     int32_t lora_maa, lora_decay;   /* v6 LoRA ranks (32 / 64 in released models) */
-    int32_t rescale_layer, weights_u8;
+    int32_t rescale_layer, weights_u8;   /* weights_u8 as in rwkv_v4_model */
     const rwkv_half *emb, *ln_out_w, *ln_out_b;
     rwkv_mat head;
     const rwkv_v56_layer *layers;

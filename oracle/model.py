@@ -31,7 +31,49 @@ import numpy as np
 from . import ops, quant
 from .ops import Mat, f16, f32
 
-_STRATEGY = re.compile(r"^ *(cuda(?::0)?|cpu) (fp16|fp32)(i8)? *$")
+_SEGMENT = re.compile(r"^ *(cuda(?::0)?|cpu) (fp16|fp32)(i8)?(?: \*(\d+))? *$")
+
+
+def plan_wtypes(strategy, n_layer):
+    """Weight type of each of the n_layer + 1 slots (the last holds ln_out + head) for a chain of segments
+    ``device dtype[i8] [*N]`` on ONE device with ONE activation dtype: the slot allocation of
+    model.py:694-750 restricted to what the oracle emulates (no streaming, no second device).  Segments with a
+    count take that many slots in order, the segments without one share the rest equally, and what is
+    still left goes to the last segment.  Returns (device, activation, [is_uint8 per slot])."""
+    segs = []
+    for part in strategy.split('->'):
+        m = _SEGMENT.match(part)
+        if not m:
+            raise ValueError("oracle supports chains of 'cpu|cuda fp16|fp32[i8] [*N]' segments")
+        segs.append((m.group(1).replace(':0', ''), m.group(2), bool(m.group(3)), int(m.group(4)) if m.group(4) else None))
+    if len({(d, a) for d, a, _, _ in segs}) != 1:
+        raise ValueError("oracle emulates one device and one activation dtype")
+    slots = n_layer + 1
+    counts = [c or 0 for _, _, _, c in segs]
+    dealt = 0
+    for i, c in enumerate(counts):                                    # model.py:709-722
+        if segs[i][3] is None:
+            continue
+        dealt += c
+        if dealt >= slots:
+            counts[i] += slots - dealt
+            for j in range(i + 1, len(counts)):
+                counts[j] = 0
+            dealt = slots
+            break
+    open_segs = [i for i, s in enumerate(segs) if s[3] is None]
+    if dealt < slots and open_segs:                                   # model.py:723-735
+        left = len(open_segs)
+        for i in open_segs:
+            counts[i] = (slots - dealt) // left
+            dealt += counts[i]
+            left -= 1
+    if dealt < slots:
+        counts[-1] += slots - dealt
+    kinds = []
+    for (dev, at, i8, _), c in zip(segs, counts):
+        kinds += [i8] * c
+    return segs[0][0], segs[0][1], kinds[:slots]
 
 _MATRIX_KEYS = ('key.weight', 'value.weight', 'receptance.weight', 'gate.weight',
                 'output.weight', 'head.weight')
@@ -43,12 +85,11 @@ def _np(t):
 
 class OracleRWKV:
     def __init__(self, checkpoint, strategy, rescale_layer=None, cache_dequant=None):
-        m = _STRATEGY.match(strategy)
-        if not m:
-            raise ValueError("oracle supports single-segment cpu/cuda fp32/fp16[i8] strategies")
-        self.device, at, i8 = m.group(1), m.group(2), m.group(3)
+        self.strategy = strategy
+        n_layer = 1 + max(int(k.split('.')[1]) for k in checkpoint if k.startswith('blocks.'))
+        self.device, at, self.slot_u8 = plan_wtypes(strategy, n_layer)
         self.atype = f32 if at == 'fp32' else f16
-        self.wtype = np.uint8 if i8 else self.atype
+        self.wtype = np.uint8 if all(self.slot_u8) else self.atype      # of a uniform model
         # model.py:631-634
         if rescale_layer is None:
             env = os.environ.get("RWKV_RESCALE_LAYER")
@@ -162,7 +203,8 @@ class OracleRWKV:
             elif '.ln_x' in x:                                       # model.py:815-816
                 out[x] = t.astype(f32)
             elif t.ndim == 2 and 'emb' not in x and '_w1' not in x and '_w2' not in x:
-                if self.wtype != np.uint8:                           # model.py:819-820
+                # the slot of the tensor's layer decides; ln_out / head sit in the last slot (model.py:776-778)
+                if not self.slot_u8[lid if 'blocks.' in x else self.n_layer]:   # model.py:819-820
                     out[x] = np.ascontiguousarray(t).astype(self.wtype)
                 else:                                                # model.py:821-847
                     q, mx, rx, my, ry = quant.quantize_u8(t, atype=A)

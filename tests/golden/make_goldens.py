@@ -18,6 +18,8 @@ RWKV_CUDA_ON=0 (no native build), feeds it synthetic checkpoints from
                             tensors, RESCALE_LAYER = 6): pins where the fp16 path rounds; and
   e2e_<ver>_l8_cpu_fp16.npz 8-layer RWKV-4 / RWKV-6 models (n_embd 64) under 'cpu fp16', deep enough for
                             the rescale (x / 2 after layer 6, matrices of layers >= 6 halved) to act
+  e2e_<ver>_mixed_cpu.npz   RWKV-4 / RWKV-6 under 'cpu fp32i8 *2 -> cpu fp32': uint8 weights for two layers, float
+                            weights for the third and the head
   planner.json              the per-slot plan the reference prints for a list of strategy strings
   e2e_v4_169m_cpu_fp32i8.npz  the 169M-shape model: 128-token prefill + 32 greedy steps;
                             argmax per position, 256 fixed logits per position, state sums
@@ -96,6 +98,32 @@ def quant_cuda_convert(tmp):
 
 def _state_np(state):
     return {f"state_{i}": s.detach().float().cpu().contiguous().numpy() for i, s in enumerate(state)}
+
+
+MIXED = "cpu fp32i8 *2 -> cpu fp32"
+
+
+def e2e_mixed(tmp):
+    """A chain of weight types on one device: uint8 for the first two layers, float for the third and the head."""
+    RWKV = _ref()
+    for ver, tag in ((4, "v4"), (6, "v6_0")):
+        ck = synth.make_checkpoint(version=ver, seed=200 + int(ver * 10), **TINY)
+        p = os.path.join(tmp, f"mixed_{tag}.pth")
+        _save_ckpt(ck, p)
+        toks = synth.random_tokens(9, TINY["vocab"], seed=PROMPT_SEED)
+        m = RWKV(p, MIXED, verbose=False)
+        kinds = [str(m.w[f"blocks.{i}.att.key.weight"].dtype) for i in range(TINY["n_layer"])] + [str(m.w["head.weight"].dtype)]
+        full, st_full = m.forward(toks, None, full_output=True)
+        outs, st = [], None
+        for a, b in ((0, 2), (2, 3), (3, 7), (7, 8), (8, 9)):
+            o, st = m.forward(toks[a:b], st)
+            outs.append(o.detach().float().cpu().numpy())
+        d = {"tokens": np.array(toks), "full_logits": full.detach().float().cpu().numpy(), "chunk_logits": np.stack(outs),
+             "weight_kinds": np.array(kinds)}
+        d.update({"chunk_" + k: v for k, v in _state_np(st).items()})
+        name = f"e2e_{tag}_mixed_cpu.npz"
+        np.savez_compressed(os.path.join(HERE, name), **d)
+        print("wrote", name, kinds)
 
 
 def e2e_deep_fp16(tmp):
@@ -190,6 +218,8 @@ PLAN_STRATEGIES = [
     "cuda fp16 *0+ -> cpu fp32 *1", "cuda fp16i8 *4 -> cuda fp16 *3 -> cpu fp32", "cuda fp16 *6+",
     "cuda fp16i8 *2 -> cuda fp16 *2+ -> cpu fp32 *1", "cuda fp16 -> cuda:1 fp16", "cpu bf16", "cuda fp16i8 *100",
     "cuda fp16 *3 -> cuda:1 fp16 *3 -> cpu fp32",
+    "cuda fp16 *3 -> cuda fp16i8", "cuda fp16i8 *2 -> cuda fp16 *3 -> cuda fp16i8", "cuda fp16i8 -> cuda fp16",
+    "cuda fp16i8 *2 -> cuda fp16 -> cuda fp16i8 *1", "cuda fp16i8 *9 -> cuda fp16", "cuda:0 fp16i8 *5 -> cuda fp16",
 ]
 
 
@@ -221,13 +251,15 @@ def planner(tmp):
 if __name__ == "__main__":
     torch.manual_seed(0)
     with tempfile.TemporaryDirectory() as tmp:
-        which = sys.argv[1:] or ["quant_cpu", "quant_cuda", "tiny", "fp16", "169m", "planner"]
+        which = sys.argv[1:] or ["quant_cpu", "quant_cuda", "tiny", "fp16", "mixed", "169m", "planner"]
         if "planner" in which:
             planner(tmp)
         if "fp16" in which and "tiny" not in which:
             e2e_tiny(tmp, which_strats=("cpu fp16",))   # only the half-precision files
         if "fp16" in which:
             e2e_deep_fp16(tmp)
+        if "mixed" in which:
+            e2e_mixed(tmp)
         if "quant_cpu" in which:
             quant_cpu(tmp)
         if "quant_cuda" in which:

@@ -401,3 +401,34 @@ def test_v56_side_stream_path(ver):
         scale = max(float(np.abs(ref.astype(np.float32)).max()), 1.0)
         assert np.abs(_np(s) - ref.astype(np.float32)).max() <= 1e-2 * scale, i
         assert np.abs(_np(s) - _np(s2)).max() <= 1e-2 * scale, i
+
+
+@pytest.mark.parametrize("ver", [4, 5.2, 6])
+@pytest.mark.parametrize("strat", ["cuda fp16i8 *2 -> cuda fp16", "cuda fp16 *1 -> cuda fp16i8"])
+def test_mixed_weight_types_on_one_gpu(ver, strat):
+    """Chains of 'cuda fp16i8' and 'cuda fp16' segments on the one GPU: every layer (and the head) runs with the
+    weight type of its slot.  Against the oracle's emulation of the same chain: converted weights, logits of
+    a sequence call with full_output, one-token steps (graph replay) and the final state."""
+    ck = synth.make_checkpoint(version=ver, seed=410 + int(ver * 10), **TINY)
+    m, o = _rwkv()(ck, strat, verbose=False), OracleRWKV(ck, strat)
+    for i in range(TINY["n_layer"]):
+        k = f"blocks.{i}.att.key.weight"
+        assert (m.w[k].dtype == torch.uint8) == (o.w[k].dtype == np.uint8) == bool(o.slot_u8[i]), k
+        if o.slot_u8[i]:
+            assert np.array_equal(m.w[k].cpu().numpy(), o.w[k])
+    assert (m.w["head.weight"].dtype == torch.uint8) == bool(o.slot_u8[-1])
+    kinds = {bool(b) for b in o.slot_u8}
+    assert kinds == {True, False}
+    toks = synth.random_tokens(12, TINY["vocab"], seed=PROMPT_SEED)
+    full, st = m.forward(toks[:9], None, full_output=True)
+    ofull, ost = o.forward(toks[:9], None, full_output=True)
+    d = float(np.abs(_np(full) - ofull).max())
+    assert d <= LOGIT_TOL, d
+    assert _argmax_agree(_np(full), ofull, d)
+    for t in toks[9:]:
+        out, st = m.forward([t], st)
+        oo, ost = o.forward([t], ost)
+        assert np.abs(_np(out) - oo).max() <= LOGIT_TOL
+    for i, (s, ref) in enumerate(zip(st, ost)):
+        scale = max(float(np.abs(ref.astype(np.float32)).max()), 1.0)
+        assert np.abs(_np(s) - ref.astype(np.float32)).max() <= 1e-2 * scale, i

@@ -144,3 +144,27 @@ def test_fp16_rescale_matches_reference(ver, tag):
     full, _ = wrong.forward(toks, None, full_output=True)
     # mathematically invisible (LayerNorm follows), so still close: the check above is what pins the placement
     assert np.abs(full - ref["full_logits"]).max() < 0.05
+
+
+@pytest.mark.parametrize("ver,tag", [(4, "v4"), (6, "v6_0")])
+def test_mixed_weight_types_match_reference(ver, tag):
+    """'cpu fp32i8 *2 -> cpu fp32': two uint8 layers, then a float layer and a float head, against the
+    reference's run of the same chain."""
+    from tests.golden.make_goldens import MIXED
+    ref = _load(f"e2e_{tag}_mixed_cpu.npz")
+    ck = synth.make_checkpoint(version=ver, seed=200 + int(ver * 10), **TINY)
+    o = OracleRWKV(ck, MIXED)
+    kinds = [str(k) for k in ref["weight_kinds"]]
+    assert kinds == ["torch.uint8", "torch.uint8", "torch.float32", "torch.float32"]
+    assert [o.w[f"blocks.{i}.att.key.weight"].dtype == np.uint8 for i in range(3)] + [o.w["head.weight"].dtype == np.uint8] \
+        == [True, True, False, False]
+    toks = [int(t) for t in ref["tokens"]]
+    full, _ = o.forward(toks, None, full_output=True)
+    np.testing.assert_allclose(full, ref["full_logits"], rtol=2e-4, atol=2e-5)
+    st, outs = None, []
+    for a, b in ((0, 2), (2, 3), (3, 7), (7, 8), (8, 9)):
+        out, st = o.forward(toks[a:b], st)
+        outs.append(out)
+    np.testing.assert_allclose(np.stack(outs), ref["chunk_logits"], rtol=2e-4, atol=2e-5)
+    for i, s in enumerate(st):
+        np.testing.assert_allclose(s, ref[f"chunk_state_{i}"], rtol=2e-4, atol=2e-5, err_msg=str(i))

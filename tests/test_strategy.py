@@ -33,11 +33,33 @@ def test_only_single_gpu_plans_are_accepted():
     assert strategy.require_single_gpu(strategy.plan("cuda fp16i8", 4)) == "u8"
     assert strategy.require_single_gpu(strategy.plan("cuda:0 fp16", 4)) == "f16"
     assert strategy.require_single_gpu(strategy.plan("cuda fp16i8 *100", 4)) == "u8"
+    # chains of the two weight types on the one GPU
+    assert strategy.require_single_gpu(strategy.plan("cuda fp16i8 *1 -> cuda fp16", 4)) == "mixed"
+    assert strategy.require_single_gpu(strategy.plan("cuda:0 fp16 *2 -> cuda fp16i8", 4)) == "mixed"
+    assert strategy.require_single_gpu(strategy.plan("cuda fp16i8 *9 -> cuda fp16", 4)) == "u8"   # the first segment takes all
     for s in ("cpu fp32", "cpu fp32i8", "cuda fp32", "cuda bf16", "cuda fp16i8 -> cpu fp32 *1", "cuda fp16 *2+",
-              "cuda fp16 -> cuda:1 fp16", "cuda:1 fp16", "cuda fp16i8 *1 -> cuda fp16"):
+              "cuda fp16 -> cuda:1 fp16", "cuda:1 fp16", "cuda fp16i8 *1 -> cuda fp32"):
         with pytest.raises(NotImplementedError):
             strategy.require_single_gpu(strategy.plan(s, 4))
 
 
 def test_normalize_spelling():
     assert strategy.normalize("cuda fp16i8 *2->cpu fp32") == "cuda fp16i8 *2 -> cpu fp32"
+
+
+def test_oracle_planner_matches_reference():
+    """The oracle's own restatement of the slot allocation (used for chains of weight types on one device)
+    against the same golden plans."""
+    from oracle.model import plan_wtypes
+    gold = json.load(open(os.path.join(G, "planner.json")))
+    n = 0
+    for strat, line in gold["plans"].items():
+        try:
+            dev, at, kinds = plan_wtypes(strat, gold["n_layer"])
+        except ValueError:
+            continue                      # second device, streaming, bf16: not emulated
+        ref = [tok.split("-") for tok in line.split()]
+        assert [r[3] == "uint8" for r in ref] == kinds, strat
+        assert all(r[1].replace(":0", "") == dev for r in ref), strat
+        n += 1
+    assert n >= 14
