@@ -208,6 +208,26 @@ def test_v7_side_stream_path(tiny7):
         assert np.abs(_np(s) - _np(s2)).max() <= 1e-2 * scale, i
 
 
+def test_v7_wider_model_default_lora_ranks():
+    """n_embd 1024 (16 heads) with the LoRA ranks released checkpoints of that width use (64, 64, 32, 160: two of
+    them need padding): a 300-token call (side streams, several staging slabs), then one-token steps."""
+    cfg = dict(n_layer=2, n_embd=1024, n_ffn=4096, vocab=400)
+    assert synth.v7_lora_dims(1024) == (64, 64, 32, 160)
+    ck = synth.make_checkpoint_v7(seed=72, **cfg)
+    m, o = _x070()(ck, "cuda fp16"), OracleRWKV7(ck, "cuda fp16", kernel_form=True)
+    toks = synth.random_tokens(304, cfg["vocab"], seed=12)
+    out, st = m.forward(toks[:300], None)
+    oo, ost = o.forward(toks[:300], None)
+    assert np.abs(_np(out) - oo.astype(np.float32)).max() <= LOGIT_TOL
+    for t in toks[300:]:
+        out, st = m.forward([t], st)
+        oo, ost = o.forward([t], ost)
+        assert np.abs(_np(out) - oo.astype(np.float32)).max() <= LOGIT_TOL
+    for i, (s, ref) in enumerate(zip(st, ost)):
+        scale = max(float(np.abs(ref.astype(np.float32)).max()), 1.0)
+        assert np.abs(_np(s) - ref.astype(np.float32)).max() <= 1e-2 * scale, i
+
+
 def test_v7_api_errors(tiny7):
     m, _, ck = tiny7
     with pytest.raises(IndexError):
