@@ -125,19 +125,40 @@ def mm8(x, w, mx, rx, my, ry):
     return cuda_mm8_seq(x.shape[0], w.shape[0], w.shape[1], x, w, mx, rx, my, ry)
 
 
+def _input_contiguous_f16(b):
+    """A 2-D fp16 matrix [N, M] in the layout the kernels stream (strides (1, N)); copies only if it is not."""
+    if b.stride(0) == 1 and b.stride(1) >= b.shape[0] and b.stride(1) % 8 == 0:
+        return b
+    return b.t().contiguous().t()
+
+
 def matmul_float(a, b, output_dtype=None):
     """model.py:144-161 (gemm_fp16_cublas): fp16 x fp16, fp32 accumulation, output written
-    directly in ``output_dtype`` (fp16 or fp32).  1-D ``a`` gives a 1-D result."""
+    directly in ``output_dtype`` (fp16 or fp32).  1-D ``a`` gives a 1-D result; 3-D ``a`` and ``b`` are a
+    batch of products (cuda/gemm_fp16_cublas.cpp:61-75), run one after the other."""
     _need_cuda(a, b)
     if output_dtype is None:
         output_dtype = a.dtype
     assert a.dtype == b.dtype == torch.float16
     assert output_dtype in (torch.float16, torch.float32)
+    if a.dim() == 3:
+        assert b.dim() == 3 and a.shape[0] == b.shape[0]
+        c = torch.empty((a.shape[0], a.shape[1], b.shape[-1]), dtype=output_dtype, device=a.device)
+        for i in range(a.shape[0]):
+            c[i] = matmul_float(a[i], b[i], output_dtype=output_dtype)
+        return c
     one = a.dim() == 1
     a2 = a.unsqueeze(0) if one else a
     assert a2.dim() == 2 and b.dim() == 2
-    if a2.stride(1) != 1:
+    # the contraction kernel steps K by 64 (8 for a one-row product): pad the inner dimension with zeros
+    step = 8 if a2.shape[0] == 1 else 64
+    if a2.shape[1] % step:
+        pad = step - a2.shape[1] % step
+        a2 = torch.nn.functional.pad(a2, (0, pad))
+        b = torch.nn.functional.pad(b, (0, 0, 0, pad))
+    if a2.stride(1) != 1 or a2.stride(0) % 8 != 0:
         a2 = a2.contiguous()
+    b = _input_contiguous_f16(b)
     B, N = a2.shape
     M = b.shape[1]
     c = torch.empty((B, M), dtype=output_dtype, device=a.device)

@@ -145,6 +145,22 @@ def test_gemm_f16(N, M, B, out_dtype):
     assert d <= tol, (d, tol)
 
 
+def test_gemm_f16_batched_and_row_major():
+    """3-D operands are a batch of products (the RWKV-6 LoRA use, model.py:1269: [5, T, 32] x [5, 32, C]), and a
+    plain row-major weight tensor is accepted (converted to the streamed layout)."""
+    ops = _ops()
+    r = _rng(99)
+    a = (r.standard_normal((5, 9, 32))).astype(np.float16)
+    b = (r.standard_normal((5, 32, 256)) * 0.1).astype(np.float16)
+    ref = np.einsum("bij,bjk->bik", a.astype(np.float64), b.astype(np.float64))
+    y = ops.matmul_float(torch.from_numpy(a).to(DEV), torch.from_numpy(b).to(DEV))
+    assert y.dtype == torch.float16 and tuple(y.shape) == (5, 9, 256)
+    assert np.abs(y.cpu().numpy().astype(np.float64) - ref).max() <= np.abs(ref).max() * 2 ** -10 + 1e-4
+    y32 = ops.matmul_float(torch.from_numpy(a[0]).to(DEV), torch.from_numpy(b[0]).to(DEV), output_dtype=torch.float32)
+    assert y32.dtype == torch.float32
+    assert np.abs(y32.cpu().numpy().astype(np.float64) - ref[0]).max() <= 1e-4 * max(np.abs(ref[0]).max(), 1.0)
+
+
 # ------------------------------------------------------------------------------ WKV
 @pytest.mark.parametrize("T,C", [(1, 768), (7, 768), (64, 1000), (300, 768), (1024, 4096)])
 def test_wkv4(T, C):
