@@ -80,6 +80,26 @@ def test_wkv7_operator(dtype):
         assert np.abs(_np(S) - S_ref).max() <= 2e-5 * max(float(np.abs(S_ref).max()), 1.0), T
 
 
+def test_rwkv7_op_wrapper():
+    """ops.RWKV7_OP keeps the reference's call form (model.py:218-219)."""
+    from chatrwkv_amd import ops
+    rng = np.random.Generator(np.random.PCG64(18))
+    T, H, N = 5, 2, 64
+    C = H * N
+    r, k, v = ((rng.standard_normal((T, C)) * 0.5).astype(np.float16) for _ in range(3))
+    kk = rng.standard_normal((T, C))
+    kk /= np.linalg.norm(kk.reshape(T, H, N), axis=-1, keepdims=True).repeat(N, -1).reshape(T, C)
+    a, b = (-kk).astype(np.float16), (kk * rng.random((T, C))).astype(np.float16)
+    w = rng.uniform(-4.0, -0.5, (T, C)).astype(np.float16)
+    S0 = (rng.standard_normal((H, N, N)) * 0.1).astype(np.float32)
+    y_ref, S_ref = model_v7.wkv7_kernel(S0, r, w, k, v, a, b)
+    S = torch.from_numpy(S0.copy()).cuda()
+    y = ops.RWKV7_OP(S, *(torch.from_numpy(x).cuda() for x in (r, w, k, v, a, b)))
+    assert y.dtype == torch.float16 and tuple(y.shape) == (T, C)
+    assert np.abs(_np(y) - y_ref.astype(np.float32)).max() <= 2e-3 * max(float(np.abs(y_ref.astype(np.float32)).max()), 1.0)
+    assert np.abs(_np(S) - S_ref).max() <= 2e-5 * max(float(np.abs(S_ref).max()), 1.0)
+
+
 def test_wkv7_operator_rejects_bad_shapes():
     from chatrwkv_amd import lib as _lib
     L = _lib.load()
