@@ -16,6 +16,7 @@ One JSON line is printed:
                         the 8 TB/s HBM peak
   decode_hbm            whole-step figure: uint8 weight bytes per token x tokens/s / 8 TB/s
   prefill               prefill tokens/s and the MFMA fraction of the whole prefill
+  isolated_mm8_op       the dequant-matmul operator alone at the 7B shapes: mm8_one GB/s, mm8_seq TFLOP/s
   prefill_roofline      the prefill contraction alone on the model's largest matrix shape: 2 T N M flops /
                         mean launch duration (HIP events), against the 2.5 PFLOP/s dense fp16 MFMA peak
   cpu_baseline          the oracle's 'cpu fp32i8' path (numpy port of the reference's CPU arithmetic)
@@ -138,6 +139,58 @@ def gemm_roofline(T, N, M, u8, reps=10):
     return {"bound": "mfma", "kernel": f"{name}, [{T} x {N}] x [{N} x {M}]", "achieved": flops / t / 1e12,
             "peak": MFMA_F16_PEAK / 1e12, "unit": "TFLOP/s", "frac": flops / t / MFMA_F16_PEAK, "traffic": None,
             "flops_per_launch": flops, "ms_per_launch": t * 1e3}
+
+
+def isolated_mm8(reps=40):
+    """The isolated uint8 dequant-matmul operator at the 7B shapes (uint8 [4096 x 4096] and [4096 x 16384] with
+    fp16 scales, fp16 x ~ N(0, 1)): mm8_one as GB/s of weight bytes (each call streams a different copy of the
+    matrix, more than the 256 MB memory-side cache in total) and mm8_seq at 1024 rows as TFLOP/s, both
+    through the C ABI and timed with events on the launch stream."""
+    import torch
+    from chatrwkv_amd import lib
+    L = lib.load()
+    dev = "cuda:0"
+    st = torch.cuda.current_stream().cuda_stream
+    out = {}
+    for N, M in ((4096, 4096), (4096, 16384)):
+        ncopy = max(2, (640 << 20) // (N * M))
+        w = torch.randint(0, 256, (ncopy, M, N), dtype=torch.uint8, device=dev)
+        mx = torch.randn(M, device=dev).half(); rx = (torch.rand(M, device=dev) * 0.01).half()
+        my = torch.randn(N, device=dev).half(); ry = (torch.rand(N, device=dev) * 0.06).half()
+        x1 = torch.randn(N, device=dev).half()
+        y1 = torch.empty(M, device=dev, dtype=torch.float16)
+
+        def one(i):
+            lib.check(L.rwkv_mm8_one_f16(N, M, x1.data_ptr(), w[i % ncopy].data_ptr(), 1, N, mx.data_ptr(), rx.data_ptr(),
+                                         my.data_ptr(), ry.data_ptr(), y1.data_ptr(), lib.RWKV_DT_F16, st), "rwkv_mm8_one_f16")
+        T = 1024
+        xs = torch.randn(T, N, device=dev).half()
+        ys = torch.empty(T, M, device=dev, dtype=torch.float16)
+        nbytes = L.rwkv_mm8_seq_workspace(T, N)
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+
+        def seq(i):
+            lib.check(L.rwkv_mm8_seq_f16(T, N, M, xs.data_ptr(), N, w[i % ncopy].data_ptr(), 1, N, mx.data_ptr(), rx.data_ptr(),
+                                         my.data_ptr(), ry.data_ptr(), ys.data_ptr(), M, ws.data_ptr(), nbytes, st),
+                      "rwkv_mm8_seq_f16")
+        for name, fn, n in (("mm8_one", one, reps), ("mm8_seq", seq, max(4, reps // 4))):
+            for i in range(3):
+                fn(i)
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            torch.cuda.synchronize()
+            e0.record()
+            for i in range(n):
+                fn(i)
+            e1.record()
+            torch.cuda.synchronize()
+            t = e0.elapsed_time(e1) * 1e-3 / n
+            if name == "mm8_one":
+                out[f"mm8_one [{N}] x [{N} x {M}]"] = {"us": t * 1e6, "GBps": N * M / t / 1e9, "frac_of_hbm_peak": N * M / t / HBM_PEAK}
+            else:
+                out[f"mm8_seq [{T} x {N}] x [{N} x {M}]"] = {"us": t * 1e6, "TFLOPs": 2.0 * T * N * M / t / 1e12,
+                                                           "frac_of_mfma_peak": 2.0 * T * N * M / t / MFMA_F16_PEAK}
+        del w
+    return out
 
 
 def main():
@@ -286,6 +339,8 @@ def main():
                     "frac_of_mfma_peak": prefill_flops / t_prefill / MFMA_F16_PEAK},
         "prefill_roofline": gemm_roofline(min(chunk, args.prefill), C, F, u8),
     }
+    if args.shape == "v4-7b" and u8:
+        res["isolated_mm8_op"] = isolated_mm8()
     if not args.no_cpu and version != 7:
         res["cpu_baseline"] = cpu_baseline(args.shape)
     else:
