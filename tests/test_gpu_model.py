@@ -432,3 +432,96 @@ def test_mixed_weight_types_on_one_gpu(ver, strat):
     for i, (s, ref) in enumerate(zip(st, ost)):
         scale = max(float(np.abs(ref.astype(np.float32)).max()), 1.0)
         assert np.abs(_np(s) - ref.astype(np.float32)).max() <= 1e-2 * scale, i
+
+
+def test_7b_shape_properties():
+    """The headline configuration at its full size (RWKV-4, 32 layers would take a minute to build: 6 layers of
+    the 7B shape, n_embd 4096 / ffn 16384 / vocab 50277, carry every kernel configuration the full model uses).
+    No CPU oracle at this size; the properties the path must have whatever the size:
+      * quantizer invariants on every matrix: each row and each column of the uint8 matrix holds a 0 and a 255;
+      * a 1024-token prompt in one call (side streams, large tiles, split-K) and in calls of 256 and of 1 + 1023
+        gives the same next-token logits and state within the fp16 tolerance;
+      * the one-token step is deterministic and its graph replay equals the direct launch bit for bit."""
+    L, C, F, V = 6, 4096, 16384, 50277
+    ck = synth.make_checkpoint(version=4, n_layer=L, n_embd=C, n_ffn=F, vocab=V, seed=3, device="cuda:0")
+    m = _rwkv()(ck, "cuda fp16i8", verbose=False)
+    del ck
+    torch.cuda.empty_cache()
+    for name in ("blocks.0.att.key.weight", "blocks.3.ffn.key.weight", "blocks.5.ffn.value.weight", "head.weight"):
+        q = m.w[name]                                   # logical [N, M], stored input-contiguous
+        assert q.dtype == torch.uint8
+        for dim in (0, 1):
+            assert int(q.amin(dim=dim).max()) == 0 and int(q.amax(dim=dim).min()) == 255, (name, dim)
+    toks = synth.random_tokens(1024, V, seed=4)
+    out_a, st_a = m.forward(toks, None)
+    st_b = None
+    for i in range(0, 1024, 256):
+        out_b, st_b = m.forward(toks[i:i + 256], st_b)
+    out_c, st_c = m.forward(toks[:1], None)
+    out_c, st_c = m.forward(toks[1:], st_c)
+    torch.cuda.synchronize()
+    scale = float(out_a.abs().max())
+    for other in (out_b, out_c):
+        assert float((out_a - other).abs().max()) <= LOGIT_TOL * max(scale, 1.0)
+        assert int(out_a.argmax()) == int(other.argmax())
+    for sa, sb, sc in zip(st_a, st_b, st_c):
+        big = max(float(sa.float().abs().max()), 1.0)
+        assert float((sa.float() - sb.float()).abs().max()) <= 1e-2 * big
+        assert float((sa.float() - sc.float()).abs().max()) <= 1e-2 * big
+    # one-token steps: graph replay against the direct launch from the same state, twice in a row
+    tok = int(out_a.argmax())
+    for _ in range(2):
+        snap = copy.deepcopy(st_a)
+        os.environ["RWKV_HIP_GRAPH"] = "0"
+        try:
+            eager, _ = m.forward([tok], list(snap))
+        finally:
+            os.environ["RWKV_HIP_GRAPH"] = "1"
+        torch.cuda.synchronize()
+        out, st_a = m.forward([tok], st_a)
+        assert torch.equal(out, eager)
+        for a, b in zip(st_a, snap):
+            assert torch.equal(a, b)
+        tok = int(out.argmax())
+
+
+@pytest.mark.parametrize("kind", ["v6", "v7"])
+def test_7b_shape_properties_v6_v7(kind):
+    """Two layers of the RWKV-6 ('cuda fp16i8') and RWKV-7 ('cuda fp16') 7B shapes (n_embd 4096, 64 heads, vocab
+    65536): a 1024-token prompt in one call and in calls of 256 agrees within the fp16 tolerance, and the
+    one-token graph replay equals the direct launch bit for bit."""
+    V = 65536
+    if kind == "v6":
+        ck = synth.make_checkpoint(version=6, n_layer=2, n_embd=4096, n_ffn=14336, vocab=V, seed=5, device="cuda:0")
+        m = _rwkv()(ck, "cuda fp16i8", verbose=False)
+    else:
+        from chatrwkv_amd.model_v7 import RWKV_x070
+        ck = synth.make_checkpoint_v7(n_layer=2, n_embd=4096, n_ffn=16384, vocab=V, seed=5, device="cuda:0")
+        m = RWKV_x070(ck, "cuda fp16")
+    del ck
+    torch.cuda.empty_cache()
+    toks = synth.random_tokens(1024, V, seed=6)
+    out_a, st_a = m.forward(toks, None)
+    st_b = None
+    for i in range(0, 1024, 256):
+        out_b, st_b = m.forward(toks[i:i + 256], st_b)
+    torch.cuda.synchronize()
+    scale = max(float(out_a.float().abs().max()), 1.0)
+    assert float((out_a.float() - out_b.float()).abs().max()) <= LOGIT_TOL * scale
+    for sa, sb in zip(st_a, st_b):
+        big = max(float(sa.float().abs().max()), 1.0)
+        assert float((sa.float() - sb.float()).abs().max()) <= 1e-2 * big
+    tok = int(out_a.argmax())
+    for _ in range(2):
+        snap = copy.deepcopy(st_a)
+        os.environ["RWKV_HIP_GRAPH"] = "0"
+        try:
+            eager, _ = m.forward([tok], list(snap))
+        finally:
+            os.environ["RWKV_HIP_GRAPH"] = "1"
+        torch.cuda.synchronize()
+        out, st_a = m.forward([tok], st_a)
+        assert torch.equal(out, eager)
+        for a, b in zip(st_a, snap):
+            assert torch.equal(a, b)
+        tok = int(out.argmax())
