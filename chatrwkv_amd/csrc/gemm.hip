@@ -17,6 +17,7 @@
 // only used when a larger tile would leave most CUs idle.
 // Workgroup ids are remapped so that the workgroups which share a weight tile (same m0,
 // different t0) run on the same XCD and the tile is fetched into that XCD's L2 once.
+#include <algorithm>
 #include "kernels.h"
 #include <cstdlib>
 
@@ -78,9 +79,8 @@ __global__ __launch_bounds__(256) void splitk_epilogue_kernel(int T, int M, int 
 }
 
 template <bool W_U8, int BT, int BM, int WT, int WM, int PF, bool SPLIT>
-__global__ __launch_bounds__(64 * WT * WM) void gemm_kernel(int T, int N, int M, const h16 *__restrict__ A, int64_t lda,
-                                                   const void *__restrict__ Wv, int64_t ldw, void *__restrict__ Y,
-                                                   int64_t ldy, GemmEpi ep, int nk_split, float *__restrict__ part) {
+DEV void gemm_body(int T, int N, int M, const h16 *__restrict__ A, int64_t lda, const void *__restrict__ Wv, int64_t ldw,
+                   void *__restrict__ Y, int64_t ldy, const GemmEpi &ep, int nk_split, float *__restrict__ part) {
     constexpr int NT = 64 * WT * WM;                 // threads per workgroup
     constexpr int RA = NT / 8, RB8 = NT / 4;         // tile rows one pass of 16-byte loads covers (fp16 / uint8 rows)
     static_assert(BT % (32 * WT) == 0 && BM % (32 * WM) == 0 && BT % RA == 0 && BM % RB8 == 0, "tile");
@@ -100,6 +100,7 @@ __global__ __launch_bounds__(64 * WT * WM) void gemm_kernel(int T, int N, int M,
     int bid = blockIdx.x;
     if ((gridDim.x & 7) == 0) bid = (bid & 7) * (gridDim.x >> 3) + (bid >> 3);
     const int t0 = (bid % tiles_t) * BT, m0 = (bid / tiles_t) * BM;
+    if (m0 >= M) return;   // grouped launches size the grid for their widest member
 
     constexpr int A_LD = BT / RA;                    // 16-byte loads per thread for the A tile
     constexpr int B_LD = W_U8 ? BM / RB8 : BM / RA;  // 16-byte loads per thread for the W tile
@@ -242,6 +243,37 @@ __global__ __launch_bounds__(64 * WT * WM) void gemm_kernel(int T, int N, int M,
     }
 }
 
+template <bool W_U8, int BT, int BM, int WT, int WM, int PF, bool SPLIT>
+__global__ __launch_bounds__(64 * WT * WM) void gemm_kernel(int T, int N, int M, const h16 *__restrict__ A, int64_t lda,
+                                                   const void *__restrict__ Wv, int64_t ldw, void *__restrict__ Y,
+                                                   int64_t ldy, GemmEpi ep, int nk_split, float *__restrict__ part) {
+    gemm_body<W_U8, BT, BM, WT, WM, PF, SPLIT>(T, N, M, A, lda, Wv, ldw, Y, ldy, ep, nk_split, part);
+}
+
+// Up to four contractions [T, N] x [N, M_i] in one launch (blockIdx.y picks the operands), at full depth: short
+// calls, where each of them alone would split K and need a reduction pass.
+struct GemmGroup {
+    const h16 *A[4];
+    const void *W[4];
+    void *Y[4];
+    int64_t lda, ldw[4];
+    int M[4];
+    GemmEpi ep[4];
+};
+
+template <bool W_U8, int BT, int BM, int WT, int WM, int PF>
+__global__ __launch_bounds__(64 * WT * WM) void gemm_group_kernel(int T, int N, GemmGroup g) {
+    const int gi = blockIdx.y, M = g.M[gi];
+    gemm_body<W_U8, BT, BM, WT, WM, PF, false>(T, N, M, g.A[gi], g.lda, g.W[gi], g.ldw[gi], g.Y[gi], M, g.ep[gi], N / BK,
+                                               nullptr);
+}
+
+struct PrepGroup {
+    const rwkv_half *x[4], *ry[4], *my[4];
+    rwkv_half *xs[4];
+    float *s0[4], *s2[4];
+};
+
 // xs[t, j] = fp16(x[t, j] * ry[j]);  s0[t] = sum_j x[t, j];  s2[t] = sum_j x[t, j] * my[j].  One wave per row.
 __global__ __launch_bounds__(256) void mm8_prepare_kernel(int T, int N, const rwkv_half *__restrict__ x, int64_t ldx,
                                                           const rwkv_half *__restrict__ ry,
@@ -269,6 +301,31 @@ __global__ __launch_bounds__(256) void mm8_prepare_kernel(int T, int N, const rw
     a0 = wave_sum(a0);
     a2 = wave_sum(a2);
     if (lane == 0) { s0[t] = a0; s2[t] = a2; }
+}
+
+// the same for up to four (x, matrix) pairs in one launch: blockIdx.y picks the pair
+__global__ __launch_bounds__(256) void mm8_prepare_group_kernel(int T, int N, PrepGroup g) {
+    const int gi = blockIdx.y;
+    const int t = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+    if (t >= T) return;
+    const rwkv_half *x = g.x[gi], *ry = g.ry[gi], *my = g.my[gi];
+    rwkv_half *xs = g.xs[gi];
+    float a0 = 0.f, a2 = 0.f;
+    for (int j = lane * 8; j < N; j += 64 * 8) {
+        const h16x8 xh = *(const h16x8 *)(x + (size_t)t * N + j), rh = *(const h16x8 *)(ry + j), mh = *(const h16x8 *)(my + j);
+        h16x8 o;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const float xf = (float)xh[e];
+            o[e] = (h16)(xf * (float)rh[e]);
+            a0 += xf;
+            a2 += xf * (float)mh[e];
+        }
+        *(h16x8 *)(xs + (size_t)t * N + j) = o;
+    }
+    a0 = wave_sum(a0);
+    a2 = wave_sum(a2);
+    if (lane == 0) { g.s0[gi][t] = a0; g.s2[gi][t] = a2; }
 }
 
 
@@ -362,6 +419,38 @@ int mm8_prepare_launch(int64_t T, int64_t N, const rwkv_half *x, int64_t ldx, co
     return RWKV_OK;
 }
 
+
+// n (2..4) products [T, N] x [N, M_i] of uint8 or fp16 weights with their own inputs, outputs and epilogues in one
+// launch.  uint8: x[i] is the unscaled activation, xs[i] / sums[i] (2 T floats) are scratch.
+int gemm_group_launch(bool w_u8, int n, int64_t T, int64_t N, const rwkv_half *const *x, const rwkv_mat *const *mats,
+                      void *const *Y, const GemmEpi *eps, rwkv_half *const *xs, float *const *sums, hipStream_t st) {
+    if (n < 2 || n > 4 || (N % BK)) return RWKV_E_SHAPE;
+    GemmGroup g{};
+    g.lda = N;
+    if (w_u8) {
+        PrepGroup p{};
+        for (int i = 0; i < n; ++i) {
+            p.x[i] = x[i]; p.ry[i] = mats[i]->ry; p.my[i] = mats[i]->my; p.xs[i] = xs[i]; p.s0[i] = sums[i]; p.s2[i] = sums[i] + T;
+        }
+        hipLaunchKernelGGL(mm8_prepare_group_kernel, dim3((unsigned)((T + 3) / 4), (unsigned)n), dim3(256), 0, st, (int)T, (int)N, p);
+    }
+    int64_t tiles = 0;
+    for (int i = 0; i < n; ++i) {
+        if (mats[i]->N != N) return RWKV_E_SHAPE;
+        g.A[i] = (const h16 *)(w_u8 ? xs[i] : x[i]);
+        g.W[i] = mats[i]->w; g.ldw[i] = mats[i]->ld; g.Y[i] = Y[i]; g.M[i] = (int)mats[i]->M;
+        g.ep[i] = eps[i];
+        g.ep[i].ldres = g.ep[i].ldgate = mats[i]->M;
+        if (w_u8) { g.ep[i].mx = mats[i]->mx; g.ep[i].rx = mats[i]->rx; g.ep[i].s0 = sums[i]; g.ep[i].s2 = sums[i] + T; }
+        tiles = std::max<int64_t>(tiles, ((T + 127) / 128) * ((mats[i]->M + 127) / 128));
+    }
+    constexpr size_t lds = 2 * (size_t)(128 + 128) * BK * sizeof(h16);
+    const dim3 grid((unsigned)tiles, (unsigned)n);
+    if (w_u8) hipLaunchKernelGGL((gemm_group_kernel<true, 128, 128, 2, 2, 4>), grid, dim3(256), lds, st, (int)T, (int)N, g);
+    else hipLaunchKernelGGL((gemm_group_kernel<false, 128, 128, 2, 2, 4>), grid, dim3(256), lds, st, (int)T, (int)N, g);
+    RWKV_LAUNCH_CHECK();
+    return RWKV_OK;
+}
 
 extern "C" size_t rwkv_mm8_seq_workspace(int64_t B, int64_t N) {
     if (B <= 0 || N <= 0) return 0;

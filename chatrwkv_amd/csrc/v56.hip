@@ -124,8 +124,8 @@ __global__ __launch_bounds__(256) void v6_mix2_kernel(Mix2Args a) {
 struct Ws56 {
     rwkv_half *x, *xx, *sxd, *xxx, *t1, *mix[5], *d1, *d2, *r, *k, *v, *g, *att, *vx, *xs, *xx_att, *xx_ffn;
     float *sums, *splitk, *y32;
-    rwkv_half *xs_side[2];   // scaled-activation scratch of the products that run on side streams [T, C]
-    float *sums_side[2];
+    rwkv_half *xs_side[3];   // scaled-activation scratch of the products that run beside the first one [T, C]
+    float *sums_side[3];
     size_t total;
 };
 
@@ -142,8 +142,8 @@ Ws56 carve56(void *base, int64_t T, int64_t C, int64_t F, int64_t lm, int64_t ld
     w.vx = take(tf); w.xs = take(tf > tc ? tf : tc);
     w.xx_att = take((size_t)C * 2); w.xx_ffn = take((size_t)C * 2);
     w.sums = (float *)take((size_t)T * 2 * sizeof(float));
-    for (int j = 0; j < 2; ++j) {
-        w.xs_side[j] = take(T >= 256 ? tc : 256);
+    for (int j = 0; j < 3; ++j) {
+        w.xs_side[j] = take(T > 1 ? tc : 256);
         w.sums_side[j] = (float *)take((size_t)T * 2 * sizeof(float));
     }
     w.splitk = (float *)take(RWKV_SPLITK_WS_BYTES);
@@ -282,6 +282,24 @@ extern "C" int rwkv_v56_forward(const rwkv_v56_model *m, const rwkv_v56_layer_st
             if (fuse_d1) { a.xin = wx; a.xmat = l.td_w1; a.xm = ld; a.xout = ws.d1; }
             multi_vec_launch(u8, a, c.grid, st);
         } else {
+            // short calls: receptance, key, value (and gate) as one grouped launch at full depth, where each
+            // product alone would split K and need a reduction pass
+            if (!ss && ((T + 127) / 128) * (C / 128) <= 128 && !(C & 127)) {
+                const int n = gated ? 4 : 3;
+                const rwkv_half *xin[4] = {rx, kx, vx, gx};
+                const rwkv_mat *mats[4] = {&l.att_receptance, &l.att_key, &l.att_value, &l.att_gate};
+                void *outs[4] = {ws.r, ws.k, ws.v, ws.g};
+                rwkv_half *xsc[4] = {ws.xs, ws.xs_side[0], ws.xs_side[1], ws.xs_side[2]};
+                float *sm[4] = {ws.sums, ws.sums_side[0], ws.sums_side[1], ws.sums_side[2]};
+                GemmEpi ep[4];
+                for (int j = 0; j < 4; ++j) {
+                    ep[j] = GemmEpi{};
+                    ep[j].act = j == 3 ? ACT_SILU : ACT_NONE; ep[j].out_scale = 1.f; ep[j].out_dtype = RWKV_DT_F16;
+                    ep[j].ldres = C; ep[j].ldgate = C;
+                }
+                if ((rc = copy_h16_launch(C, ws.xx_att, s.att_xx, st))) return rc;
+                if ((rc = gemm_group_launch(u8, n, T, C, xin, mats, outs, ep, xsc, sm, st))) return rc;
+            } else {
             // receptance (then gate) on the caller's stream, key and value on the side streams
             const bool par = ss && fork_streams(ss, st, 2);
             Ctx cr = c;
@@ -291,6 +309,7 @@ extern "C" int rwkv_v56_forward(const rwkv_v56_model *m, const rwkv_v56_layer_st
             if ((rc = mm(par ? cs[1] : c, l.att_value, u8, vx, ACT_NONE, nullptr, nullptr, 1.f, ws.v))) return rc;
             if (gated && (rc = mm(c, l.att_gate, u8, gx, ACT_SILU, nullptr, nullptr, 1.f, ws.g))) return rc;
             if (par && !join_streams(ss, st, 2)) return (int)hipErrorUnknown;
+            }
         }
         // one token of v6: the second decay LoRA product is done inside the WKV kernel
         const bool d2_fused = v6 && T == 1;
@@ -322,7 +341,19 @@ extern "C" int rwkv_v56_forward(const rwkv_v56_model *m, const rwkv_v56_layer_st
             for (int j = 0; j < 2; ++j) { a.ry[j] = nullptr; a.my[j] = nullptr; a.xs[j] = ws.mix[j]; }
             if ((rc = lnmix_seq_launch(a, 2, st))) return rc;
         }
-        {
+        if (!ss && ((T + 127) / 128) * (C / 128) <= 128 && ((T + 127) / 128) * (F / 128) <= 256 && !(C & 127) && !(F & 127)) {
+            // short calls: receptance and key in one grouped launch at full depth
+            const rwkv_half *xin[2] = {ws.mix[0], ws.mix[1]};
+            const rwkv_mat *mats[2] = {&l.ffn_receptance, &l.ffn_key};
+            void *outs[2] = {ws.r, ws.vx};
+            rwkv_half *xsc[2] = {ws.xs, ws.xs_side[0]};
+            float *sm[2] = {ws.sums, ws.sums_side[0]};
+            GemmEpi ep[2] = {};
+            ep[0].act = ACT_SIGMOID; ep[1].act = ACT_RELU_SQ;
+            for (int j = 0; j < 2; ++j) { ep[j].out_scale = 1.f; ep[j].out_dtype = RWKV_DT_F16; }
+            if ((rc = copy_h16_launch(C, ws.xx_ffn, s.ffn_xx, st))) return rc;
+            if ((rc = gemm_group_launch(u8, 2, T, C, xin, mats, outs, ep, xsc, sm, st))) return rc;
+        } else {
             // channel-mix receptance beside the key product
             const bool par = ss && fork_streams(ss, st, 1);
             if (par && (rc = copy_h16_launch(C, ws.xx_ffn, s.ffn_xx, st))) return rc;
