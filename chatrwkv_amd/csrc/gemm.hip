@@ -33,26 +33,36 @@ constexpr int BK = 64;  // halves per LDS row
 DEV int swz(int row, int chunk) { return row * BK + ((chunk ^ ((row & 7) ^ ((row >> 3) & 1))) << 3); }
 
 // Epilogue of one output element: rank-1 corrections of the uint8 format, activation / residual, store.
-DEV void gemm_epilogue(float v, int t, int m, float rxm, float mxm, const GemmEpi &ep, void *Y, int64_t ldy) {
-    if (ep.rx) v = rxm * v + mxm * ep.s0[t] + ep.s2[t];
-    if (ep.raw_f32) {
-        ((float *)Y)[(size_t)t * ldy + m] = v;
-        return;
-    }
+// explicit fused multiply-adds: every kernel that ends in this epilogue rounds the same way
+DEV float epi_affine(float v, float rxm, float mxm, float s0, float s2) { return __builtin_fmaf(rxm, v, __builtin_fmaf(mxm, s0, s2)); }
+// v: the contraction after epi_affine; res / gate: the residual and gate inputs where ep.act uses them
+DEV float epi_act(float v, float res, float gate, const GemmEpi &ep) {
     float o = round_h(v);
     switch (ep.act) {
         case ACT_SIGMOID: o = sigmoidf_(o); break;
         case ACT_RELU_SQ: o = fmaxf(o, 0.f); o = o * o; break;
         case ACT_SILU: o = o * sigmoidf_(o); break;
         case ACT_TANH: o = tanhf(o); break;
-        case ACT_RESIDUAL: o = h2f(ep.res[(size_t)t * ep.ldres + m]) + o; break;
+        case ACT_RESIDUAL: o = res + o; break;
         case ACT_GATED_RESIDUAL:
-            o = round_h(h2f(ep.gate[(size_t)t * ep.ldgate + m]) * o);
-            o = h2f(ep.res[(size_t)t * ep.ldres + m]) + o;
+            o = round_h(gate * o);
+            o = res + o;
             break;
         default: break;
     }
     if (ep.out_scale != 1.f) o = round_h(o) * ep.out_scale;
+    return o;
+}
+DEV void gemm_epilogue(float v, int t, int m, float rxm, float mxm, const GemmEpi &ep, void *Y, int64_t ldy) {
+    if (ep.rx) v = epi_affine(v, rxm, mxm, ep.s0[t], ep.s2[t]);
+    if (ep.raw_f32) {
+        ((float *)Y)[(size_t)t * ldy + m] = v;
+        return;
+    }
+    float res = 0.f, gate = 0.f;
+    if (ep.act == ACT_RESIDUAL || ep.act == ACT_GATED_RESIDUAL) res = h2f(ep.res[(size_t)t * ep.ldres + m]);
+    if (ep.act == ACT_GATED_RESIDUAL) gate = h2f(ep.gate[(size_t)t * ep.ldgate + m]);
+    const float o = epi_act(v, res, gate, ep);
     if (ep.out_dtype == RWKV_DT_F32)
         ((float *)Y)[(size_t)t * ldy + m] = round_h(o);
     else
@@ -250,6 +260,225 @@ __global__ __launch_bounds__(64 * WT * WM) void gemm_kernel(int T, int N, int M,
     gemm_body<W_U8, BT, BM, WT, WM, PF, SPLIT>(T, N, M, A, lda, Wv, ldw, Y, ldy, ep, nk_split, part);
 }
 
+// ---- uint8 weights, large products: operands go from global memory straight into LDS ------------------------
+// 256 x 256 tile, 8 waves (2 x 4, each 128 x 64), three LDS stages of one 64-deep k-tile each.  The loads are
+// global_load_lds_dwordx4: one wave instruction copies 64 x 16 B into 1 KB of LDS without passing through
+// registers, so no wave spends issue slots on ds_write or on holding prefetched tiles.  The weight tile stays
+// uint8 in LDS (half the bytes of fp16) and becomes fp16 in the B fragments on the way to the matrix cores.
+// LDS layout of a stage: A tile [256 rows][8 chunks of 16 B], chunk c of row r at slot c ^ ((r >> 1) & 7);
+// W tile [256 rows][4 chunks of 16 B], chunk c of row r at slot c ^ ((r >> 2) & 3): both make the fragment reads
+// (32 rows x one chunk per half-wave) hit every bank once.  The swizzle is applied on the global side: the lane
+// that fills slot p of row r loads chunk p ^ key(r).
+// Schedule of one k-tile: fragments of step ks + 1 are read while step ks multiplies (registers double-buffered);
+// after the third of four steps every wave waits for its own loads of the next tile and meets the others at the
+// one barrier, then issues the loads of tile kt + 3 into the stage it has just finished and reads the first
+// fragments of tile kt + 1 while the fourth step multiplies.  LDS reads are inline asm with hand-placed
+// s_waitcnt: the compiler waits for lgkmcnt(0) wherever older and newer reads are both outstanding.
+constexpr int DT = 256, DM = 256, D_A = DT * BK * 2, D_W = DM * BK, D_STAGE = D_A + D_W, D_NST = 3;
+
+template <bool SPLIT>
+DEV void gemm_dma_body(int T, int N, int M, const h16 *__restrict__ A, int64_t lda, const uint8_t *__restrict__ W, int64_t ldw,
+                       void *__restrict__ Y, int64_t ldy, const GemmEpi &ep, int nk_split, float *__restrict__ part) {
+    extern __shared__ __align__(1024) unsigned char smem[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wr = wave >> 2, wc = wave & 3;
+    const int tiles_t = (T + DT - 1) / DT;
+    int bid = blockIdx.x;
+    if ((gridDim.x & 7) == 0) bid = (bid & 7) * (gridDim.x >> 3) + (bid >> 3);
+    const int t0 = (bid % tiles_t) * DT, m0 = (bid / tiles_t) * DM;
+    if (m0 >= M) return;   // grouped launches size the grid for their widest member
+    const int kbase = SPLIT ? blockIdx.y * nk_split : 0, nk = SPLIT ? nk_split : N / BK;
+
+    // load sources; rows past the end re-read the last row (never stored)
+    const h16 *ga[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int r = (wave * 4 + i) * 8 + (lane >> 3), c = (lane & 7) ^ ((r >> 1) & 7);
+        ga[i] = A + (size_t)min(t0 + r, T - 1) * lda + (size_t)kbase * BK + c * 8;
+    }
+    const uint8_t *gw[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int r = (wave * 2 + i) * 16 + (lane >> 2), c = (lane & 3) ^ ((r >> 2) & 3);
+        gw[i] = W + (size_t)min(m0 + r, M - 1) * ldw + (size_t)kbase * BK + c * 16;
+    }
+    typedef __attribute__((address_space(1))) const void *gptr;
+    typedef __attribute__((address_space(3))) void *lptr;
+    auto issue = [&](int kt, int so) {
+        unsigned char *base = smem + so;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            __builtin_amdgcn_global_load_lds((gptr)(ga[i] + kt * BK), (lptr)(base + (wave * 4 + i) * 1024), 16, 0, 0);
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+            __builtin_amdgcn_global_load_lds((gptr)(gw[i] + kt * BK), (lptr)(base + D_A + (wave * 2 + i) * 1024), 16, 0, 0);
+    };
+
+    f32x16 acc[4][2];
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[a][b][e] = 0.f;
+
+    // fragment addresses within a stage; the swizzle keys depend on the lane only
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem;
+    uint32_t vA[4], vB[4];
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+        vA[ks] = lds0 + (wr * 128 + (lane & 31)) * 128 + (((2 * ks + (lane >> 5)) ^ ((lane >> 1) & 7)) << 4);
+        vB[ks] = lds0 + D_A + (wc * 64 + (lane & 31)) * 64 + ((ks ^ ((lane >> 2) & 3)) << 4) + (lane >> 5) * 8;
+    }
+    h16x8 fa[2][4];
+    u32x2 rawb[2][2];
+    auto ldfrag = [&](int buf, int so, int ks) {
+        const uint32_t pa = vA[ks] + so, pb = vB[ks] + so;
+        asm volatile("ds_read_b64 %0, %1" : "=v"(rawb[buf][0]) : "v"(pb));
+        asm volatile("ds_read_b64 %0, %1 offset:2048" : "=v"(rawb[buf][1]) : "v"(pb));
+        asm volatile("ds_read_b128 %0, %1" : "=v"(fa[buf][0]) : "v"(pa));
+        asm volatile("ds_read_b128 %0, %1 offset:4096" : "=v"(fa[buf][1]) : "v"(pa));
+        asm volatile("ds_read_b128 %0, %1 offset:8192" : "=v"(fa[buf][2]) : "v"(pa));
+        asm volatile("ds_read_b128 %0, %1 offset:12288" : "=v"(fa[buf][3]) : "v"(pa));
+    };
+    const h16x2 off = {(h16)1023.5f, (h16)1023.5f};
+    // waits until at most `newer` of this wave's LDS reads are outstanding, i.e. the six before them have returned
+    auto older_reads_done = [&](int newer) {
+        if (newer) __builtin_amdgcn_s_waitcnt(0xC67F); else __builtin_amdgcn_s_waitcnt(0xC07F);   // lgkmcnt(6) / lgkmcnt(0)
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    auto multiply = [&](int cur) {
+        h16x8 fb[2];
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+            const u32x2 raw = rawb[cur][b];
+            const h16x2 q0 = u8pair_lo_1024(raw.x) - off, q1 = u8pair_hi_1024(raw.x) - off;
+            const h16x2 q2 = u8pair_lo_1024(raw.y) - off, q3 = u8pair_hi_1024(raw.y) - off;
+            fb[b] = h16x8{q0.x, q0.y, q1.x, q1.y, q2.x, q2.y, q3.x, q3.y};
+        }
+#pragma unroll
+        for (int a = 0; a < 4; ++a)
+#pragma unroll
+            for (int b = 0; b < 2; ++b) acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[cur][a], fb[b], acc[a][b], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+
+    // Every wave issues exactly six loads per tile, so "vmcnt(6 n)" means "all but my newest n tiles have landed".
+    // Past the last tile the loads repeat it into a stage nobody reads any more, which keeps the counts static.
+    issue(0, 0);
+    issue(min(1, nk - 1), D_STAGE);
+    issue(min(2, nk - 1), 2 * D_STAGE);
+    __builtin_amdgcn_s_waitcnt(0x0F7C);   // vmcnt(12): tile 0 has landed
+    __builtin_amdgcn_s_barrier();
+    ldfrag(0, 0, 0);
+    int so = 0;
+    for (int kt = 0; kt < nk; ++kt) {
+        const int sn = so + D_STAGE >= D_NST * D_STAGE ? 0 : so + D_STAGE;
+        ldfrag(1, so, 1);
+        __builtin_amdgcn_sched_barrier(0);
+        older_reads_done(6);
+        multiply(0);
+        ldfrag(0, so, 2);
+        __builtin_amdgcn_sched_barrier(0);
+        older_reads_done(6);
+        multiply(1);
+        ldfrag(1, so, 3);
+        __builtin_amdgcn_sched_barrier(0);
+        older_reads_done(6);
+        multiply(0);
+        // all my reads of this stage have returned and my part of tile kt + 1 has landed (tile kt + 2 may be in flight)
+        __builtin_amdgcn_s_waitcnt(0x0076);   // vmcnt(6) lgkmcnt(0)
+        __builtin_amdgcn_s_barrier();
+        issue(min(kt + 3, nk - 1), so);
+        ldfrag(0, sn, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(1);
+        so = sn;
+    }
+    __builtin_amdgcn_s_waitcnt(0x0070);   // vmcnt(0) lgkmcnt(0): nothing may land in LDS after the workgroup has gone
+
+    if constexpr (SPLIT) {
+        float *slab = part + (size_t)blockIdx.y * T * M;
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+            const int m = m0 + wc * 64 + b * 32 + (lane & 31);
+#pragma unroll
+            for (int a = 0; a < 4; ++a)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    const int t = t0 + wr * 128 + a * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
+                    if (m < M && t < T) slab[(size_t)t * M + m] = acc[a][b][e];
+                }
+        }
+        return;
+    } else {
+        // The accumulators pass through LDS (free now), 128 rows at a time, so that each thread finishes eight
+        // consecutive outputs of one row: 16-byte loads of the residual / gate rows, 16-byte stores, and a body
+        // small enough to stay in the instruction cache (per-element code for 128 accumulators does not).
+        constexpr int SW = 264;   // row stride in floats: 4 rows apart = 32 banks apart for the two half-waves
+        float *stg = (float *)smem;
+        const int cq = tid & 31, col = m0 + cq * 8;
+        const bool col_ok = col < M;   // M % 8 == 0
+        h16x8 rx8, mx8;
+        if (col_ok) { rx8 = *(const h16x8 *)(ep.rx + col); mx8 = *(const h16x8 *)(ep.mx + col); }
+        __syncthreads();   // every wave has read its last fragments
+#pragma unroll 1
+        for (int h = 0; h < 2; ++h) {
+            if (wr == h) {
+#pragma unroll
+                for (int b = 0; b < 2; ++b)
+#pragma unroll
+                    for (int a = 0; a < 4; ++a)
+#pragma unroll
+                        for (int e = 0; e < 16; ++e)
+                            stg[(a * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3)) * SW + wc * 64 + b * 32 + (lane & 31)] = acc[a][b][e];
+            }
+            __syncthreads();
+#pragma unroll 1
+            for (int it = 0; it < 8; ++it) {
+                const int row = it * 16 + (tid >> 5), t = t0 + h * 128 + row;
+                if (t < T && col_ok) {
+                    const f32x4 v0 = *(const f32x4 *)(stg + row * SW + cq * 8), v1 = *(const f32x4 *)(stg + row * SW + cq * 8 + 4);
+                    const float s0t = ep.s0[t], s2t = ep.s2[t];
+                    float v[8];
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) v[e] = epi_affine(e < 4 ? v0[e & 3] : v1[e & 3], (float)rx8[e], (float)mx8[e], s0t, s2t);
+                    if (ep.raw_f32) {
+                        float *yo = (float *)Y + (size_t)t * ldy + col;
+                        *(f32x4 *)yo = f32x4{v[0], v[1], v[2], v[3]};
+                        *(f32x4 *)(yo + 4) = f32x4{v[4], v[5], v[6], v[7]};
+                    } else {
+                        h16x8 res8 = {}, gate8 = {};
+                        if (ep.act == ACT_RESIDUAL || ep.act == ACT_GATED_RESIDUAL) res8 = *(const h16x8 *)(ep.res + (size_t)t * ep.ldres + col);
+                        if (ep.act == ACT_GATED_RESIDUAL) gate8 = *(const h16x8 *)(ep.gate + (size_t)t * ep.ldgate + col);
+                        float o[8];
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) o[e] = epi_act(v[e], (float)res8[e], (float)gate8[e], ep);
+                        if (ep.out_dtype == RWKV_DT_F32) {
+                            float *yo = (float *)Y + (size_t)t * ldy + col;
+                            *(f32x4 *)yo = f32x4{round_h(o[0]), round_h(o[1]), round_h(o[2]), round_h(o[3])};
+                            *(f32x4 *)(yo + 4) = f32x4{round_h(o[4]), round_h(o[5]), round_h(o[6]), round_h(o[7])};
+                        } else {
+                            h16x8 y8;
+#pragma unroll
+                            for (int e = 0; e < 8; ++e) y8[e] = (h16)o[e];
+                            *(h16x8 *)((rwkv_half *)Y + (size_t)t * ldy + col) = y8;
+                        }
+                    }
+                }
+            }
+            __syncthreads();
+        }
+    }
+}
+
+template <bool SPLIT>
+__global__ __launch_bounds__(512) void gemm_dma_kernel(int T, int N, int M, const h16 *__restrict__ A, int64_t lda,
+                                                       const uint8_t *__restrict__ W, int64_t ldw, void *__restrict__ Y,
+                                                       int64_t ldy, GemmEpi ep, int nk_split, float *__restrict__ part) {
+    gemm_dma_body<SPLIT>(T, N, M, A, lda, W, ldw, Y, ldy, ep, nk_split, part);
+}
+
 // Up to four contractions [T, N] x [N, M_i] in one launch (blockIdx.y picks the operands), at full depth: short
 // calls, where each of them alone would split K and need a reduction pass.
 struct GemmGroup {
@@ -266,6 +495,12 @@ __global__ __launch_bounds__(64 * WT * WM) void gemm_group_kernel(int T, int N, 
     const int gi = blockIdx.y, M = g.M[gi];
     gemm_body<W_U8, BT, BM, WT, WM, PF, false>(T, N, M, g.A[gi], g.lda, g.W[gi], g.ldw[gi], g.Y[gi], M, g.ep[gi], N / BK,
                                                nullptr);
+}
+
+// the same through the direct-to-LDS kernel (uint8 weights, long calls)
+__global__ __launch_bounds__(512) void gemm_dma_group_kernel(int T, int N, GemmGroup g) {
+    const int gi = blockIdx.y, M = g.M[gi];
+    gemm_dma_body<false>(T, N, M, g.A[gi], g.lda, (const uint8_t *)g.W[gi], g.ldw[gi], g.Y[gi], M, g.ep[gi], N / BK, nullptr);
 }
 
 struct PrepGroup {
@@ -376,6 +611,56 @@ int launch_cfg(int64_t T, int64_t N, int64_t M, const rwkv_half *A, int64_t lda,
     return RWKV_OK;
 }
 
+// what gemm_dma_kernel assumes: whole k-tiles, 16-byte rows and row starts for its loads and its eight-wide epilogue
+bool dma_ok(int64_t N, int64_t M, const void *A, int64_t lda, const void *W, int64_t ldw, const void *Y, int64_t ldy, const GemmEpi &ep) {
+    auto a16 = [](const void *p) { return (((uintptr_t)p) & 15) == 0; };
+    if (!ep.rx || !ep.mx || !ep.s0 || !ep.s2 || (N % BK) || (M & 7) || (lda & 7) || (ldw & 15) || (ldy & 7)) return false;
+    if (!a16(A) || !a16(W) || !a16(Y) || !a16(ep.rx) || !a16(ep.mx)) return false;
+    if (ep.act == ACT_RESIDUAL || ep.act == ACT_GATED_RESIDUAL)
+        if (!ep.res || !a16(ep.res) || (ep.ldres & 7)) return false;
+    if (ep.act == ACT_GATED_RESIDUAL)
+        if (!ep.gate || !a16(ep.gate) || (ep.ldgate & 7)) return false;
+    return true;
+}
+
+// uint8 weights through gemm_dma_kernel.  Fewer than 192 tiles (narrow outputs): the contraction is split over
+// workgroups of the same tile until about one workgroup per CU is in flight; slabs and the second pass as in launch_cfg.
+int launch_dma(int64_t T, int64_t N, int64_t M, const rwkv_half *A, int64_t lda, const void *W, int64_t ldw, void *Y,
+               int64_t ldy, const GemmEpi &ep, hipStream_t st) {
+    constexpr size_t lds = (size_t)D_NST * D_STAGE;
+    static bool attr_done = false;
+    if (!attr_done) {
+        hipError_t e = hipFuncSetAttribute((const void *)gemm_dma_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e == hipSuccess)
+            e = hipFuncSetAttribute((const void *)gemm_dma_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return (int)e;
+        attr_done = true;
+    }
+    if (!dma_ok(N, M, A, lda, W, ldw, Y, ldy, ep)) return RWKV_E_LAYOUT;
+    const int64_t tiles = ((T + DT - 1) / DT) * ((M + DM - 1) / DM);
+    const int nk = (int)(N / BK);
+    int ks = 1;
+    if (ep.splitk_ws && tiles < 192 && (M & 3) == 0)
+        for (int c = 2; c <= 8; c <<= 1) {
+            if (nk % c || nk / c < 8) break;
+            if ((size_t)c * T * M * sizeof(float) > ep.splitk_bytes) break;
+            ks = c;
+            if (tiles * c >= 192) break;
+        }
+    if (ks > 1) {
+        hipLaunchKernelGGL(gemm_dma_kernel<true>, dim3((unsigned)tiles, (unsigned)ks), dim3(512), lds, st, (int)T, (int)N, (int)M,
+                           (const h16 *)A, lda, (const uint8_t *)W, ldw, Y, ldy, ep, nk / ks, ep.splitk_ws);
+        const int64_t n = T * M;
+        const unsigned blocks = (unsigned)((n + 1023) / 1024 < 16384 ? (n + 1023) / 1024 : 16384);
+        hipLaunchKernelGGL(splitk_epilogue_kernel, dim3(blocks), dim3(256), 0, st, (int)T, (int)M, ks, ep.splitk_ws, Y, ldy, ep);
+    } else {
+        hipLaunchKernelGGL(gemm_dma_kernel<false>, dim3((unsigned)tiles), dim3(512), lds, st, (int)T, (int)N, (int)M, (const h16 *)A,
+                           lda, (const uint8_t *)W, ldw, Y, ldy, ep, nk, (float *)nullptr);
+    }
+    RWKV_LAUNCH_CHECK();
+    return RWKV_OK;
+}
+
 template <bool W_U8>
 int launch_pick(int cfg, int64_t T, int64_t N, int64_t M, const rwkv_half *A, int64_t lda, const void *W, int64_t ldw,
                 void *Y, int64_t ldy, const GemmEpi &ep, hipStream_t st) {
@@ -384,29 +669,34 @@ int launch_pick(int cfg, int64_t T, int64_t N, int64_t M, const rwkv_half *A, in
         case 9:
             if constexpr (W_U8) return launch_cfg<true, 256, 256, 4, 4, 2>(T, N, M, A, lda, W, ldw, Y, ldy, ep, st);
             return RWKV_E_DTYPE;
+        case 14:
+            if constexpr (W_U8) return launch_dma(T, N, M, A, lda, W, ldw, Y, ldy, ep, st);
+            return RWKV_E_DTYPE;
         default: return RWKV_E_DTYPE;
     }
 }
 
 // Tile choice (RWKV_GEMM_CFG overrides it for tuning sweeps).
-int pick_cfg(int64_t T, int64_t M) {
+//   14  uint8 weights, 512 rows or more and an output of 3 M elements or more, operands laid out for 16-byte loads:
+//       the direct-to-LDS kernel (256 x 256 tiles; it splits K itself when there are few tiles)
+//    9  uint8 weights otherwise, where 256 x 256 tiles of the register-staged kernel fill the chip: one per CU and
+//       round, the last round at least 70 % full
+//    3  everything else: 128 x 128 tiles, 4 k-tiles of prefetch
+int pick_cfg(int64_t T, int64_t M, bool w_u8, bool alone, bool dma) {
     const char *e = getenv("RWKV_GEMM_CFG");  // tuning override
     if (e && *e) return atoi(e);
-    // The kernel is bound by how fast a CU's L1 can be filled, and a 256 x 256 tile (16 waves) fetches half the
-    // operand bytes per flop of a 128 x 128 one: +30 % on [1024 x 4096] x [4096 x 16384].  Only where such tiles
-    // fill the chip: one per CU and round, the last round at least 70 % full.
+    if (!w_u8 || !alone) return 3;   // fp16 weight tiles are twice the bytes; a 256 x 256 tile's LDS leaves no room beside it
     const int64_t big = ((T + 255) / 256) * ((M + 255) / 256), rounds = (big + 255) / 256;
-    if (big * 10 >= rounds * 256 * 7) return 9;
-    return 3;  // 128 x 128 tile, 4 k-tiles of prefetch
+    const bool fills = big * 10 >= rounds * 256 * 7;
+    if (dma && T >= 512 && T * M >= ((int64_t)3 << 20) && (big < 192 || fills)) return 14;
+    return fills ? 9 : 3;
 }
 
 }  // namespace
 
 int gemm_launch(bool w_u8, int64_t T, int64_t N, int64_t M, const rwkv_half *A, int64_t lda, const void *W,
                 int64_t ldw, void *Y, int64_t ldy, const GemmEpi &ep, hipStream_t st) {
-    int cfg = pick_cfg(T, M);
-    // the large tile pays with uint8 weights only: fp16 weight tiles are twice the bytes and its registers spill
-    if ((ep.small_tiles || !w_u8) && cfg == 9) cfg = 3;
+    const int cfg = pick_cfg(T, M, w_u8, !ep.small_tiles, w_u8 && dma_ok(N, M, A, lda, W, ldw, Y, ldy, ep));
     return w_u8 ? launch_pick<true>(cfg, T, N, M, A, lda, W, ldw, Y, ldy, ep, st)
                 : launch_pick<false>(cfg, T, N, M, A, lda, W, ldw, Y, ldy, ep, st);
 }
@@ -421,28 +711,46 @@ int mm8_prepare_launch(int64_t T, int64_t N, const rwkv_half *x, int64_t ldx, co
 
 
 // n (2..4) products [T, N] x [N, M_i] of uint8 or fp16 weights with their own inputs, outputs and epilogues in one
-// launch.  uint8: x[i] is the unscaled activation, xs[i] / sums[i] (2 T floats) are scratch.
+// launch.  uint8 with xs != NULL: x[i] is the unscaled activation and xs[i] / sums[i] (2 T floats) are scratch;
+// uint8 with xs == NULL: x[i] is already scaled by ry and sums[i] holds its row sums.
+// Calls of 512 rows or more with uint8 weights go through the direct-to-LDS kernel, others through 128 x 128 tiles.
 int gemm_group_launch(bool w_u8, int n, int64_t T, int64_t N, const rwkv_half *const *x, const rwkv_mat *const *mats,
                       void *const *Y, const GemmEpi *eps, rwkv_half *const *xs, float *const *sums, hipStream_t st) {
     if (n < 2 || n > 4 || (N % BK)) return RWKV_E_SHAPE;
     GemmGroup g{};
     g.lda = N;
-    if (w_u8) {
+    const bool prep = w_u8 && xs;
+    if (prep) {
         PrepGroup p{};
         for (int i = 0; i < n; ++i) {
             p.x[i] = x[i]; p.ry[i] = mats[i]->ry; p.my[i] = mats[i]->my; p.xs[i] = xs[i]; p.s0[i] = sums[i]; p.s2[i] = sums[i] + T;
         }
         hipLaunchKernelGGL(mm8_prepare_group_kernel, dim3((unsigned)((T + 3) / 4), (unsigned)n), dim3(256), 0, st, (int)T, (int)N, p);
     }
-    int64_t tiles = 0;
+    int64_t tiles = 0, tiles_dma = 0;
+    bool dma = w_u8 && T >= 512;
     for (int i = 0; i < n; ++i) {
         if (mats[i]->N != N) return RWKV_E_SHAPE;
-        g.A[i] = (const h16 *)(w_u8 ? xs[i] : x[i]);
+        g.A[i] = (const h16 *)(prep ? xs[i] : x[i]);
         g.W[i] = mats[i]->w; g.ldw[i] = mats[i]->ld; g.Y[i] = Y[i]; g.M[i] = (int)mats[i]->M;
         g.ep[i] = eps[i];
         g.ep[i].ldres = g.ep[i].ldgate = mats[i]->M;
         if (w_u8) { g.ep[i].mx = mats[i]->mx; g.ep[i].rx = mats[i]->rx; g.ep[i].s0 = sums[i]; g.ep[i].s2 = sums[i] + T; }
         tiles = std::max<int64_t>(tiles, ((T + 127) / 128) * ((mats[i]->M + 127) / 128));
+        tiles_dma = std::max<int64_t>(tiles_dma, ((T + DT - 1) / DT) * ((mats[i]->M + DM - 1) / DM));
+        dma = dma && dma_ok(N, mats[i]->M, g.A[i], N, g.W[i], g.ldw[i], g.Y[i], mats[i]->M, g.ep[i]);
+    }
+    if (dma) {
+        constexpr size_t lds = (size_t)D_NST * D_STAGE;
+        static bool attr_done = false;
+        if (!attr_done) {
+            hipError_t e = hipFuncSetAttribute((const void *)gemm_dma_group_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            if (e != hipSuccess) return (int)e;
+            attr_done = true;
+        }
+        hipLaunchKernelGGL(gemm_dma_group_kernel, dim3((unsigned)tiles_dma, (unsigned)n), dim3(512), lds, st, (int)T, (int)N, g);
+        RWKV_LAUNCH_CHECK();
+        return RWKV_OK;
     }
     constexpr size_t lds = 2 * (size_t)(128 + 128) * BK * sizeof(h16);
     const dim3 grid((unsigned)tiles, (unsigned)n);

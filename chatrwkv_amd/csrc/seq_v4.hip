@@ -3,6 +3,7 @@
 //   -> WKV-4 over T (r gating fused) -> prepare -> GEMM Wo (+ residual)
 //   lnmix_seq (LN2, ...) -> GEMM Wr (sigmoid), GEMM Wk (relu^2) -> prepare -> GEMM Wv (gate, residual, /2)
 // and LN_out + head on the last row (GEMV) or on every row (GEMM) for full_output.
+#include <cstdlib>
 #include "kernels.h"
 
 namespace {
@@ -301,7 +302,18 @@ extern "C" int rwkv_v4_forward_seq(const rwkv_v4_model *m, const rwkv_v4_layer_s
         // k, v: uint8 weights return fp16 (widened by the consumer); fp16 weights return fp32 directly
         e.act = ACT_NONE; e.out_dtype = u8 ? RWKV_DT_F16 : RWKV_DT_F32; e.raw_f32 = u8 ? 0 : 1;
         // side by side when none of them would split K (the split-K scratch is shared)
-        const bool par = ss && (T / 128) * (C / 128) > 128 && fork_streams(ss, st, 2);
+        // long calls with uint8 weights: every product through the direct-to-LDS kernel, one after the other (its
+        // tiles take a whole CU, so products side by side on several streams gain nothing); k, v, r as one group
+        const bool dma_seq = u8 && T >= 512;
+        const bool par = ss && !dma_seq && (T / 128) * (C / 128) > 128 && fork_streams(ss, st, 2);
+        if (dma_seq) {
+            const rwkv_half *xin[3] = {ws.xs[0], ws.xs[1], ws.xs[2]};
+            const rwkv_mat *mats[3] = {&l.att_key, &l.att_value, &l.att_receptance};
+            void *outs[3] = {ws.k, ws.v, ws.r};
+            GemmEpi ep[3] = {e, e, e};
+            ep[2].act = ACT_SIGMOID; ep[2].out_dtype = RWKV_DT_F16; ep[2].raw_f32 = 0;
+            if ((rc = gemm_group_launch(true, 3, T, C, xin, mats, outs, ep, nullptr, s0, st))) return rc;
+        } else {
         hipStream_t sv = par ? ss->s[0] : st, sr = par ? ss->s[1] : st;
         float *sk = par ? nullptr : ws.splitk;   // products that run side by side do not split K
         if ((rc = run_gemm(l.att_key, u8, T, ws.xs[0], s0[0], s2[0], ws.k, C, e, st, sk))) return rc;
@@ -309,6 +321,7 @@ extern "C" int rwkv_v4_forward_seq(const rwkv_v4_model *m, const rwkv_v4_layer_s
         e.act = ACT_SIGMOID; e.out_dtype = RWKV_DT_F16; e.raw_f32 = 0;
         if ((rc = run_gemm(l.att_receptance, u8, T, ws.xs[2], s0[2], s2[2], ws.r, C, e, sr, sk))) return rc;
         if (par && !join_streams(ss, st, 2)) return (int)hipErrorUnknown;
+        }
         if ((rc = wkv4_fused_launch((int)T, C, l.time_decay, l.time_first, ws.k, ws.v, u8 ? 0 : 1, ws.r, ws.rwkv, s.aa,
                                     s.bb, s.pp, st, ws.wkv)))
             return rc;
@@ -338,7 +351,7 @@ extern "C" int rwkv_v4_forward_seq(const rwkv_v4_model *m, const rwkv_v4_layer_s
         e = GemmEpi{};
         e.out_scale = 1.f; e.out_dtype = RWKV_DT_F16;
         e.act = ACT_SIGMOID;
-        const bool par2 = ss && (T / 128) * (C / 128) > 128 && fork_streams(ss, st, 1);
+        const bool par2 = ss && !dma_seq && (T / 128) * (C / 128) > 128 && fork_streams(ss, st, 1);
         float *sk2 = par2 ? nullptr : ws.splitk;
         if ((rc = run_gemm(l.ffn_receptance, u8, T, ws.xs[0], s0[0], s2[0], ws.r, C, e, par2 ? ss->s[0] : st, sk2))) return rc;
         e.act = ACT_RELU_SQ;

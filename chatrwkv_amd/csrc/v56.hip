@@ -233,6 +233,9 @@ extern "C" int rwkv_v56_forward(const rwkv_v56_model *m, const rwkv_v56_layer_st
         const rwkv_v56_layer &l = m->layers[i];
         const rwkv_v56_layer_state &s = states[i];
         const bool u8 = mat_is_u8(m->weights_u8, l.att_key);
+        // long calls with uint8 weights: every product through the direct-to-LDS kernel, one after the other (its
+        // tiles take a whole CU, so products side by side on several streams gain nothing)
+        const bool dma_seq = u8 && T >= 512;
         const rwkv_half *kx, *vx, *rx, *gx = nullptr, *wx = nullptr;
         bool fuse_d1 = false;
         if (v6) {
@@ -282,9 +285,10 @@ extern "C" int rwkv_v56_forward(const rwkv_v56_model *m, const rwkv_v56_layer_st
             if (fuse_d1) { a.xin = wx; a.xmat = l.td_w1; a.xm = ld; a.xout = ws.d1; }
             multi_vec_launch(u8, a, c.grid, st);
         } else {
-            // short calls: receptance, key, value (and gate) as one grouped launch at full depth, where each
-            // product alone would split K and need a reduction pass
-            if (!ss && ((T + 127) / 128) * (C / 128) <= 128 && !(C & 127)) {
+            // One grouped launch at full depth for receptance, key, value (and gate): in short calls, where each
+            // product alone would split K and need a reduction pass, and in long calls with uint8 weights, where
+            // the group fills the chip with the 256 x 256 tiles of the direct-to-LDS kernel.
+            if ((dma_seq || (!ss && ((T + 127) / 128) * (C / 128) <= 128)) && !(C & 127)) {
                 const int n = gated ? 4 : 3;
                 const rwkv_half *xin[4] = {rx, kx, vx, gx};
                 const rwkv_mat *mats[4] = {&l.att_receptance, &l.att_key, &l.att_value, &l.att_gate};
@@ -301,7 +305,7 @@ extern "C" int rwkv_v56_forward(const rwkv_v56_model *m, const rwkv_v56_layer_st
                 if ((rc = gemm_group_launch(u8, n, T, C, xin, mats, outs, ep, xsc, sm, st))) return rc;
             } else {
             // receptance (then gate) on the caller's stream, key and value on the side streams
-            const bool par = ss && fork_streams(ss, st, 2);
+            const bool par = ss && !dma_seq && fork_streams(ss, st, 2);
             Ctx cr = c;
             if (par) cr.splitk = nullptr;
             if ((rc = mm(cr, l.att_receptance, u8, rx, ACT_NONE, nullptr, nullptr, 1.f, ws.r, ws.xx_att, s.att_xx, C))) return rc;
@@ -355,7 +359,7 @@ extern "C" int rwkv_v56_forward(const rwkv_v56_model *m, const rwkv_v56_layer_st
             if ((rc = gemm_group_launch(u8, 2, T, C, xin, mats, outs, ep, xsc, sm, st))) return rc;
         } else {
             // channel-mix receptance beside the key product
-            const bool par = ss && fork_streams(ss, st, 1);
+            const bool par = ss && !dma_seq && fork_streams(ss, st, 1);
             if (par && (rc = copy_h16_launch(C, ws.xx_ffn, s.ffn_xx, st))) return rc;
             if (par) {
                 if ((rc = mm(cs[0], l.ffn_receptance, u8, ws.mix[0], ACT_SIGMOID, nullptr, nullptr, 1.f, ws.r))) return rc;
