@@ -274,11 +274,23 @@ __global__ __launch_bounds__(64 * WT * WM) void gemm_kernel(int T, int N, int M,
 // one barrier, then issues the loads of tile kt + 3 into the stage it has just finished and reads the first
 // fragments of tile kt + 1 while the fourth step multiplies.  LDS reads are inline asm with hand-placed
 // s_waitcnt: the compiler waits for lgkmcnt(0) wherever older and newer reads are both outstanding.
-constexpr int DT = 256, DM = 256, D_A = DT * BK * 2, D_W = DM * BK, D_STAGE = D_A + D_W, D_NST = 3;
+// fp16 weights (W_U8 = false): the weight tile is laid out like the A tile (32 KB), a stage is 64 KB and two fit, so
+// one tile is in flight while one multiplies.
+constexpr int DT = 256, DM = 256, D_A = DT * BK * 2;
+template <bool W_U8> struct DmaCfg {
+    static constexpr int W = W_U8 ? DM * BK : DM * BK * 2, STAGE = D_A + W, NST = W_U8 ? 3 : 2, LOADS = 4 + W / 8192;
+    static constexpr int STG_STRIDE = 264;   // epilogue staging: 128 rows of 256 floats, padded (see the epilogue)
+    static constexpr size_t LDS = (size_t)NST * STAGE > (size_t)128 * STG_STRIDE * 4 ? (size_t)NST * STAGE : (size_t)128 * STG_STRIDE * 4;
+};
+// s_waitcnt immediates: vmcnt(n) alone, and vmcnt(n) with lgkmcnt(0)
+constexpr int vm_only(int n) { return 0x0F70 | (n & 15) | ((n >> 4) << 14); }
+constexpr int vm_lgkm0(int n) { return 0x0070 | (n & 15) | ((n >> 4) << 14); }
 
-template <bool SPLIT>
-DEV void gemm_dma_body(int T, int N, int M, const h16 *__restrict__ A, int64_t lda, const uint8_t *__restrict__ W, int64_t ldw,
+template <bool W_U8, bool SPLIT>
+DEV void gemm_dma_body(int T, int N, int M, const h16 *__restrict__ A, int64_t lda, const void *__restrict__ Wv, int64_t ldw,
                        void *__restrict__ Y, int64_t ldy, const GemmEpi &ep, int nk_split, float *__restrict__ part) {
+    using Cfg = DmaCfg<W_U8>;
+    constexpr int D_STAGE = Cfg::STAGE, D_NST = Cfg::NST, WL = Cfg::W / 8192;   // WL: weight loads per wave and tile
     extern __shared__ __align__(1024) unsigned char smem[];
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wr = wave >> 2, wc = wave & 3;
@@ -296,11 +308,16 @@ DEV void gemm_dma_body(int T, int N, int M, const h16 *__restrict__ A, int64_t l
         const int r = (wave * 4 + i) * 8 + (lane >> 3), c = (lane & 7) ^ ((r >> 1) & 7);
         ga[i] = A + (size_t)min(t0 + r, T - 1) * lda + (size_t)kbase * BK + c * 8;
     }
-    const uint8_t *gw[2];
+    const unsigned char *gw[WL];   // byte pointers
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-        const int r = (wave * 2 + i) * 16 + (lane >> 2), c = (lane & 3) ^ ((r >> 2) & 3);
-        gw[i] = W + (size_t)min(m0 + r, M - 1) * ldw + (size_t)kbase * BK + c * 16;
+    for (int i = 0; i < WL; ++i) {
+        if (W_U8) {
+            const int r = (wave * 2 + i) * 16 + (lane >> 2), c = (lane & 3) ^ ((r >> 2) & 3);
+            gw[i] = (const unsigned char *)Wv + (size_t)min(m0 + r, M - 1) * ldw + (size_t)kbase * BK + c * 16;
+        } else {
+            const int r = (wave * 4 + i) * 8 + (lane >> 3), c = (lane & 7) ^ ((r >> 1) & 7);
+            gw[i] = (const unsigned char *)((const h16 *)Wv + (size_t)min(m0 + r, M - 1) * ldw + (size_t)kbase * BK + c * 8);
+        }
     }
     typedef __attribute__((address_space(1))) const void *gptr;
     typedef __attribute__((address_space(3))) void *lptr;
@@ -310,8 +327,8 @@ DEV void gemm_dma_body(int T, int N, int M, const h16 *__restrict__ A, int64_t l
         for (int i = 0; i < 4; ++i)
             __builtin_amdgcn_global_load_lds((gptr)(ga[i] + kt * BK), (lptr)(base + (wave * 4 + i) * 1024), 16, 0, 0);
 #pragma unroll
-        for (int i = 0; i < 2; ++i)
-            __builtin_amdgcn_global_load_lds((gptr)(gw[i] + kt * BK), (lptr)(base + D_A + (wave * 2 + i) * 1024), 16, 0, 0);
+        for (int i = 0; i < WL; ++i)
+            __builtin_amdgcn_global_load_lds((gptr)(gw[i] + kt * BK * (W_U8 ? 1 : 2)), (lptr)(base + D_A + (wave * WL + i) * 1024), 16, 0, 0);
     };
 
     f32x16 acc[4][2];
@@ -328,14 +345,20 @@ DEV void gemm_dma_body(int T, int N, int M, const h16 *__restrict__ A, int64_t l
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
         vA[ks] = lds0 + (wr * 128 + (lane & 31)) * 128 + (((2 * ks + (lane >> 5)) ^ ((lane >> 1) & 7)) << 4);
-        vB[ks] = lds0 + D_A + (wc * 64 + (lane & 31)) * 64 + ((ks ^ ((lane >> 2) & 3)) << 4) + (lane >> 5) * 8;
+        if (W_U8) vB[ks] = lds0 + D_A + (wc * 64 + (lane & 31)) * 64 + ((ks ^ ((lane >> 2) & 3)) << 4) + (lane >> 5) * 8;
+        else vB[ks] = lds0 + D_A + (wc * 64 + (lane & 31)) * 128 + (((2 * ks + (lane >> 5)) ^ ((lane >> 1) & 7)) << 4);
     }
-    h16x8 fa[2][4];
-    u32x2 rawb[2][2];
+    h16x8 fa[2][4], fbh[2][2];   // fbh: B fragments of fp16 weights
+    u32x2 rawb[2][2];            // B fragments of uint8 weights, before conversion
     auto ldfrag = [&](int buf, int so, int ks) {
         const uint32_t pa = vA[ks] + so, pb = vB[ks] + so;
-        asm volatile("ds_read_b64 %0, %1" : "=v"(rawb[buf][0]) : "v"(pb));
-        asm volatile("ds_read_b64 %0, %1 offset:2048" : "=v"(rawb[buf][1]) : "v"(pb));
+        if constexpr (W_U8) {
+            asm volatile("ds_read_b64 %0, %1" : "=v"(rawb[buf][0]) : "v"(pb));
+            asm volatile("ds_read_b64 %0, %1 offset:2048" : "=v"(rawb[buf][1]) : "v"(pb));
+        } else {
+            asm volatile("ds_read_b128 %0, %1" : "=v"(fbh[buf][0]) : "v"(pb));
+            asm volatile("ds_read_b128 %0, %1 offset:4096" : "=v"(fbh[buf][1]) : "v"(pb));
+        }
         asm volatile("ds_read_b128 %0, %1" : "=v"(fa[buf][0]) : "v"(pa));
         asm volatile("ds_read_b128 %0, %1 offset:4096" : "=v"(fa[buf][1]) : "v"(pa));
         asm volatile("ds_read_b128 %0, %1 offset:8192" : "=v"(fa[buf][2]) : "v"(pa));
@@ -351,10 +374,14 @@ DEV void gemm_dma_body(int T, int N, int M, const h16 *__restrict__ A, int64_t l
         h16x8 fb[2];
 #pragma unroll
         for (int b = 0; b < 2; ++b) {
-            const u32x2 raw = rawb[cur][b];
-            const h16x2 q0 = u8pair_lo_1024(raw.x) - off, q1 = u8pair_hi_1024(raw.x) - off;
-            const h16x2 q2 = u8pair_lo_1024(raw.y) - off, q3 = u8pair_hi_1024(raw.y) - off;
-            fb[b] = h16x8{q0.x, q0.y, q1.x, q1.y, q2.x, q2.y, q3.x, q3.y};
+            if constexpr (W_U8) {
+                const u32x2 raw = rawb[cur][b];
+                const h16x2 q0 = u8pair_lo_1024(raw.x) - off, q1 = u8pair_hi_1024(raw.x) - off;
+                const h16x2 q2 = u8pair_lo_1024(raw.y) - off, q3 = u8pair_hi_1024(raw.y) - off;
+                fb[b] = h16x8{q0.x, q0.y, q1.x, q1.y, q2.x, q2.y, q3.x, q3.y};
+            } else {
+                fb[b] = fbh[cur][b];
+            }
         }
 #pragma unroll
         for (int a = 0; a < 4; ++a)
@@ -363,12 +390,12 @@ DEV void gemm_dma_body(int T, int N, int M, const h16 *__restrict__ A, int64_t l
         __builtin_amdgcn_sched_barrier(0);
     };
 
-    // Every wave issues exactly six loads per tile, so "vmcnt(6 n)" means "all but my newest n tiles have landed".
-    // Past the last tile the loads repeat it into a stage nobody reads any more, which keeps the counts static.
+    // Every wave issues exactly LOADS loads per tile, so "vmcnt(LOADS n)" means "all but my newest n tiles have
+    // landed".  Past the last tile the loads repeat it into a stage nobody reads any more, which keeps the counts static.
     issue(0, 0);
     issue(min(1, nk - 1), D_STAGE);
-    issue(min(2, nk - 1), 2 * D_STAGE);
-    __builtin_amdgcn_s_waitcnt(0x0F7C);   // vmcnt(12): tile 0 has landed
+    if (D_NST > 2) issue(min(2, nk - 1), 2 * D_STAGE);
+    __builtin_amdgcn_s_waitcnt(vm_only((D_NST - 1) * Cfg::LOADS));   // tile 0 has landed
     __builtin_amdgcn_s_barrier();
     ldfrag(0, 0, 0);
     int so = 0;
@@ -386,10 +413,11 @@ DEV void gemm_dma_body(int T, int N, int M, const h16 *__restrict__ A, int64_t l
         __builtin_amdgcn_sched_barrier(0);
         older_reads_done(6);
         multiply(0);
-        // all my reads of this stage have returned and my part of tile kt + 1 has landed (tile kt + 2 may be in flight)
-        __builtin_amdgcn_s_waitcnt(0x0076);   // vmcnt(6) lgkmcnt(0)
+        // all my reads of this stage have returned and my part of tile kt + 1 has landed (with three stages tile
+        // kt + 2 may be in flight)
+        __builtin_amdgcn_s_waitcnt(vm_lgkm0((D_NST - 2) * Cfg::LOADS));
         __builtin_amdgcn_s_barrier();
-        issue(min(kt + 3, nk - 1), so);
+        issue(min(kt + D_NST, nk - 1), so);
         ldfrag(0, sn, 0);
         __builtin_amdgcn_sched_barrier(0);
         multiply(1);
@@ -415,12 +443,12 @@ DEV void gemm_dma_body(int T, int N, int M, const h16 *__restrict__ A, int64_t l
         // The accumulators pass through LDS (free now), 128 rows at a time, so that each thread finishes eight
         // consecutive outputs of one row: 16-byte loads of the residual / gate rows, 16-byte stores, and a body
         // small enough to stay in the instruction cache (per-element code for 128 accumulators does not).
-        constexpr int SW = 264;   // row stride in floats: 4 rows apart = 32 banks apart for the two half-waves
+        constexpr int SW = Cfg::STG_STRIDE;   // row stride in floats: 4 rows apart = 32 banks apart for the two half-waves
         float *stg = (float *)smem;
         const int cq = tid & 31, col = m0 + cq * 8;
         const bool col_ok = col < M;   // M % 8 == 0
         h16x8 rx8, mx8;
-        if (col_ok) { rx8 = *(const h16x8 *)(ep.rx + col); mx8 = *(const h16x8 *)(ep.mx + col); }
+        if (W_U8 && col_ok) { rx8 = *(const h16x8 *)(ep.rx + col); mx8 = *(const h16x8 *)(ep.mx + col); }
         __syncthreads();   // every wave has read its last fragments
 #pragma unroll 1
         for (int h = 0; h < 2; ++h) {
@@ -439,10 +467,14 @@ DEV void gemm_dma_body(int T, int N, int M, const h16 *__restrict__ A, int64_t l
                 const int row = it * 16 + (tid >> 5), t = t0 + h * 128 + row;
                 if (t < T && col_ok) {
                     const f32x4 v0 = *(const f32x4 *)(stg + row * SW + cq * 8), v1 = *(const f32x4 *)(stg + row * SW + cq * 8 + 4);
-                    const float s0t = ep.s0[t], s2t = ep.s2[t];
                     float v[8];
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) v[e] = epi_affine(e < 4 ? v0[e & 3] : v1[e & 3], (float)rx8[e], (float)mx8[e], s0t, s2t);
+                    for (int e = 0; e < 8; ++e) v[e] = e < 4 ? v0[e & 3] : v1[e & 3];
+                    if constexpr (W_U8) {
+                        const float s0t = ep.s0[t], s2t = ep.s2[t];
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) v[e] = epi_affine(v[e], (float)rx8[e], (float)mx8[e], s0t, s2t);
+                    }
                     if (ep.raw_f32) {
                         float *yo = (float *)Y + (size_t)t * ldy + col;
                         *(f32x4 *)yo = f32x4{v[0], v[1], v[2], v[3]};
@@ -472,11 +504,11 @@ DEV void gemm_dma_body(int T, int N, int M, const h16 *__restrict__ A, int64_t l
     }
 }
 
-template <bool SPLIT>
+template <bool W_U8, bool SPLIT>
 __global__ __launch_bounds__(512) void gemm_dma_kernel(int T, int N, int M, const h16 *__restrict__ A, int64_t lda,
-                                                       const uint8_t *__restrict__ W, int64_t ldw, void *__restrict__ Y,
+                                                       const void *__restrict__ W, int64_t ldw, void *__restrict__ Y,
                                                        int64_t ldy, GemmEpi ep, int nk_split, float *__restrict__ part) {
-    gemm_dma_body<SPLIT>(T, N, M, A, lda, W, ldw, Y, ldy, ep, nk_split, part);
+    gemm_dma_body<W_U8, SPLIT>(T, N, M, A, lda, W, ldw, Y, ldy, ep, nk_split, part);
 }
 
 // Up to four contractions [T, N] x [N, M_i] in one launch (blockIdx.y picks the operands), at full depth: short
@@ -498,9 +530,10 @@ __global__ __launch_bounds__(64 * WT * WM) void gemm_group_kernel(int T, int N, 
 }
 
 // the same through the direct-to-LDS kernel (uint8 weights, long calls)
+template <bool W_U8>
 __global__ __launch_bounds__(512) void gemm_dma_group_kernel(int T, int N, GemmGroup g) {
     const int gi = blockIdx.y, M = g.M[gi];
-    gemm_dma_body<false>(T, N, M, g.A[gi], g.lda, (const uint8_t *)g.W[gi], g.ldw[gi], g.Y[gi], M, g.ep[gi], N / BK, nullptr);
+    gemm_dma_body<W_U8, false>(T, N, M, g.A[gi], g.lda, g.W[gi], g.ldw[gi], g.Y[gi], M, g.ep[gi], N / BK, nullptr);
 }
 
 struct PrepGroup {
@@ -612,10 +645,13 @@ int launch_cfg(int64_t T, int64_t N, int64_t M, const rwkv_half *A, int64_t lda,
 }
 
 // what gemm_dma_kernel assumes: whole k-tiles, 16-byte rows and row starts for its loads and its eight-wide epilogue
-bool dma_ok(int64_t N, int64_t M, const void *A, int64_t lda, const void *W, int64_t ldw, const void *Y, int64_t ldy, const GemmEpi &ep) {
+bool dma_ok(bool w_u8, int64_t N, int64_t M, const void *A, int64_t lda, const void *W, int64_t ldw, const void *Y, int64_t ldy,
+            const GemmEpi &ep) {
     auto a16 = [](const void *p) { return (((uintptr_t)p) & 15) == 0; };
-    if (!ep.rx || !ep.mx || !ep.s0 || !ep.s2 || (N % BK) || (M & 7) || (lda & 7) || (ldw & 15) || (ldy & 7)) return false;
-    if (!a16(A) || !a16(W) || !a16(Y) || !a16(ep.rx) || !a16(ep.mx)) return false;
+    if ((N % BK) || (M & 7) || (lda & 7) || (ldw & (w_u8 ? 15 : 7)) || (ldy & 7)) return false;
+    if (!a16(A) || !a16(W) || !a16(Y)) return false;
+    if (w_u8 && (!ep.rx || !ep.mx || !ep.s0 || !ep.s2 || !a16(ep.rx) || !a16(ep.mx))) return false;
+    if (!w_u8 && ep.rx) return false;
     if (ep.act == ACT_RESIDUAL || ep.act == ACT_GATED_RESIDUAL)
         if (!ep.res || !a16(ep.res) || (ep.ldres & 7)) return false;
     if (ep.act == ACT_GATED_RESIDUAL)
@@ -623,20 +659,21 @@ bool dma_ok(int64_t N, int64_t M, const void *A, int64_t lda, const void *W, int
     return true;
 }
 
-// uint8 weights through gemm_dma_kernel.  Fewer than 192 tiles (narrow outputs): the contraction is split over
-// workgroups of the same tile until about one workgroup per CU is in flight; slabs and the second pass as in launch_cfg.
+// gemm_dma_kernel.  Fewer than 192 tiles (narrow outputs): the contraction is split over workgroups of the same
+// tile until about one workgroup per CU is in flight; slabs and the second pass as in launch_cfg.
+template <bool W_U8>
 int launch_dma(int64_t T, int64_t N, int64_t M, const rwkv_half *A, int64_t lda, const void *W, int64_t ldw, void *Y,
                int64_t ldy, const GemmEpi &ep, hipStream_t st) {
-    constexpr size_t lds = (size_t)D_NST * D_STAGE;
+    constexpr size_t lds = DmaCfg<W_U8>::LDS;
     static bool attr_done = false;
     if (!attr_done) {
-        hipError_t e = hipFuncSetAttribute((const void *)gemm_dma_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        hipError_t e = hipFuncSetAttribute((const void *)gemm_dma_kernel<W_U8, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e == hipSuccess)
-            e = hipFuncSetAttribute((const void *)gemm_dma_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            e = hipFuncSetAttribute((const void *)gemm_dma_kernel<W_U8, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return (int)e;
         attr_done = true;
     }
-    if (!dma_ok(N, M, A, lda, W, ldw, Y, ldy, ep)) return RWKV_E_LAYOUT;
+    if (!dma_ok(W_U8, N, M, A, lda, W, ldw, Y, ldy, ep)) return RWKV_E_LAYOUT;
     const int64_t tiles = ((T + DT - 1) / DT) * ((M + DM - 1) / DM);
     const int nk = (int)(N / BK);
     int ks = 1;
@@ -648,14 +685,14 @@ int launch_dma(int64_t T, int64_t N, int64_t M, const rwkv_half *A, int64_t lda,
             if (tiles * c >= 192) break;
         }
     if (ks > 1) {
-        hipLaunchKernelGGL(gemm_dma_kernel<true>, dim3((unsigned)tiles, (unsigned)ks), dim3(512), lds, st, (int)T, (int)N, (int)M,
-                           (const h16 *)A, lda, (const uint8_t *)W, ldw, Y, ldy, ep, nk / ks, ep.splitk_ws);
+        hipLaunchKernelGGL((gemm_dma_kernel<W_U8, true>), dim3((unsigned)tiles, (unsigned)ks), dim3(512), lds, st, (int)T, (int)N, (int)M,
+                           (const h16 *)A, lda, W, ldw, Y, ldy, ep, nk / ks, ep.splitk_ws);
         const int64_t n = T * M;
         const unsigned blocks = (unsigned)((n + 1023) / 1024 < 16384 ? (n + 1023) / 1024 : 16384);
         hipLaunchKernelGGL(splitk_epilogue_kernel, dim3(blocks), dim3(256), 0, st, (int)T, (int)M, ks, ep.splitk_ws, Y, ldy, ep);
     } else {
-        hipLaunchKernelGGL(gemm_dma_kernel<false>, dim3((unsigned)tiles), dim3(512), lds, st, (int)T, (int)N, (int)M, (const h16 *)A,
-                           lda, (const uint8_t *)W, ldw, Y, ldy, ep, nk, (float *)nullptr);
+        hipLaunchKernelGGL((gemm_dma_kernel<W_U8, false>), dim3((unsigned)tiles), dim3(512), lds, st, (int)T, (int)N, (int)M, (const h16 *)A,
+                           lda, W, ldw, Y, ldy, ep, nk, (float *)nullptr);
     }
     RWKV_LAUNCH_CHECK();
     return RWKV_OK;
@@ -669,34 +706,32 @@ int launch_pick(int cfg, int64_t T, int64_t N, int64_t M, const rwkv_half *A, in
         case 9:
             if constexpr (W_U8) return launch_cfg<true, 256, 256, 4, 4, 2>(T, N, M, A, lda, W, ldw, Y, ldy, ep, st);
             return RWKV_E_DTYPE;
-        case 14:
-            if constexpr (W_U8) return launch_dma(T, N, M, A, lda, W, ldw, Y, ldy, ep, st);
-            return RWKV_E_DTYPE;
+        case 14: return launch_dma<W_U8>(T, N, M, A, lda, W, ldw, Y, ldy, ep, st);
         default: return RWKV_E_DTYPE;
     }
 }
 
 // Tile choice (RWKV_GEMM_CFG overrides it for tuning sweeps).
-//   14  uint8 weights, 512 rows or more and an output of 3 M elements or more, operands laid out for 16-byte loads:
-//       the direct-to-LDS kernel (256 x 256 tiles; it splits K itself when there are few tiles)
+//   14  512 rows or more and an output of 3 M elements or more, operands laid out for 16-byte loads, no other product
+//       running beside this one: the direct-to-LDS kernel (256 x 256 tiles; it splits K itself when there are few tiles)
 //    9  uint8 weights otherwise, where 256 x 256 tiles of the register-staged kernel fill the chip: one per CU and
 //       round, the last round at least 70 % full
 //    3  everything else: 128 x 128 tiles, 4 k-tiles of prefetch
 int pick_cfg(int64_t T, int64_t M, bool w_u8, bool alone, bool dma) {
     const char *e = getenv("RWKV_GEMM_CFG");  // tuning override
     if (e && *e) return atoi(e);
-    if (!w_u8 || !alone) return 3;   // fp16 weight tiles are twice the bytes; a 256 x 256 tile's LDS leaves no room beside it
+    if (!alone) return 3;   // a 256 x 256 tile's LDS leaves no room beside it on the CU
     const int64_t big = ((T + 255) / 256) * ((M + 255) / 256), rounds = (big + 255) / 256;
     const bool fills = big * 10 >= rounds * 256 * 7;
     if (dma && T >= 512 && T * M >= ((int64_t)3 << 20) && (big < 192 || fills)) return 14;
-    return fills ? 9 : 3;
+    return w_u8 && fills ? 9 : 3;   // fp16 weight tiles are twice the bytes: the register-staged large tile spills
 }
 
 }  // namespace
 
 int gemm_launch(bool w_u8, int64_t T, int64_t N, int64_t M, const rwkv_half *A, int64_t lda, const void *W,
                 int64_t ldw, void *Y, int64_t ldy, const GemmEpi &ep, hipStream_t st) {
-    const int cfg = pick_cfg(T, M, w_u8, !ep.small_tiles, w_u8 && dma_ok(N, M, A, lda, W, ldw, Y, ldy, ep));
+    const int cfg = pick_cfg(T, M, w_u8, !ep.small_tiles, dma_ok(w_u8, N, M, A, lda, W, ldw, Y, ldy, ep));
     return w_u8 ? launch_pick<true>(cfg, T, N, M, A, lda, W, ldw, Y, ldy, ep, st)
                 : launch_pick<false>(cfg, T, N, M, A, lda, W, ldw, Y, ldy, ep, st);
 }
@@ -728,7 +763,7 @@ int gemm_group_launch(bool w_u8, int n, int64_t T, int64_t N, const rwkv_half *c
         hipLaunchKernelGGL(mm8_prepare_group_kernel, dim3((unsigned)((T + 3) / 4), (unsigned)n), dim3(256), 0, st, (int)T, (int)N, p);
     }
     int64_t tiles = 0, tiles_dma = 0;
-    bool dma = w_u8 && T >= 512;
+    bool dma = T >= 512;
     for (int i = 0; i < n; ++i) {
         if (mats[i]->N != N) return RWKV_E_SHAPE;
         g.A[i] = (const h16 *)(prep ? xs[i] : x[i]);
@@ -738,17 +773,22 @@ int gemm_group_launch(bool w_u8, int n, int64_t T, int64_t N, const rwkv_half *c
         if (w_u8) { g.ep[i].mx = mats[i]->mx; g.ep[i].rx = mats[i]->rx; g.ep[i].s0 = sums[i]; g.ep[i].s2 = sums[i] + T; }
         tiles = std::max<int64_t>(tiles, ((T + 127) / 128) * ((mats[i]->M + 127) / 128));
         tiles_dma = std::max<int64_t>(tiles_dma, ((T + DT - 1) / DT) * ((mats[i]->M + DM - 1) / DM));
-        dma = dma && dma_ok(N, mats[i]->M, g.A[i], N, g.W[i], g.ldw[i], g.Y[i], mats[i]->M, g.ep[i]);
+        dma = dma && dma_ok(w_u8, N, mats[i]->M, g.A[i], N, g.W[i], g.ldw[i], g.Y[i], mats[i]->M, g.ep[i]);
     }
     if (dma) {
-        constexpr size_t lds = (size_t)D_NST * D_STAGE;
         static bool attr_done = false;
         if (!attr_done) {
-            hipError_t e = hipFuncSetAttribute((const void *)gemm_dma_group_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            hipError_t e = hipFuncSetAttribute((const void *)gemm_dma_group_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                               (int)DmaCfg<true>::LDS);
+            if (e == hipSuccess)
+                e = hipFuncSetAttribute((const void *)gemm_dma_group_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                        (int)DmaCfg<false>::LDS);
             if (e != hipSuccess) return (int)e;
             attr_done = true;
         }
-        hipLaunchKernelGGL(gemm_dma_group_kernel, dim3((unsigned)tiles_dma, (unsigned)n), dim3(512), lds, st, (int)T, (int)N, g);
+        const dim3 grid((unsigned)tiles_dma, (unsigned)n);
+        if (w_u8) hipLaunchKernelGGL(gemm_dma_group_kernel<true>, grid, dim3(512), DmaCfg<true>::LDS, st, (int)T, (int)N, g);
+        else hipLaunchKernelGGL(gemm_dma_group_kernel<false>, grid, dim3(512), DmaCfg<false>::LDS, st, (int)T, (int)N, g);
         RWKV_LAUNCH_CHECK();
         return RWKV_OK;
     }

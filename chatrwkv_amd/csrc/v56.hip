@@ -233,9 +233,9 @@ extern "C" int rwkv_v56_forward(const rwkv_v56_model *m, const rwkv_v56_layer_st
         const rwkv_v56_layer &l = m->layers[i];
         const rwkv_v56_layer_state &s = states[i];
         const bool u8 = mat_is_u8(m->weights_u8, l.att_key);
-        // long calls with uint8 weights: every product through the direct-to-LDS kernel, one after the other (its
-        // tiles take a whole CU, so products side by side on several streams gain nothing)
-        const bool dma_seq = u8 && T >= 512;
+        // long calls: every product through the direct-to-LDS kernel, one after the other (its tiles take a whole
+        // CU, so products side by side on several streams gain nothing)
+        const bool dma_seq = T >= 512;
         const rwkv_half *kx, *vx, *rx, *gx = nullptr, *wx = nullptr;
         bool fuse_d1 = false;
         if (v6) {
@@ -286,8 +286,8 @@ extern "C" int rwkv_v56_forward(const rwkv_v56_model *m, const rwkv_v56_layer_st
             multi_vec_launch(u8, a, c.grid, st);
         } else {
             // One grouped launch at full depth for receptance, key, value (and gate): in short calls, where each
-            // product alone would split K and need a reduction pass, and in long calls with uint8 weights, where
-            // the group fills the chip with the 256 x 256 tiles of the direct-to-LDS kernel.
+            // product alone would split K and need a reduction pass, and in long calls, where the group fills the
+            // chip with the 256 x 256 tiles of the direct-to-LDS kernel.
             if ((dma_seq || (!ss && ((T + 127) / 128) * (C / 128) <= 128)) && !(C & 127)) {
                 const int n = gated ? 4 : 3;
                 const rwkv_half *xin[4] = {rx, kx, vx, gx};

@@ -583,13 +583,25 @@ extern "C" int rwkv_v7_forward(const rwkv_v7_model *m, const rwkv_v56_layer_stat
         // The three C x C products and the LoRA chain are independent of each other.  Long calls run them on three
         // streams: receptance and key on the caller's, value on the first side stream, the eight small LoRA
         // products (the only ones that split K: they share the split-K scratch) on the second.
-        const bool par = ss && fork_streams(ss, st, 2);
+        const bool dma_seq = T >= 512;   // long calls: direct-to-LDS kernel, whose tiles take a whole CU each
+        const bool par = ss && !dma_seq && fork_streams(ss, st, 2);
         Ctx cm = c, cv = c, cl = c;
         if (par) { cm.splitk = nullptr; cv.splitk = nullptr; cv.st = ss->s[0]; cl.st = ss->s[1]; }
         // the first matrix call also commits the new token-shift state (all readers of the old one are done)
+        if (dma_seq && !(C & 7)) {
+            // receptance, key and value as one grouped launch
+            const rwkv_half *xin[3] = {xr, xk, xv};
+            const rwkv_mat *mats[3] = {&l.att_receptance, &l.att_key, &l.att_value};
+            void *outs[3] = {ws.r, ws.k, v};
+            GemmEpi ep[3] = {};
+            for (int j = 0; j < 3; ++j) { ep[j].act = ACT_NONE; ep[j].out_scale = 1.f; ep[j].out_dtype = RWKV_DT_F16; }
+            if ((rc = copy_h16_launch(C, ws.xx_att, s.att_xx, st))) return rc;
+            if ((rc = gemm_group_launch(false, 3, T, C, xin, mats, outs, ep, nullptr, nullptr, st))) return rc;
+        } else {
         if ((rc = mm(cm, l.att_receptance, false, xr, ACT_NONE, nullptr, nullptr, 1.f, ws.r, ws.xx_att, s.att_xx, C))) return rc;
         if ((rc = mm(cm, l.att_key, false, xk, ACT_NONE, nullptr, nullptr, 1.f, ws.k))) return rc;
         if ((rc = mm(cv, l.att_value, false, xv, ACT_NONE, nullptr, nullptr, 1.f, v))) return rc;
+        }
         if ((rc = mm(cl, lora_first(l, 0, m->lora_w), false, xw, ACT_TANH, nullptr, nullptr, 1.f, ws.lw))) return rc;
         if ((rc = mm(cl, lora_second(l, 0, m->lora_w), false, ws.lw, ACT_NONE, nullptr, nullptr, 1.f, ws.w_raw))) return rc;
         if ((rc = mm(cl, lora_first(l, o_a, m->lora_a), false, xa, ACT_NONE, nullptr, nullptr, 1.f, ws.la))) return rc;
