@@ -425,7 +425,45 @@ DEV void gemm_dma_body(int T, int N, int M, const h16 *__restrict__ A, int64_t l
     }
     __builtin_amdgcn_s_waitcnt(0x0070);   // vmcnt(0) lgkmcnt(0): nothing may land in LDS after the workgroup has gone
 
+    // Each thread finishes eight consecutive outputs of one row: 16-byte loads of the residual / gate rows, 16-byte
+    // stores, and a body small enough to stay in the instruction cache (per-element code for 128 accumulators
+    // does not).
+    const int cq = tid & 31, col = m0 + cq * 8;
+    const bool col_ok = col < M;   // M % 8 == 0
+    h16x8 rx8, mx8;
+    if (W_U8 && col_ok) { rx8 = *(const h16x8 *)(ep.rx + col); mx8 = *(const h16x8 *)(ep.mx + col); }
+    auto finish8 = [&](int t, float (&v)[8]) {
+        if constexpr (W_U8) {
+            const float s0t = ep.s0[t], s2t = ep.s2[t];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[e] = epi_affine(v[e], (float)rx8[e], (float)mx8[e], s0t, s2t);
+        }
+        if (ep.raw_f32) {
+            float *yo = (float *)Y + (size_t)t * ldy + col;
+            *(f32x4 *)yo = f32x4{v[0], v[1], v[2], v[3]};
+            *(f32x4 *)(yo + 4) = f32x4{v[4], v[5], v[6], v[7]};
+            return;
+        }
+        h16x8 res8 = {}, gate8 = {};
+        if (ep.act == ACT_RESIDUAL || ep.act == ACT_GATED_RESIDUAL) res8 = *(const h16x8 *)(ep.res + (size_t)t * ep.ldres + col);
+        if (ep.act == ACT_GATED_RESIDUAL) gate8 = *(const h16x8 *)(ep.gate + (size_t)t * ep.ldgate + col);
+        float o[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) o[e] = epi_act(v[e], (float)res8[e], (float)gate8[e], ep);
+        if (ep.out_dtype == RWKV_DT_F32) {
+            float *yo = (float *)Y + (size_t)t * ldy + col;
+            *(f32x4 *)yo = f32x4{round_h(o[0]), round_h(o[1]), round_h(o[2]), round_h(o[3])};
+            *(f32x4 *)(yo + 4) = f32x4{round_h(o[4]), round_h(o[5]), round_h(o[6]), round_h(o[7])};
+        } else {
+            h16x8 y8;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) y8[e] = (h16)o[e];
+            *(h16x8 *)((rwkv_half *)Y + (size_t)t * ldy + col) = y8;
+        }
+    };
+
     if constexpr (SPLIT) {
+        // partial sums go to this split's fp32 slab; splitk_epilogue_kernel adds the slabs and finishes
         float *slab = part + (size_t)blockIdx.y * T * M;
 #pragma unroll
         for (int b = 0; b < 2; ++b) {
@@ -438,17 +476,10 @@ DEV void gemm_dma_body(int T, int N, int M, const h16 *__restrict__ A, int64_t l
                     if (m < M && t < T) slab[(size_t)t * M + m] = acc[a][b][e];
                 }
         }
-        return;
     } else {
-        // The accumulators pass through LDS (free now), 128 rows at a time, so that each thread finishes eight
-        // consecutive outputs of one row: 16-byte loads of the residual / gate rows, 16-byte stores, and a body
-        // small enough to stay in the instruction cache (per-element code for 128 accumulators does not).
+        // The accumulators pass through LDS (free now), 128 rows at a time.
         constexpr int SW = Cfg::STG_STRIDE;   // row stride in floats: 4 rows apart = 32 banks apart for the two half-waves
         float *stg = (float *)smem;
-        const int cq = tid & 31, col = m0 + cq * 8;
-        const bool col_ok = col < M;   // M % 8 == 0
-        h16x8 rx8, mx8;
-        if (W_U8 && col_ok) { rx8 = *(const h16x8 *)(ep.rx + col); mx8 = *(const h16x8 *)(ep.mx + col); }
         __syncthreads();   // every wave has read its last fragments
 #pragma unroll 1
         for (int h = 0; h < 2; ++h) {
@@ -467,36 +498,8 @@ DEV void gemm_dma_body(int T, int N, int M, const h16 *__restrict__ A, int64_t l
                 const int row = it * 16 + (tid >> 5), t = t0 + h * 128 + row;
                 if (t < T && col_ok) {
                     const f32x4 v0 = *(const f32x4 *)(stg + row * SW + cq * 8), v1 = *(const f32x4 *)(stg + row * SW + cq * 8 + 4);
-                    float v[8];
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) v[e] = e < 4 ? v0[e & 3] : v1[e & 3];
-                    if constexpr (W_U8) {
-                        const float s0t = ep.s0[t], s2t = ep.s2[t];
-#pragma unroll
-                        for (int e = 0; e < 8; ++e) v[e] = epi_affine(v[e], (float)rx8[e], (float)mx8[e], s0t, s2t);
-                    }
-                    if (ep.raw_f32) {
-                        float *yo = (float *)Y + (size_t)t * ldy + col;
-                        *(f32x4 *)yo = f32x4{v[0], v[1], v[2], v[3]};
-                        *(f32x4 *)(yo + 4) = f32x4{v[4], v[5], v[6], v[7]};
-                    } else {
-                        h16x8 res8 = {}, gate8 = {};
-                        if (ep.act == ACT_RESIDUAL || ep.act == ACT_GATED_RESIDUAL) res8 = *(const h16x8 *)(ep.res + (size_t)t * ep.ldres + col);
-                        if (ep.act == ACT_GATED_RESIDUAL) gate8 = *(const h16x8 *)(ep.gate + (size_t)t * ep.ldgate + col);
-                        float o[8];
-#pragma unroll
-                        for (int e = 0; e < 8; ++e) o[e] = epi_act(v[e], (float)res8[e], (float)gate8[e], ep);
-                        if (ep.out_dtype == RWKV_DT_F32) {
-                            float *yo = (float *)Y + (size_t)t * ldy + col;
-                            *(f32x4 *)yo = f32x4{round_h(o[0]), round_h(o[1]), round_h(o[2]), round_h(o[3])};
-                            *(f32x4 *)(yo + 4) = f32x4{round_h(o[4]), round_h(o[5]), round_h(o[6]), round_h(o[7])};
-                        } else {
-                            h16x8 y8;
-#pragma unroll
-                            for (int e = 0; e < 8; ++e) y8[e] = (h16)o[e];
-                            *(h16x8 *)((rwkv_half *)Y + (size_t)t * ldy + col) = y8;
-                        }
-                    }
+                    float v[8] = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
+                    finish8(t, v);
                 }
             }
             __syncthreads();
