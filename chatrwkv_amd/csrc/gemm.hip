@@ -288,7 +288,7 @@ constexpr int vm_lgkm0(int n) { return 0x0070 | (n & 15) | ((n >> 4) << 14); }
 
 template <bool W_U8, bool SPLIT>
 DEV void gemm_dma_body(int T, int N, int M, const h16 *__restrict__ A, int64_t lda, const void *__restrict__ Wv, int64_t ldw,
-                       void *__restrict__ Y, int64_t ldy, const GemmEpi &ep, int nk_split, float *__restrict__ part) {
+                       void *__restrict__ Y, int64_t ldy, const GemmEpi &ep, int nk_split, float *__restrict__ part, int split) {
     using Cfg = DmaCfg<W_U8>;
     constexpr int D_STAGE = Cfg::STAGE, D_NST = Cfg::NST, WL = Cfg::W / 8192;   // WL: weight loads per wave and tile
     extern __shared__ __align__(1024) unsigned char smem[];
@@ -299,7 +299,7 @@ DEV void gemm_dma_body(int T, int N, int M, const h16 *__restrict__ A, int64_t l
     if ((gridDim.x & 7) == 0) bid = (bid & 7) * (gridDim.x >> 3) + (bid >> 3);
     const int t0 = (bid % tiles_t) * DT, m0 = (bid / tiles_t) * DM;
     if (m0 >= M) return;   // grouped launches size the grid for their widest member
-    const int kbase = SPLIT ? blockIdx.y * nk_split : 0, nk = SPLIT ? nk_split : N / BK;
+    const int kbase = SPLIT ? split * nk_split : 0, nk = SPLIT ? nk_split : N / BK;
 
     // load sources; rows past the end re-read the last row (never stored)
     const h16 *ga[4];
@@ -464,7 +464,7 @@ DEV void gemm_dma_body(int T, int N, int M, const h16 *__restrict__ A, int64_t l
 
     if constexpr (SPLIT) {
         // partial sums go to this split's fp32 slab; splitk_epilogue_kernel adds the slabs and finishes
-        float *slab = part + (size_t)blockIdx.y * T * M;
+        float *slab = part + (size_t)split * T * M;
 #pragma unroll
         for (int b = 0; b < 2; ++b) {
             const int m = m0 + wc * 64 + b * 32 + (lane & 31);
@@ -511,7 +511,7 @@ template <bool W_U8, bool SPLIT>
 __global__ __launch_bounds__(512) void gemm_dma_kernel(int T, int N, int M, const h16 *__restrict__ A, int64_t lda,
                                                        const void *__restrict__ W, int64_t ldw, void *__restrict__ Y,
                                                        int64_t ldy, GemmEpi ep, int nk_split, float *__restrict__ part) {
-    gemm_dma_body<W_U8, SPLIT>(T, N, M, A, lda, W, ldw, Y, ldy, ep, nk_split, part);
+    gemm_dma_body<W_U8, SPLIT>(T, N, M, A, lda, W, ldw, Y, ldy, ep, nk_split, part, SPLIT ? blockIdx.y : 0);
 }
 
 // Up to four contractions [T, N] x [N, M_i] in one launch (blockIdx.y picks the operands), at full depth: short
@@ -522,6 +522,8 @@ struct GemmGroup {
     void *Y[4];
     int64_t lda, ldw[4];
     int M[4];
+    float *part[4];   // split-K slabs of member i, [splits][T][M_i] (direct-to-LDS group only)
+    int nk_split;
     GemmEpi ep[4];
 };
 
@@ -532,11 +534,31 @@ __global__ __launch_bounds__(64 * WT * WM) void gemm_group_kernel(int T, int N, 
                                                nullptr);
 }
 
-// the same through the direct-to-LDS kernel (uint8 weights, long calls)
-template <bool W_U8>
+// the same through the direct-to-LDS kernel; blockIdx.z is the k split when the group has too few tiles for the chip
+template <bool W_U8, bool SPLIT>
 __global__ __launch_bounds__(512) void gemm_dma_group_kernel(int T, int N, GemmGroup g) {
     const int gi = blockIdx.y, M = g.M[gi];
-    gemm_dma_body<W_U8, false>(T, N, M, g.A[gi], g.lda, g.W[gi], g.ldw[gi], g.Y[gi], M, g.ep[gi], N / BK, nullptr);
+    gemm_dma_body<W_U8, SPLIT>(T, N, M, g.A[gi], g.lda, g.W[gi], g.ldw[gi], g.Y[gi], M, g.ep[gi], SPLIT ? g.nk_split : N / BK,
+                               g.part[gi], SPLIT ? blockIdx.z : 0);
+}
+
+// second pass of a split group: member blockIdx.y, as splitk_epilogue_kernel
+__global__ __launch_bounds__(256) void splitk_group_epilogue_kernel(int T, int KS, GemmGroup g) {
+    const int gi = blockIdx.y, M = g.M[gi];
+    const float *__restrict__ part = g.part[gi];
+    const int64_t n4 = (int64_t)T * M / 4, n = (int64_t)T * M;
+    const int m4 = M / 4;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n4; i += (int64_t)gridDim.x * 256) {
+        const int t = (int)(i / m4), m = (int)(i - (int64_t)t * m4) * 4;
+        f32x4 v = *(const f32x4 *)(part + 4 * i);
+        for (int k = 1; k < KS; ++k) v += *(const f32x4 *)(part + (size_t)k * n + 4 * i);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            float rxm = 1.f, mxm = 0.f;
+            if (g.ep[gi].rx) { rxm = h2f(g.ep[gi].rx[m + e]); mxm = h2f(g.ep[gi].mx[m + e]); }
+            gemm_epilogue(v[e], t, m + e, rxm, mxm, g.ep[gi], g.Y[gi], M);
+        }
+    }
 }
 
 struct PrepGroup {
@@ -751,9 +773,11 @@ int mm8_prepare_launch(int64_t T, int64_t N, const rwkv_half *x, int64_t ldx, co
 // n (2..4) products [T, N] x [N, M_i] of uint8 or fp16 weights with their own inputs, outputs and epilogues in one
 // launch.  uint8 with xs != NULL: x[i] is the unscaled activation and xs[i] / sums[i] (2 T floats) are scratch;
 // uint8 with xs == NULL: x[i] is already scaled by ry and sums[i] holds its row sums.
-// Calls of 512 rows or more with uint8 weights go through the direct-to-LDS kernel, others through 128 x 128 tiles.
+// Calls of 256 rows or more go through the direct-to-LDS kernel (splitting K over splitk_ws, RWKV_SPLITK_WS_BYTES of
+// scratch or NULL, while the group has fewer than 192 tiles), shorter ones through 128 x 128 tiles at full depth.
 int gemm_group_launch(bool w_u8, int n, int64_t T, int64_t N, const rwkv_half *const *x, const rwkv_mat *const *mats,
-                      void *const *Y, const GemmEpi *eps, rwkv_half *const *xs, float *const *sums, hipStream_t st) {
+                      void *const *Y, const GemmEpi *eps, rwkv_half *const *xs, float *const *sums, float *splitk_ws,
+                      hipStream_t st) {
     if (n < 2 || n > 4 || (N % BK)) return RWKV_E_SHAPE;
     GemmGroup g{};
     g.lda = N;
@@ -765,8 +789,8 @@ int gemm_group_launch(bool w_u8, int n, int64_t T, int64_t N, const rwkv_half *c
         }
         hipLaunchKernelGGL(mm8_prepare_group_kernel, dim3((unsigned)((T + 3) / 4), (unsigned)n), dim3(256), 0, st, (int)T, (int)N, p);
     }
-    int64_t tiles = 0, tiles_dma = 0;
-    bool dma = T >= 512;
+    int64_t tiles = 0, tiles_dma = 0, total_dma = 0, out_elems = 0, max_out = 0;
+    bool dma = T >= 256, m4 = true;
     for (int i = 0; i < n; ++i) {
         if (mats[i]->N != N) return RWKV_E_SHAPE;
         g.A[i] = (const h16 *)(prep ? xs[i] : x[i]);
@@ -775,23 +799,50 @@ int gemm_group_launch(bool w_u8, int n, int64_t T, int64_t N, const rwkv_half *c
         g.ep[i].ldres = g.ep[i].ldgate = mats[i]->M;
         if (w_u8) { g.ep[i].mx = mats[i]->mx; g.ep[i].rx = mats[i]->rx; g.ep[i].s0 = sums[i]; g.ep[i].s2 = sums[i] + T; }
         tiles = std::max<int64_t>(tiles, ((T + 127) / 128) * ((mats[i]->M + 127) / 128));
-        tiles_dma = std::max<int64_t>(tiles_dma, ((T + DT - 1) / DT) * ((mats[i]->M + DM - 1) / DM));
+        const int64_t td = ((T + DT - 1) / DT) * ((mats[i]->M + DM - 1) / DM);
+        tiles_dma = std::max(tiles_dma, td);
+        total_dma += td;
+        out_elems += T * mats[i]->M;
+        max_out = std::max<int64_t>(max_out, T * mats[i]->M);
+        m4 = m4 && !(mats[i]->M & 3);
         dma = dma && dma_ok(w_u8, N, mats[i]->M, g.A[i], N, g.W[i], g.ldw[i], g.Y[i], mats[i]->M, g.ep[i]);
     }
     if (dma) {
         static bool attr_done = false;
         if (!attr_done) {
-            hipError_t e = hipFuncSetAttribute((const void *)gemm_dma_group_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                               (int)DmaCfg<true>::LDS);
-            if (e == hipSuccess)
-                e = hipFuncSetAttribute((const void *)gemm_dma_group_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                        (int)DmaCfg<false>::LDS);
-            if (e != hipSuccess) return (int)e;
+            const void *fn[4] = {(const void *)gemm_dma_group_kernel<true, false>, (const void *)gemm_dma_group_kernel<true, true>,
+                                 (const void *)gemm_dma_group_kernel<false, false>, (const void *)gemm_dma_group_kernel<false, true>};
+            for (int i = 0; i < 4; ++i) {
+                hipError_t e = hipFuncSetAttribute(fn[i], hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                   (int)(i < 2 ? DmaCfg<true>::LDS : DmaCfg<false>::LDS));
+                if (e != hipSuccess) return (int)e;
+            }
             attr_done = true;
         }
-        const dim3 grid((unsigned)tiles_dma, (unsigned)n);
-        if (w_u8) hipLaunchKernelGGL(gemm_dma_group_kernel<true>, grid, dim3(512), DmaCfg<true>::LDS, st, (int)T, (int)N, g);
-        else hipLaunchKernelGGL(gemm_dma_group_kernel<false>, grid, dim3(512), DmaCfg<false>::LDS, st, (int)T, (int)N, g);
+        const int nk = (int)(N / BK);
+        int ks = 1;
+        if (splitk_ws && total_dma < 192 && m4)
+            for (int c = 2; c <= 8; c <<= 1) {
+                if (nk % c || nk / c < 8) break;
+                if ((size_t)c * out_elems * sizeof(float) > RWKV_SPLITK_WS_BYTES) break;
+                ks = c;
+                if (total_dma * c >= 192) break;
+            }
+        g.nk_split = nk / ks;
+        if (ks > 1) {
+            float *p = splitk_ws;
+            for (int i = 0; i < n; ++i) { g.part[i] = p; p += (size_t)ks * T * mats[i]->M; }
+        }
+        const dim3 grid((unsigned)tiles_dma, (unsigned)n, (unsigned)ks);
+        const size_t lds = w_u8 ? DmaCfg<true>::LDS : DmaCfg<false>::LDS;
+        if (w_u8 && ks > 1) hipLaunchKernelGGL((gemm_dma_group_kernel<true, true>), grid, dim3(512), lds, st, (int)T, (int)N, g);
+        else if (w_u8) hipLaunchKernelGGL((gemm_dma_group_kernel<true, false>), grid, dim3(512), lds, st, (int)T, (int)N, g);
+        else if (ks > 1) hipLaunchKernelGGL((gemm_dma_group_kernel<false, true>), grid, dim3(512), lds, st, (int)T, (int)N, g);
+        else hipLaunchKernelGGL((gemm_dma_group_kernel<false, false>), grid, dim3(512), lds, st, (int)T, (int)N, g);
+        if (ks > 1) {
+            const unsigned blocks = (unsigned)std::min<int64_t>((max_out + 1023) / 1024, 16384);
+            hipLaunchKernelGGL(splitk_group_epilogue_kernel, dim3(blocks, (unsigned)n), dim3(256), 0, st, (int)T, ks, g);
+        }
         RWKV_LAUNCH_CHECK();
         return RWKV_OK;
     }

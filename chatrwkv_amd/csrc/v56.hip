@@ -286,9 +286,9 @@ extern "C" int rwkv_v56_forward(const rwkv_v56_model *m, const rwkv_v56_layer_st
             multi_vec_launch(u8, a, c.grid, st);
         } else {
             // One grouped launch at full depth for receptance, key, value (and gate): in short calls, where each
-            // product alone would split K and need a reduction pass, and in long calls, where the group fills the
-            // chip with the 256 x 256 tiles of the direct-to-LDS kernel.
-            if ((dma_seq || (!ss && ((T + 127) / 128) * (C / 128) <= 128)) && !(C & 127)) {
+            // product alone would split K and need a reduction pass, and from 256 rows on, where the group goes
+            // through the direct-to-LDS kernel (256 x 256 tiles, K split while the group has few tiles).
+            if ((T >= 256 || (!ss && ((T + 127) / 128) * (C / 128) <= 128)) && !(C & 127)) {
                 const int n = gated ? 4 : 3;
                 const rwkv_half *xin[4] = {rx, kx, vx, gx};
                 const rwkv_mat *mats[4] = {&l.att_receptance, &l.att_key, &l.att_value, &l.att_gate};
@@ -302,7 +302,7 @@ extern "C" int rwkv_v56_forward(const rwkv_v56_model *m, const rwkv_v56_layer_st
                     ep[j].ldres = C; ep[j].ldgate = C;
                 }
                 if ((rc = copy_h16_launch(C, ws.xx_att, s.att_xx, st))) return rc;
-                if ((rc = gemm_group_launch(u8, n, T, C, xin, mats, outs, ep, xsc, sm, st))) return rc;
+                if ((rc = gemm_group_launch(u8, n, T, C, xin, mats, outs, ep, xsc, sm, ws.splitk, st))) return rc;
             } else {
             // receptance (then gate) on the caller's stream, key and value on the side streams
             const bool par = ss && !dma_seq && fork_streams(ss, st, 2);
@@ -356,7 +356,7 @@ extern "C" int rwkv_v56_forward(const rwkv_v56_model *m, const rwkv_v56_layer_st
             ep[0].act = ACT_SIGMOID; ep[1].act = ACT_RELU_SQ;
             for (int j = 0; j < 2; ++j) { ep[j].out_scale = 1.f; ep[j].out_dtype = RWKV_DT_F16; }
             if ((rc = copy_h16_launch(C, ws.xx_ffn, s.ffn_xx, st))) return rc;
-            if ((rc = gemm_group_launch(u8, 2, T, C, xin, mats, outs, ep, xsc, sm, st))) return rc;
+            if ((rc = gemm_group_launch(u8, 2, T, C, xin, mats, outs, ep, xsc, sm, ws.splitk, st))) return rc;
         } else {
             // channel-mix receptance beside the key product
             const bool par = ss && !dma_seq && fork_streams(ss, st, 1);

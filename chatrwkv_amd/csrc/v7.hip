@@ -580,13 +580,14 @@ extern "C" int rwkv_v7_forward(const rwkv_v7_model *m, const rwkv_v56_layer_stat
         const rwkv_half *xr = ws.mix[0], *xw = ws.mix[1], *xk = ws.mix[2], *xv = ws.mix[3], *xa = ws.mix[4],
                         *xg = ws.mix[5];
         rwkv_half *v = i == 0 ? ws.v_first : ws.v;
-        // The three C x C products and the LoRA chain are independent of each other.  Long calls run them on three
-        // streams: receptance and key on the caller's, value on the first side stream, the eight small LoRA
-        // products (the only ones that split K: they share the split-K scratch) on the second.
-        const bool dma_seq = T >= 512;   // long calls: direct-to-LDS kernel, whose tiles take a whole CU each
-        const bool par = ss && !dma_seq && fork_streams(ss, st, 2);
+        // The three C x C products and the LoRA chain are independent of each other.  From 256 rows on receptance,
+        // key and value are one grouped launch of the direct-to-LDS kernel; where that group fills three quarters
+        // of the chip without splitting K, the eight small LoRA products (which do split K: one user of the split-K
+        // scratch at a time) run beside it on a side stream, on the CUs the group leaves free.
+        const bool dma_seq = T >= 256;
+        const bool par = ss && dma_seq && 3 * ((T + 255) / 256) * ((C + 255) / 256) >= 192 && fork_streams(ss, st, 1);
         Ctx cm = c, cv = c, cl = c;
-        if (par) { cm.splitk = nullptr; cv.splitk = nullptr; cv.st = ss->s[0]; cl.st = ss->s[1]; }
+        if (par) cl.st = ss->s[0];
         // the first matrix call also commits the new token-shift state (all readers of the old one are done)
         if (dma_seq && !(C & 7)) {
             // receptance, key and value as one grouped launch
@@ -596,7 +597,7 @@ extern "C" int rwkv_v7_forward(const rwkv_v7_model *m, const rwkv_v56_layer_stat
             GemmEpi ep[3] = {};
             for (int j = 0; j < 3; ++j) { ep[j].act = ACT_NONE; ep[j].out_scale = 1.f; ep[j].out_dtype = RWKV_DT_F16; }
             if ((rc = copy_h16_launch(C, ws.xx_att, s.att_xx, st))) return rc;
-            if ((rc = gemm_group_launch(false, 3, T, C, xin, mats, outs, ep, nullptr, nullptr, st))) return rc;
+            if ((rc = gemm_group_launch(false, 3, T, C, xin, mats, outs, ep, nullptr, nullptr, ws.splitk, st))) return rc;
         } else {
         if ((rc = mm(cm, l.att_receptance, false, xr, ACT_NONE, nullptr, nullptr, 1.f, ws.r, ws.xx_att, s.att_xx, C))) return rc;
         if ((rc = mm(cm, l.att_key, false, xk, ACT_NONE, nullptr, nullptr, 1.f, ws.k))) return rc;
@@ -612,7 +613,7 @@ extern "C" int rwkv_v7_forward(const rwkv_v7_model *m, const rwkv_v56_layer_stat
         }
         if ((rc = mm(cl, lora_first(l, o_g, m->lora_g), false, xg, ACT_SIGMOID, nullptr, nullptr, 1.f, ws.lg))) return rc;
         if ((rc = mm(cl, lora_second(l, o_g, m->lora_g), false, ws.lg, ACT_NONE, nullptr, nullptr, 1.f, ws.g))) return rc;
-        if (par && !join_streams(ss, st, 2)) return (int)hipErrorUnknown;
+        if (par && !join_streams(ss, st, 1)) return (int)hipErrorUnknown;
         {
             Prep7Args a{};
             a.T = (int)T; a.C = C; a.H = H; a.r = ws.r; a.k = ws.k; a.v = v; a.w_raw = ws.w_raw; a.a_raw = ws.a_raw;
