@@ -684,6 +684,21 @@ bool dma_ok(bool w_u8, int64_t N, int64_t M, const void *A, int64_t lda, const v
     return true;
 }
 
+// K split of a direct-to-LDS launch with `tiles` 256 x 256 tiles of nk k-tiles each: whole rounds over the 256 CUs
+// cost their k-tiles plus about six k-tile times of fill and drain, and every split adds a slab to write and read
+// back (about one and a half k-tile times).  1 where the tiles fill the chip anyway.
+int dma_split(int64_t tiles, int nk, size_t out_bytes, size_t ws_bytes) {
+    if (tiles >= 192) return 1;
+    int best = 1;
+    double best_cost = 1e30;
+    for (int c = 1; c <= 8; ++c) {
+        if (nk % c || (c > 1 && nk / c < 8) || (c > 1 && c * out_bytes > ws_bytes)) continue;
+        const double cost = (double)((tiles * c + 255) / 256) * (nk / c + 6) + (c > 1 ? 1.5 * c : 0.0);
+        if (cost < best_cost) { best_cost = cost; best = c; }
+    }
+    return best;
+}
+
 // gemm_dma_kernel.  Fewer than 192 tiles (narrow outputs): the contraction is split over workgroups of the same
 // tile until about one workgroup per CU is in flight; slabs and the second pass as in launch_cfg.
 template <bool W_U8>
@@ -702,13 +717,7 @@ int launch_dma(int64_t T, int64_t N, int64_t M, const rwkv_half *A, int64_t lda,
     const int64_t tiles = ((T + DT - 1) / DT) * ((M + DM - 1) / DM);
     const int nk = (int)(N / BK);
     int ks = 1;
-    if (ep.splitk_ws && tiles < 192 && (M & 3) == 0)
-        for (int c = 2; c <= 8; c <<= 1) {
-            if (nk % c || nk / c < 8) break;
-            if ((size_t)c * T * M * sizeof(float) > ep.splitk_bytes) break;
-            ks = c;
-            if (tiles * c >= 192) break;
-        }
+    if (ep.splitk_ws && (M & 3) == 0) ks = dma_split(tiles, nk, (size_t)T * M * sizeof(float), ep.splitk_bytes);
     if (ks > 1) {
         hipLaunchKernelGGL((gemm_dma_kernel<W_U8, true>), dim3((unsigned)tiles, (unsigned)ks), dim3(512), lds, st, (int)T, (int)N, (int)M,
                            (const h16 *)A, lda, W, ldw, Y, ldy, ep, nk / ks, ep.splitk_ws);
@@ -821,13 +830,7 @@ int gemm_group_launch(bool w_u8, int n, int64_t T, int64_t N, const rwkv_half *c
         }
         const int nk = (int)(N / BK);
         int ks = 1;
-        if (splitk_ws && total_dma < 192 && m4)
-            for (int c = 2; c <= 8; c <<= 1) {
-                if (nk % c || nk / c < 8) break;
-                if ((size_t)c * out_elems * sizeof(float) > RWKV_SPLITK_WS_BYTES) break;
-                ks = c;
-                if (total_dma * c >= 192) break;
-            }
+        if (splitk_ws && m4) ks = dma_split(total_dma, nk, (size_t)out_elems * sizeof(float), RWKV_SPLITK_WS_BYTES);
         g.nk_split = nk / ks;
         if (ks > 1) {
             float *p = splitk_ws;
