@@ -276,46 +276,53 @@ __global__ __launch_bounds__(64 * WT * WM) void gemm_kernel(int T, int N, int M,
 // s_waitcnt: the compiler waits for lgkmcnt(0) wherever older and newer reads are both outstanding.
 // fp16 weights (W_U8 = false): the weight tile is laid out like the A tile (32 KB), a stage is 64 KB and two fit, so
 // one tile is in flight while one multiplies.
-constexpr int DT = 256, DM = 256, D_A = DT * BK * 2;
-template <bool W_U8> struct DmaCfg {
-    static constexpr int W = W_U8 ? DM * BK : DM * BK * 2, STAGE = D_A + W, NST = W_U8 ? 3 : 2, LOADS = 4 + W / 8192;
-    static constexpr int STG_STRIDE = 264;   // epilogue staging: 128 rows of 256 floats, padded (see the epilogue)
+// Tile TM x TN is 256 x 256 (wave tile 128 x 64: the long, wide products) or 128 x 128 (wave tile 64 x 32, a stage of
+// 24 KB: products with too few 256 x 256 tiles for the chip run at full depth with these instead of splitting K).
+constexpr int DT = 256, DM = 256;
+template <bool W_U8, int TM, int TN> struct DmaCfg {
+    static constexpr int A = TM * BK * 2, W = W_U8 ? TN * BK : TN * BK * 2, STAGE = A + W;
+    static constexpr int NST = (W_U8 || TM < 256) ? 3 : 2;
+    static constexpr int AL = TM / 64, WL = W / 8192, LOADS = AL + WL;   // 1 KB loads per wave and tile
+    static constexpr int MI = TM / 64, NI = TN / 128;                    // 32 x 32 blocks per wave (2 x 4 waves)
+    static constexpr int STG_STRIDE = TN + 8;   // epilogue staging: 128 rows of TN floats, padded (see the epilogue)
     static constexpr size_t LDS = (size_t)NST * STAGE > (size_t)128 * STG_STRIDE * 4 ? (size_t)NST * STAGE : (size_t)128 * STG_STRIDE * 4;
 };
-// s_waitcnt immediates: vmcnt(n) alone, and vmcnt(n) with lgkmcnt(0)
+// s_waitcnt immediates: vmcnt(n) alone, vmcnt(n) with lgkmcnt(0), lgkmcnt(n) alone
 constexpr int vm_only(int n) { return 0x0F70 | (n & 15) | ((n >> 4) << 14); }
 constexpr int vm_lgkm0(int n) { return 0x0070 | (n & 15) | ((n >> 4) << 14); }
+constexpr int lgkm_only(int n) { return 0xC07F | (n << 8); }
 
-template <bool W_U8, bool SPLIT>
+template <bool W_U8, bool SPLIT, int TM, int TN>
 DEV void gemm_dma_body(int T, int N, int M, const h16 *__restrict__ A, int64_t lda, const void *__restrict__ Wv, int64_t ldw,
                        void *__restrict__ Y, int64_t ldy, const GemmEpi &ep, int nk_split, float *__restrict__ part, int split) {
-    using Cfg = DmaCfg<W_U8>;
-    constexpr int D_STAGE = Cfg::STAGE, D_NST = Cfg::NST, WL = Cfg::W / 8192;   // WL: weight loads per wave and tile
+    using Cfg = DmaCfg<W_U8, TM, TN>;
+    constexpr int D_A = Cfg::A, D_STAGE = Cfg::STAGE, D_NST = Cfg::NST, AL = Cfg::AL, WL = Cfg::WL, MI = Cfg::MI, NI = Cfg::NI;
+    static_assert((TM == 256 || TM == 128) && (TN == 256 || TN == 128), "tile");
     extern __shared__ __align__(1024) unsigned char smem[];
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wr = wave >> 2, wc = wave & 3;
-    const int tiles_t = (T + DT - 1) / DT;
+    const int tiles_t = (T + TM - 1) / TM;
     int bid = blockIdx.x;
     if ((gridDim.x & 7) == 0) bid = (bid & 7) * (gridDim.x >> 3) + (bid >> 3);
-    const int t0 = (bid % tiles_t) * DT, m0 = (bid / tiles_t) * DM;
+    const int t0 = (bid % tiles_t) * TM, m0 = (bid / tiles_t) * TN;
     if (m0 >= M) return;   // grouped launches size the grid for their widest member
     const int kbase = SPLIT ? split * nk_split : 0, nk = SPLIT ? nk_split : N / BK;
 
     // load sources; rows past the end re-read the last row (never stored)
-    const h16 *ga[4];
+    const h16 *ga[AL];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int r = (wave * 4 + i) * 8 + (lane >> 3), c = (lane & 7) ^ ((r >> 1) & 7);
+    for (int i = 0; i < AL; ++i) {
+        const int r = (wave * AL + i) * 8 + (lane >> 3), c = (lane & 7) ^ ((r >> 1) & 7);
         ga[i] = A + (size_t)min(t0 + r, T - 1) * lda + (size_t)kbase * BK + c * 8;
     }
     const unsigned char *gw[WL];   // byte pointers
 #pragma unroll
     for (int i = 0; i < WL; ++i) {
         if (W_U8) {
-            const int r = (wave * 2 + i) * 16 + (lane >> 2), c = (lane & 3) ^ ((r >> 2) & 3);
+            const int r = (wave * WL + i) * 16 + (lane >> 2), c = (lane & 3) ^ ((r >> 2) & 3);
             gw[i] = (const unsigned char *)Wv + (size_t)min(m0 + r, M - 1) * ldw + (size_t)kbase * BK + c * 16;
         } else {
-            const int r = (wave * 4 + i) * 8 + (lane >> 3), c = (lane & 7) ^ ((r >> 1) & 7);
+            const int r = (wave * WL + i) * 8 + (lane >> 3), c = (lane & 7) ^ ((r >> 1) & 7);
             gw[i] = (const unsigned char *)((const h16 *)Wv + (size_t)min(m0 + r, M - 1) * ldw + (size_t)kbase * BK + c * 8);
         }
     }
@@ -324,18 +331,18 @@ DEV void gemm_dma_body(int T, int N, int M, const h16 *__restrict__ A, int64_t l
     auto issue = [&](int kt, int so) {
         unsigned char *base = smem + so;
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-            __builtin_amdgcn_global_load_lds((gptr)(ga[i] + kt * BK), (lptr)(base + (wave * 4 + i) * 1024), 16, 0, 0);
+        for (int i = 0; i < AL; ++i)
+            __builtin_amdgcn_global_load_lds((gptr)(ga[i] + kt * BK), (lptr)(base + (wave * AL + i) * 1024), 16, 0, 0);
 #pragma unroll
         for (int i = 0; i < WL; ++i)
             __builtin_amdgcn_global_load_lds((gptr)(gw[i] + kt * BK * (W_U8 ? 1 : 2)), (lptr)(base + D_A + (wave * WL + i) * 1024), 16, 0, 0);
     };
 
-    f32x16 acc[4][2];
+    f32x16 acc[MI][NI];
 #pragma unroll
-    for (int a = 0; a < 4; ++a)
+    for (int a = 0; a < MI; ++a)
 #pragma unroll
-        for (int b = 0; b < 2; ++b)
+        for (int b = 0; b < NI; ++b)
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[a][b][e] = 0.f;
 
@@ -344,36 +351,38 @@ DEV void gemm_dma_body(int T, int N, int M, const h16 *__restrict__ A, int64_t l
     uint32_t vA[4], vB[4];
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
-        vA[ks] = lds0 + (wr * 128 + (lane & 31)) * 128 + (((2 * ks + (lane >> 5)) ^ ((lane >> 1) & 7)) << 4);
-        if (W_U8) vB[ks] = lds0 + D_A + (wc * 64 + (lane & 31)) * 64 + ((ks ^ ((lane >> 2) & 3)) << 4) + (lane >> 5) * 8;
-        else vB[ks] = lds0 + D_A + (wc * 64 + (lane & 31)) * 128 + (((2 * ks + (lane >> 5)) ^ ((lane >> 1) & 7)) << 4);
+        vA[ks] = lds0 + (wr * 32 * MI + (lane & 31)) * 128 + (((2 * ks + (lane >> 5)) ^ ((lane >> 1) & 7)) << 4);
+        if (W_U8) vB[ks] = lds0 + D_A + (wc * 32 * NI + (lane & 31)) * 64 + ((ks ^ ((lane >> 2) & 3)) << 4) + (lane >> 5) * 8;
+        else vB[ks] = lds0 + D_A + (wc * 32 * NI + (lane & 31)) * 128 + (((2 * ks + (lane >> 5)) ^ ((lane >> 1) & 7)) << 4);
     }
-    h16x8 fa[2][4], fbh[2][2];   // fbh: B fragments of fp16 weights
-    u32x2 rawb[2][2];            // B fragments of uint8 weights, before conversion
+    h16x8 fa[2][MI], fbh[2][NI];   // fbh: B fragments of fp16 weights
+    u32x2 rawb[2][NI];             // B fragments of uint8 weights, before conversion
     auto ldfrag = [&](int buf, int so, int ks) {
         const uint32_t pa = vA[ks] + so, pb = vB[ks] + so;
         if constexpr (W_U8) {
             asm volatile("ds_read_b64 %0, %1" : "=v"(rawb[buf][0]) : "v"(pb));
-            asm volatile("ds_read_b64 %0, %1 offset:2048" : "=v"(rawb[buf][1]) : "v"(pb));
+            if constexpr (NI > 1) asm volatile("ds_read_b64 %0, %1 offset:2048" : "=v"(rawb[buf][NI > 1 ? 1 : 0]) : "v"(pb));
         } else {
             asm volatile("ds_read_b128 %0, %1" : "=v"(fbh[buf][0]) : "v"(pb));
-            asm volatile("ds_read_b128 %0, %1 offset:4096" : "=v"(fbh[buf][1]) : "v"(pb));
+            if constexpr (NI > 1) asm volatile("ds_read_b128 %0, %1 offset:4096" : "=v"(fbh[buf][NI > 1 ? 1 : 0]) : "v"(pb));
         }
         asm volatile("ds_read_b128 %0, %1" : "=v"(fa[buf][0]) : "v"(pa));
         asm volatile("ds_read_b128 %0, %1 offset:4096" : "=v"(fa[buf][1]) : "v"(pa));
-        asm volatile("ds_read_b128 %0, %1 offset:8192" : "=v"(fa[buf][2]) : "v"(pa));
-        asm volatile("ds_read_b128 %0, %1 offset:12288" : "=v"(fa[buf][3]) : "v"(pa));
+        if constexpr (MI > 2) {
+            asm volatile("ds_read_b128 %0, %1 offset:8192" : "=v"(fa[buf][MI > 2 ? 2 : 0]) : "v"(pa));
+            asm volatile("ds_read_b128 %0, %1 offset:12288" : "=v"(fa[buf][MI > 2 ? 3 : 0]) : "v"(pa));
+        }
     };
     const h16x2 off = {(h16)1023.5f, (h16)1023.5f};
-    // waits until at most `newer` of this wave's LDS reads are outstanding, i.e. the six before them have returned
-    auto older_reads_done = [&](int newer) {
-        if (newer) __builtin_amdgcn_s_waitcnt(0xC67F); else __builtin_amdgcn_s_waitcnt(0xC07F);   // lgkmcnt(6) / lgkmcnt(0)
+    // waits until only the newest fragment set (MI + NI reads) of this wave is outstanding: the one before has returned
+    auto older_reads_done = [&]() {
+        __builtin_amdgcn_s_waitcnt(lgkm_only(MI + NI));
         __builtin_amdgcn_sched_barrier(0);
     };
     auto multiply = [&](int cur) {
-        h16x8 fb[2];
+        h16x8 fb[NI];
 #pragma unroll
-        for (int b = 0; b < 2; ++b) {
+        for (int b = 0; b < NI; ++b) {
             if constexpr (W_U8) {
                 const u32x2 raw = rawb[cur][b];
                 const h16x2 q0 = u8pair_lo_1024(raw.x) - off, q1 = u8pair_hi_1024(raw.x) - off;
@@ -384,9 +393,9 @@ DEV void gemm_dma_body(int T, int N, int M, const h16 *__restrict__ A, int64_t l
             }
         }
 #pragma unroll
-        for (int a = 0; a < 4; ++a)
+        for (int a = 0; a < MI; ++a)
 #pragma unroll
-            for (int b = 0; b < 2; ++b) acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[cur][a], fb[b], acc[a][b], 0, 0, 0);
+            for (int b = 0; b < NI; ++b) acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[cur][a], fb[b], acc[a][b], 0, 0, 0);
         __builtin_amdgcn_sched_barrier(0);
     };
 
@@ -403,15 +412,15 @@ DEV void gemm_dma_body(int T, int N, int M, const h16 *__restrict__ A, int64_t l
         const int sn = so + D_STAGE >= D_NST * D_STAGE ? 0 : so + D_STAGE;
         ldfrag(1, so, 1);
         __builtin_amdgcn_sched_barrier(0);
-        older_reads_done(6);
+        older_reads_done();
         multiply(0);
         ldfrag(0, so, 2);
         __builtin_amdgcn_sched_barrier(0);
-        older_reads_done(6);
+        older_reads_done();
         multiply(1);
         ldfrag(1, so, 3);
         __builtin_amdgcn_sched_barrier(0);
-        older_reads_done(6);
+        older_reads_done();
         multiply(0);
         // all my reads of this stage have returned and my part of tile kt + 1 has landed (with three stages tile
         // kt + 2 may be in flight)
@@ -428,7 +437,8 @@ DEV void gemm_dma_body(int T, int N, int M, const h16 *__restrict__ A, int64_t l
     // Each thread finishes eight consecutive outputs of one row: 16-byte loads of the residual / gate rows, 16-byte
     // stores, and a body small enough to stay in the instruction cache (per-element code for 128 accumulators
     // does not).
-    const int cq = tid & 31, col = m0 + cq * 8;
+    constexpr int CPR = TN / 8, RPI = 512 / CPR;   // 8-wide chunks per tile row; rows one pass of the workgroup covers
+    const int cq = tid % CPR, col = m0 + cq * 8;
     const bool col_ok = col < M;   // M % 8 == 0
     h16x8 rx8, mx8;
     if (W_U8 && col_ok) { rx8 = *(const h16x8 *)(ep.rx + col); mx8 = *(const h16x8 *)(ep.mx + col); }
@@ -466,36 +476,38 @@ DEV void gemm_dma_body(int T, int N, int M, const h16 *__restrict__ A, int64_t l
         // partial sums go to this split's fp32 slab; splitk_epilogue_kernel adds the slabs and finishes
         float *slab = part + (size_t)split * T * M;
 #pragma unroll
-        for (int b = 0; b < 2; ++b) {
-            const int m = m0 + wc * 64 + b * 32 + (lane & 31);
+        for (int b = 0; b < NI; ++b) {
+            const int m = m0 + wc * 32 * NI + b * 32 + (lane & 31);
 #pragma unroll
-            for (int a = 0; a < 4; ++a)
+            for (int a = 0; a < MI; ++a)
 #pragma unroll
                 for (int e = 0; e < 16; ++e) {
-                    const int t = t0 + wr * 128 + a * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
+                    const int t = t0 + wr * 32 * MI + a * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
                     if (m < M && t < T) slab[(size_t)t * M + m] = acc[a][b][e];
                 }
         }
     } else {
-        // The accumulators pass through LDS (free now), 128 rows at a time.
+        // The accumulators pass through LDS (free now), 128 tile rows at a time.
         constexpr int SW = Cfg::STG_STRIDE;   // row stride in floats: 4 rows apart = 32 banks apart for the two half-waves
+        constexpr int WROWS = 32 * MI;        // tile rows of one wave row
         float *stg = (float *)smem;
         __syncthreads();   // every wave has read its last fragments
 #pragma unroll 1
-        for (int h = 0; h < 2; ++h) {
-            if (wr == h) {
+        for (int h = 0; h < TM / 128; ++h) {
+            if ((wr * WROWS) / 128 == h) {
 #pragma unroll
-                for (int b = 0; b < 2; ++b)
+                for (int b = 0; b < NI; ++b)
 #pragma unroll
-                    for (int a = 0; a < 4; ++a)
+                    for (int a = 0; a < MI; ++a)
 #pragma unroll
                         for (int e = 0; e < 16; ++e)
-                            stg[(a * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3)) * SW + wc * 64 + b * 32 + (lane & 31)] = acc[a][b][e];
+                            stg[(wr * WROWS - h * 128 + a * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3)) * SW + wc * 32 * NI + b * 32 + (lane & 31)] =
+                                acc[a][b][e];
             }
             __syncthreads();
 #pragma unroll 1
-            for (int it = 0; it < 8; ++it) {
-                const int row = it * 16 + (tid >> 5), t = t0 + h * 128 + row;
+            for (int it = 0; it < 128 / RPI; ++it) {
+                const int row = it * RPI + tid / CPR, t = t0 + h * 128 + row;
                 if (t < T && col_ok) {
                     const f32x4 v0 = *(const f32x4 *)(stg + row * SW + cq * 8), v1 = *(const f32x4 *)(stg + row * SW + cq * 8 + 4);
                     float v[8] = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
@@ -507,11 +519,11 @@ DEV void gemm_dma_body(int T, int N, int M, const h16 *__restrict__ A, int64_t l
     }
 }
 
-template <bool W_U8, bool SPLIT>
+template <bool W_U8, bool SPLIT, int TM, int TN>
 __global__ __launch_bounds__(512) void gemm_dma_kernel(int T, int N, int M, const h16 *__restrict__ A, int64_t lda,
                                                        const void *__restrict__ W, int64_t ldw, void *__restrict__ Y,
                                                        int64_t ldy, GemmEpi ep, int nk_split, float *__restrict__ part) {
-    gemm_dma_body<W_U8, SPLIT>(T, N, M, A, lda, W, ldw, Y, ldy, ep, nk_split, part, SPLIT ? blockIdx.y : 0);
+    gemm_dma_body<W_U8, SPLIT, TM, TN>(T, N, M, A, lda, W, ldw, Y, ldy, ep, nk_split, part, SPLIT ? blockIdx.y : 0);
 }
 
 // Up to four contractions [T, N] x [N, M_i] in one launch (blockIdx.y picks the operands), at full depth: short
@@ -535,11 +547,30 @@ __global__ __launch_bounds__(64 * WT * WM) void gemm_group_kernel(int T, int N, 
 }
 
 // the same through the direct-to-LDS kernel; blockIdx.z is the k split when the group has too few tiles for the chip
-template <bool W_U8, bool SPLIT>
+template <bool W_U8, bool SPLIT, int TM, int TN>
 __global__ __launch_bounds__(512) void gemm_dma_group_kernel(int T, int N, GemmGroup g) {
     const int gi = blockIdx.y, M = g.M[gi];
-    gemm_dma_body<W_U8, SPLIT>(T, N, M, g.A[gi], g.lda, g.W[gi], g.ldw[gi], g.Y[gi], M, g.ep[gi], SPLIT ? g.nk_split : N / BK,
-                               g.part[gi], SPLIT ? blockIdx.z : 0);
+    gemm_dma_body<W_U8, SPLIT, TM, TN>(T, N, M, g.A[gi], g.lda, g.W[gi], g.ldw[gi], g.Y[gi], M, g.ep[gi], SPLIT ? g.nk_split : N / BK,
+                                       g.part[gi], SPLIT ? blockIdx.z : 0);
+}
+
+template <bool W_U8, int TM, int TN>
+int launch_dma_group(const GemmGroup &g, int n, int64_t T, int64_t N, int64_t grid_x, int ks, hipStream_t st) {
+    constexpr size_t lds = DmaCfg<W_U8, TM, TN>::LDS;
+    static bool attr_done = false;
+    if (!attr_done) {
+        hipError_t e = hipFuncSetAttribute((const void *)gemm_dma_group_kernel<W_U8, false, TM, TN>,
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e == hipSuccess)
+            e = hipFuncSetAttribute((const void *)gemm_dma_group_kernel<W_U8, true, TM, TN>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    (int)lds);
+        if (e != hipSuccess) return (int)e;
+        attr_done = true;
+    }
+    const dim3 grid((unsigned)grid_x, (unsigned)n, (unsigned)ks);
+    if (ks > 1) hipLaunchKernelGGL((gemm_dma_group_kernel<W_U8, true, TM, TN>), grid, dim3(512), lds, st, (int)T, (int)N, g);
+    else hipLaunchKernelGGL((gemm_dma_group_kernel<W_U8, false, TM, TN>), grid, dim3(512), lds, st, (int)T, (int)N, g);
+    return RWKV_OK;
 }
 
 // second pass of a split group: member blockIdx.y, as splitk_epilogue_kernel
@@ -684,49 +715,57 @@ bool dma_ok(bool w_u8, int64_t N, int64_t M, const void *A, int64_t lda, const v
     return true;
 }
 
-// K split of a direct-to-LDS launch with `tiles` 256 x 256 tiles of nk k-tiles each: whole rounds over the 256 CUs
-// cost their k-tiles plus about six k-tile times of fill and drain, and every split adds a slab to write and read
-// back (about one and a half k-tile times).  1 where the tiles fill the chip anyway.
-int dma_split(int64_t tiles, int nk, size_t out_bytes, size_t ws_bytes) {
-    if (tiles >= 192) return 1;
+// Cost model of a direct-to-LDS launch, in units of one k-tile step of a 256 x 256 tile (about 2.2 us): `tiles` tiles of
+// nk k-tiles split c ways run in whole rounds over the 256 CUs, each round costs its k-tiles plus a few k-tile times
+// of fill and drain, and every split adds a slab to write and read back.  A 128 x 128 tile does a quarter of the work
+// per step in 0.3 of the time.
+double dma_cost(int64_t tiles, int nk, int c, bool small_tile, size_t out_bytes) {
+    const double rounds = (double)((tiles * c + 255) / 256);
+    const double loop = rounds * (nk / c + (small_tile ? 8 : 6)) * (small_tile ? 0.3 : 1.0);
+    return loop + (c > 1 ? 2.4 * c * (double)out_bytes / (16 << 20) : 0.0);
+}
+
+// the K split (1..8, whole k-tiles, at least 8 per split, slabs within ws_bytes) of least cost
+int dma_split(int64_t tiles, int nk, bool small_tile, size_t out_bytes, size_t ws_bytes, double *cost = nullptr) {
     int best = 1;
     double best_cost = 1e30;
     for (int c = 1; c <= 8; ++c) {
         if (nk % c || (c > 1 && nk / c < 8) || (c > 1 && c * out_bytes > ws_bytes)) continue;
-        const double cost = (double)((tiles * c + 255) / 256) * (nk / c + 6) + (c > 1 ? 1.5 * c : 0.0);
-        if (cost < best_cost) { best_cost = cost; best = c; }
+        const double k = dma_cost(tiles, nk, c, small_tile, out_bytes);
+        if (k < best_cost) { best_cost = k; best = c; }
     }
+    if (cost) *cost = best_cost;
     return best;
 }
 
 // gemm_dma_kernel.  Fewer than 192 tiles (narrow outputs): the contraction is split over workgroups of the same
 // tile until about one workgroup per CU is in flight; slabs and the second pass as in launch_cfg.
-template <bool W_U8>
+template <bool W_U8, int TM, int TN>
 int launch_dma(int64_t T, int64_t N, int64_t M, const rwkv_half *A, int64_t lda, const void *W, int64_t ldw, void *Y,
                int64_t ldy, const GemmEpi &ep, hipStream_t st) {
-    constexpr size_t lds = DmaCfg<W_U8>::LDS;
+    constexpr size_t lds = DmaCfg<W_U8, TM, TN>::LDS;
     static bool attr_done = false;
     if (!attr_done) {
-        hipError_t e = hipFuncSetAttribute((const void *)gemm_dma_kernel<W_U8, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        hipError_t e = hipFuncSetAttribute((const void *)gemm_dma_kernel<W_U8, false, TM, TN>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e == hipSuccess)
-            e = hipFuncSetAttribute((const void *)gemm_dma_kernel<W_U8, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            e = hipFuncSetAttribute((const void *)gemm_dma_kernel<W_U8, true, TM, TN>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return (int)e;
         attr_done = true;
     }
     if (!dma_ok(W_U8, N, M, A, lda, W, ldw, Y, ldy, ep)) return RWKV_E_LAYOUT;
-    const int64_t tiles = ((T + DT - 1) / DT) * ((M + DM - 1) / DM);
+    const int64_t tiles = ((T + TM - 1) / TM) * ((M + TN - 1) / TN);
     const int nk = (int)(N / BK);
     int ks = 1;
-    if (ep.splitk_ws && (M & 3) == 0) ks = dma_split(tiles, nk, (size_t)T * M * sizeof(float), ep.splitk_bytes);
+    if (ep.splitk_ws && (M & 3) == 0) ks = dma_split(tiles, nk, TM < 256, (size_t)T * M * sizeof(float), ep.splitk_bytes);
     if (ks > 1) {
-        hipLaunchKernelGGL((gemm_dma_kernel<W_U8, true>), dim3((unsigned)tiles, (unsigned)ks), dim3(512), lds, st, (int)T, (int)N, (int)M,
-                           (const h16 *)A, lda, W, ldw, Y, ldy, ep, nk / ks, ep.splitk_ws);
+        hipLaunchKernelGGL((gemm_dma_kernel<W_U8, true, TM, TN>), dim3((unsigned)tiles, (unsigned)ks), dim3(512), lds, st, (int)T, (int)N,
+                           (int)M, (const h16 *)A, lda, W, ldw, Y, ldy, ep, nk / ks, ep.splitk_ws);
         const int64_t n = T * M;
         const unsigned blocks = (unsigned)((n + 1023) / 1024 < 16384 ? (n + 1023) / 1024 : 16384);
         hipLaunchKernelGGL(splitk_epilogue_kernel, dim3(blocks), dim3(256), 0, st, (int)T, (int)M, ks, ep.splitk_ws, Y, ldy, ep);
     } else {
-        hipLaunchKernelGGL((gemm_dma_kernel<W_U8, false>), dim3((unsigned)tiles), dim3(512), lds, st, (int)T, (int)N, (int)M, (const h16 *)A,
-                           lda, W, ldw, Y, ldy, ep, nk, (float *)nullptr);
+        hipLaunchKernelGGL((gemm_dma_kernel<W_U8, false, TM, TN>), dim3((unsigned)tiles), dim3(512), lds, st, (int)T, (int)N, (int)M,
+                           (const h16 *)A, lda, W, ldw, Y, ldy, ep, nk, (float *)nullptr);
     }
     RWKV_LAUNCH_CHECK();
     return RWKV_OK;
@@ -740,32 +779,40 @@ int launch_pick(int cfg, int64_t T, int64_t N, int64_t M, const rwkv_half *A, in
         case 9:
             if constexpr (W_U8) return launch_cfg<true, 256, 256, 4, 4, 2>(T, N, M, A, lda, W, ldw, Y, ldy, ep, st);
             return RWKV_E_DTYPE;
-        case 14: return launch_dma<W_U8>(T, N, M, A, lda, W, ldw, Y, ldy, ep, st);
+        case 14: return launch_dma<W_U8, 256, 256>(T, N, M, A, lda, W, ldw, Y, ldy, ep, st);
+        case 15: return launch_dma<W_U8, 128, 128>(T, N, M, A, lda, W, ldw, Y, ldy, ep, st);
         default: return RWKV_E_DTYPE;
     }
 }
 
 // Tile choice (RWKV_GEMM_CFG overrides it for tuning sweeps).
-//   14  512 rows or more and an output of 3 M elements or more, operands laid out for 16-byte loads, no other product
-//       running beside this one: the direct-to-LDS kernel (256 x 256 tiles; it splits K itself when there are few tiles)
-//    9  uint8 weights otherwise, where 256 x 256 tiles of the register-staged kernel fill the chip: one per CU and
-//       round, the last round at least 70 % full
-//    3  everything else: 128 x 128 tiles, 4 k-tiles of prefetch
-int pick_cfg(int64_t T, int64_t M, bool w_u8, bool alone, bool dma) {
+//   14 / 15  operands laid out for 16-byte loads: the direct-to-LDS kernel with 256 x 256 or 128 x 128 tiles,
+//            whichever the cost model puts first (large tiles where they fill the chip, small ones at full depth
+//            where the large ones would have to split K; small ones when another product runs beside this one)
+//    9       uint8 weights otherwise, where 256 x 256 tiles of the register-staged kernel fill the chip: one per CU
+//            and round, the last round at least 70 % full
+//    3       everything else: 128 x 128 tiles, 4 k-tiles of prefetch
+int pick_cfg(int64_t T, int64_t N, int64_t M, bool w_u8, bool alone, bool dma, bool can_split) {
     const char *e = getenv("RWKV_GEMM_CFG");  // tuning override
     if (e && *e) return atoi(e);
-    if (!alone) return 3;   // a 256 x 256 tile's LDS leaves no room beside it on the CU
+    if (!alone) return dma ? 15 : 3;   // a 256 x 256 tile's LDS leaves no room beside it on the CU, two small ones fit
+    if (dma) {
+        const int nk = (int)(N / BK);
+        const size_t out_bytes = (size_t)T * M * sizeof(float), ws = can_split && !(M & 3) ? RWKV_SPLITK_WS_BYTES : 0;
+        double c14, c15;
+        dma_split(((T + 255) / 256) * ((M + 255) / 256), nk, false, out_bytes, ws, &c14);
+        dma_split(((T + 127) / 128) * ((M + 127) / 128), nk, true, out_bytes, ws, &c15);
+        return c14 <= c15 ? 14 : 15;
+    }
     const int64_t big = ((T + 255) / 256) * ((M + 255) / 256), rounds = (big + 255) / 256;
-    const bool fills = big * 10 >= rounds * 256 * 7;
-    if (dma && T >= 512 && T * M >= ((int64_t)3 << 20) && (big < 192 || fills)) return 14;
-    return w_u8 && fills ? 9 : 3;   // fp16 weight tiles are twice the bytes: the register-staged large tile spills
+    return w_u8 && big * 10 >= rounds * 256 * 7 ? 9 : 3;   // fp16 weight tiles are twice the bytes: the large tile spills
 }
 
 }  // namespace
 
 int gemm_launch(bool w_u8, int64_t T, int64_t N, int64_t M, const rwkv_half *A, int64_t lda, const void *W,
                 int64_t ldw, void *Y, int64_t ldy, const GemmEpi &ep, hipStream_t st) {
-    const int cfg = pick_cfg(T, M, w_u8, !ep.small_tiles, dma_ok(w_u8, N, M, A, lda, W, ldw, Y, ldy, ep));
+    const int cfg = pick_cfg(T, N, M, w_u8, !ep.small_tiles, dma_ok(w_u8, N, M, A, lda, W, ldw, Y, ldy, ep), ep.splitk_ws != nullptr);
     return w_u8 ? launch_pick<true>(cfg, T, N, M, A, lda, W, ldw, Y, ldy, ep, st)
                 : launch_pick<false>(cfg, T, N, M, A, lda, W, ldw, Y, ldy, ep, st);
 }
@@ -782,8 +829,8 @@ int mm8_prepare_launch(int64_t T, int64_t N, const rwkv_half *x, int64_t ldx, co
 // n (2..4) products [T, N] x [N, M_i] of uint8 or fp16 weights with their own inputs, outputs and epilogues in one
 // launch.  uint8 with xs != NULL: x[i] is the unscaled activation and xs[i] / sums[i] (2 T floats) are scratch;
 // uint8 with xs == NULL: x[i] is already scaled by ry and sums[i] holds its row sums.
-// Calls of 256 rows or more go through the direct-to-LDS kernel (splitting K over splitk_ws, RWKV_SPLITK_WS_BYTES of
-// scratch or NULL, while the group has fewer than 192 tiles), shorter ones through 128 x 128 tiles at full depth.
+// Operands laid out for 16-byte loads: the direct-to-LDS kernel, tile size and K split (over splitk_ws,
+// RWKV_SPLITK_WS_BYTES of scratch, or NULL) from the cost model; otherwise register-staged 128 x 128 tiles at full depth.
 int gemm_group_launch(bool w_u8, int n, int64_t T, int64_t N, const rwkv_half *const *x, const rwkv_mat *const *mats,
                       void *const *Y, const GemmEpi *eps, rwkv_half *const *xs, float *const *sums, float *splitk_ws,
                       hipStream_t st) {
@@ -798,8 +845,8 @@ int gemm_group_launch(bool w_u8, int n, int64_t T, int64_t N, const rwkv_half *c
         }
         hipLaunchKernelGGL(mm8_prepare_group_kernel, dim3((unsigned)((T + 3) / 4), (unsigned)n), dim3(256), 0, st, (int)T, (int)N, p);
     }
-    int64_t tiles = 0, tiles_dma = 0, total_dma = 0, out_elems = 0, max_out = 0;
-    bool dma = T >= 256, m4 = true;
+    int64_t tiles = 0, tiles_big = 0, total_big = 0, total_small = 0, out_elems = 0, max_out = 0;
+    bool dma = true, m4 = true;
     for (int i = 0; i < n; ++i) {
         if (mats[i]->N != N) return RWKV_E_SHAPE;
         g.A[i] = (const h16 *)(prep ? xs[i] : x[i]);
@@ -807,41 +854,34 @@ int gemm_group_launch(bool w_u8, int n, int64_t T, int64_t N, const rwkv_half *c
         g.ep[i] = eps[i];
         g.ep[i].ldres = g.ep[i].ldgate = mats[i]->M;
         if (w_u8) { g.ep[i].mx = mats[i]->mx; g.ep[i].rx = mats[i]->rx; g.ep[i].s0 = sums[i]; g.ep[i].s2 = sums[i] + T; }
-        tiles = std::max<int64_t>(tiles, ((T + 127) / 128) * ((mats[i]->M + 127) / 128));
-        const int64_t td = ((T + DT - 1) / DT) * ((mats[i]->M + DM - 1) / DM);
-        tiles_dma = std::max(tiles_dma, td);
-        total_dma += td;
+        const int64_t ts = ((T + 127) / 128) * ((mats[i]->M + 127) / 128), tb = ((T + DT - 1) / DT) * ((mats[i]->M + DM - 1) / DM);
+        tiles = std::max(tiles, ts);
+        tiles_big = std::max(tiles_big, tb);
+        total_small += ts;
+        total_big += tb;
         out_elems += T * mats[i]->M;
         max_out = std::max<int64_t>(max_out, T * mats[i]->M);
         m4 = m4 && !(mats[i]->M & 3);
         dma = dma && dma_ok(w_u8, N, mats[i]->M, g.A[i], N, g.W[i], g.ldw[i], g.Y[i], mats[i]->M, g.ep[i]);
     }
     if (dma) {
-        static bool attr_done = false;
-        if (!attr_done) {
-            const void *fn[4] = {(const void *)gemm_dma_group_kernel<true, false>, (const void *)gemm_dma_group_kernel<true, true>,
-                                 (const void *)gemm_dma_group_kernel<false, false>, (const void *)gemm_dma_group_kernel<false, true>};
-            for (int i = 0; i < 4; ++i) {
-                hipError_t e = hipFuncSetAttribute(fn[i], hipFuncAttributeMaxDynamicSharedMemorySize,
-                                                   (int)(i < 2 ? DmaCfg<true>::LDS : DmaCfg<false>::LDS));
-                if (e != hipSuccess) return (int)e;
-            }
-            attr_done = true;
-        }
+        // tile size and K split of least cost, as for a single product
         const int nk = (int)(N / BK);
-        int ks = 1;
-        if (splitk_ws && m4) ks = dma_split(total_dma, nk, (size_t)out_elems * sizeof(float), RWKV_SPLITK_WS_BYTES);
+        const size_t out_bytes = (size_t)out_elems * sizeof(float), ws = splitk_ws && m4 ? RWKV_SPLITK_WS_BYTES : 0;
+        double c_big, c_small;
+        const int ks_big = dma_split(total_big, nk, false, out_bytes, ws, &c_big);
+        const int ks_small = dma_split(total_small, nk, true, out_bytes, ws, &c_small);
+        const bool big = c_big <= c_small;
+        const int ks = big ? ks_big : ks_small;
         g.nk_split = nk / ks;
         if (ks > 1) {
             float *p = splitk_ws;
             for (int i = 0; i < n; ++i) { g.part[i] = p; p += (size_t)ks * T * mats[i]->M; }
         }
-        const dim3 grid((unsigned)tiles_dma, (unsigned)n, (unsigned)ks);
-        const size_t lds = w_u8 ? DmaCfg<true>::LDS : DmaCfg<false>::LDS;
-        if (w_u8 && ks > 1) hipLaunchKernelGGL((gemm_dma_group_kernel<true, true>), grid, dim3(512), lds, st, (int)T, (int)N, g);
-        else if (w_u8) hipLaunchKernelGGL((gemm_dma_group_kernel<true, false>), grid, dim3(512), lds, st, (int)T, (int)N, g);
-        else if (ks > 1) hipLaunchKernelGGL((gemm_dma_group_kernel<false, true>), grid, dim3(512), lds, st, (int)T, (int)N, g);
-        else hipLaunchKernelGGL((gemm_dma_group_kernel<false, false>), grid, dim3(512), lds, st, (int)T, (int)N, g);
+        int rc;
+        if (big) rc = w_u8 ? launch_dma_group<true, DT, DM>(g, n, T, N, tiles_big, ks, st) : launch_dma_group<false, DT, DM>(g, n, T, N, tiles_big, ks, st);
+        else rc = w_u8 ? launch_dma_group<true, 128, 128>(g, n, T, N, tiles, ks, st) : launch_dma_group<false, 128, 128>(g, n, T, N, tiles, ks, st);
+        if (rc) return rc;
         if (ks > 1) {
             const unsigned blocks = (unsigned)std::min<int64_t>((max_out + 1023) / 1024, 16384);
             hipLaunchKernelGGL(splitk_group_epilogue_kernel, dim3(blocks, (unsigned)n), dim3(256), 0, st, (int)T, ks, g);

@@ -305,14 +305,15 @@ extern "C" int rwkv_v4_forward_seq(const rwkv_v4_model *m, const rwkv_v4_layer_s
         // long calls: every product through the direct-to-LDS kernel, one after the other (its tiles take a whole
         // CU, so products side by side on several streams gain nothing); k, v, r as one group
         const bool dma_seq = T >= 512;
-        const bool group_kvr = T >= 256;   // from 256 rows on the group goes through that kernel too, splitting K
+        const bool group_kvr = true;       // k, v, r as one grouped launch at every length (tile size and K split by cost)
         const bool par = ss && !group_kvr && (T / 128) * (C / 128) > 128 && fork_streams(ss, st, 2);
         if (group_kvr) {
             const rwkv_half *xin[3] = {ws.xs[0], ws.xs[1], ws.xs[2]};
             const rwkv_mat *mats[3] = {&l.att_key, &l.att_value, &l.att_receptance};
             void *outs[3] = {ws.k, ws.v, ws.r};
             GemmEpi ep[3] = {e, e, e};
-            ep[2].act = ACT_SIGMOID; ep[2].out_dtype = RWKV_DT_F16; ep[2].raw_f32 = 0;
+            e.act = ACT_SIGMOID; e.out_dtype = RWKV_DT_F16; e.raw_f32 = 0;   // receptance, and every product after it
+            ep[2] = e;
             if ((rc = gemm_group_launch(u8, 3, T, C, xin, mats, outs, ep, nullptr, s0, ws.splitk, st))) return rc;
         } else {
         hipStream_t sv = par ? ss->s[0] : st, sr = par ? ss->s[1] : st;

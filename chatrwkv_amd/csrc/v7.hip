@@ -584,7 +584,7 @@ extern "C" int rwkv_v7_forward(const rwkv_v7_model *m, const rwkv_v56_layer_stat
         // key and value are one grouped launch of the direct-to-LDS kernel; where that group fills three quarters
         // of the chip without splitting K, the eight small LoRA products (which do split K: one user of the split-K
         // scratch at a time) run beside it on a side stream, on the CUs the group leaves free.
-        const bool dma_seq = T >= 256;
+        const bool dma_seq = true;
         const bool par = ss && dma_seq && 3 * ((T + 255) / 256) * ((C + 255) / 256) >= 192 && fork_streams(ss, st, 1);
         Ctx cm = c, cv = c, cl = c;
         if (par) cl.st = ss->s[0];

@@ -485,15 +485,18 @@ def test_7b_shape_properties():
         tok = int(out.argmax())
 
 
-@pytest.mark.parametrize("kind", ["v6", "v7"])
+@pytest.mark.parametrize("kind", ["v6", "v7", "v4-fp16"])
 def test_7b_shape_properties_v6_v7(kind):
-    """Two layers of the RWKV-6 ('cuda fp16i8') and RWKV-7 ('cuda fp16') 7B shapes (n_embd 4096, 64 heads, vocab
-    65536): a 1024-token prompt in one call and in calls of 256 agrees within the fp16 tolerance, and the
-    one-token graph replay equals the direct launch bit for bit."""
+    """Two layers of the RWKV-6 ('cuda fp16i8'), RWKV-7 ('cuda fp16') and RWKV-4 ('cuda fp16') 7B shapes (n_embd
+    4096, 64 heads, vocab 65536): a 1024-token prompt in one call and in calls of 256 agrees within the fp16
+    tolerance, and the one-token graph replay equals the direct launch bit for bit."""
     V = 65536
     if kind == "v6":
         ck = synth.make_checkpoint(version=6, n_layer=2, n_embd=4096, n_ffn=14336, vocab=V, seed=5, device="cuda:0")
         m = _rwkv()(ck, "cuda fp16i8", verbose=False)
+    elif kind == "v4-fp16":
+        ck = synth.make_checkpoint(version=4, n_layer=2, n_embd=4096, n_ffn=16384, vocab=V, seed=5, device="cuda:0")
+        m = _rwkv()(ck, "cuda fp16", verbose=False)
     else:
         from chatrwkv_amd.model_v7 import RWKV_x070
         ck = synth.make_checkpoint_v7(n_layer=2, n_embd=4096, n_ffn=16384, vocab=V, seed=5, device="cuda:0")
