@@ -355,12 +355,22 @@ extern "C" int rwkv_v4_forward_seq(const rwkv_v4_model *m, const rwkv_v4_layer_s
         e.act = ACT_SIGMOID;
         const bool par2 = ss && !dma_seq && (T / 128) * (C / 128) > 128 && fork_streams(ss, st, 1);
         float *sk2 = par2 ? nullptr : ws.splitk;
+        if (T <= 128 && !(C & 127) && !(F & 127)) {
+            // short calls: receptance and key in one grouped launch
+            const rwkv_half *xin[2] = {ws.xs[0], ws.xs[1]};
+            const rwkv_mat *mats[2] = {&l.ffn_receptance, &l.ffn_key};
+            void *outs[2] = {ws.r, ws.vx};
+            GemmEpi ep[2] = {e, e};
+            ep[1].act = ACT_RELU_SQ;
+            if ((rc = gemm_group_launch(u8, 2, T, C, xin, mats, outs, ep, nullptr, s0, ws.splitk, st))) return rc;
+        } else {
         if ((rc = run_gemm(l.ffn_receptance, u8, T, ws.xs[0], s0[0], s2[0], ws.r, C, e, par2 ? ss->s[0] : st, sk2))) return rc;
         e.act = ACT_RELU_SQ;
         e.small_tiles = par2 ? 1 : 0;   // the receptance product runs beside this one
         if ((rc = run_gemm(l.ffn_key, u8, T, ws.xs[1], s0[1], s2[1], ws.vx, F, e, st, sk2))) return rc;
         e.small_tiles = 0;
         if (par2 && !join_streams(ss, st, 1)) return (int)hipErrorUnknown;
+        }
         const rwkv_half *a_v = ws.vx;
         if (u8) {
             if ((rc = mm8_prepare_launch(T, F, ws.vx, F, l.ffn_value.ry, l.ffn_value.my, ws.xsv, s0v, s2v, st))) return rc;

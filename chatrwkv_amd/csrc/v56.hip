@@ -345,8 +345,8 @@ extern "C" int rwkv_v56_forward(const rwkv_v56_model *m, const rwkv_v56_layer_st
             for (int j = 0; j < 2; ++j) { a.ry[j] = nullptr; a.my[j] = nullptr; a.xs[j] = ws.mix[j]; }
             if ((rc = lnmix_seq_launch(a, 2, st))) return rc;
         }
-        if (!ss && ((T + 127) / 128) * (C / 128) <= 128 && ((T + 127) / 128) * (F / 128) <= 256 && !(C & 127) && !(F & 127)) {
-            // short calls: receptance and key in one grouped launch at full depth
+        if (T <= 128 && !(C & 127) && !(F & 127)) {
+            // short calls: receptance and key in one grouped launch (measured: +7 % at 64 rows, -5 % at 256)
             const rwkv_half *xin[2] = {ws.mix[0], ws.mix[1]};
             const rwkv_mat *mats[2] = {&l.ffn_receptance, &l.ffn_key};
             void *outs[2] = {ws.r, ws.vx};
