@@ -99,7 +99,9 @@ def test_mm8_one(N, M):
 @pytest.mark.parametrize("N,M,B", [(768, 768, 2), (768, 3072, 5), (3072, 768, 128), (768, 50277, 3),
                                    (2560, 2560, 200), (4096, 4096, 1024), (4096, 16384, 256), (16384, 4096, 130),
                                    # long calls: 256 x 256 tiles loaded straight into LDS; whole, ragged and split-K
-                                   (4096, 8192, 1000), (16384, 4096, 520), (2560, 10240, 768)])
+                                   (4096, 8192, 1000), (16384, 4096, 520), (2560, 10240, 768),
+                                   # ragged tiles of the direct-to-LDS kernel: widths and row counts that end inside a tile
+                                   (128, 200, 37), (192, 1000, 300), (64, 8, 2), (1024, 136, 129)])
 def test_mm8_seq(N, M, B):
     ops = _ops()
     x, ref, (q, mx, rx, my, ry) = _mm8_case(N, M, B, N + M + B)
@@ -133,7 +135,8 @@ def test_mm8_linearity_full_size():
 @pytest.mark.parametrize("N,M,B", [(768, 768, 1), (768, 3072, 1), (4096, 4096, 1), (16384, 4096, 1), (768, 50277, 1),
                                    (768, 768, 7), (3072, 768, 128), (4096, 4096, 300), (768, 50277, 4),
                                    # long calls (256 x 256 tiles loaded straight into LDS): split-K, ragged, shallow
-                                   (4096, 4096, 1024), (4096, 8192, 520), (128, 4096, 1024)])
+                                   (4096, 4096, 1024), (4096, 8192, 520), (128, 4096, 1024),
+                                   (128, 200, 37), (192, 1000, 300), (64, 8, 2)])
 @pytest.mark.parametrize("out_dtype", [torch.float16, torch.float32])
 def test_gemm_f16(N, M, B, out_dtype):
     ops = _ops()
