@@ -328,14 +328,18 @@ DEV void gemm_dma_body(int T, int N, int M, const h16 *__restrict__ A, int64_t l
     }
     typedef __attribute__((address_space(1))) const void *gptr;
     typedef __attribute__((address_space(3))) void *lptr;
-    auto issue = [&](int kt, int so) {
+    // part 0 / 1: the halves of this wave's A loads, part 2: its weight loads; -1: all of them
+    auto issue = [&](int kt, int so, int part) {
         unsigned char *base = smem + so;
 #pragma unroll
         for (int i = 0; i < AL; ++i)
-            __builtin_amdgcn_global_load_lds((gptr)(ga[i] + kt * BK), (lptr)(base + (wave * AL + i) * 1024), 16, 0, 0);
+            if (part < 0 || part == (i >= (AL + 1) / 2 ? 1 : 0))
+                __builtin_amdgcn_global_load_lds((gptr)(ga[i] + kt * BK), (lptr)(base + (wave * AL + i) * 1024), 16, 0, 0);
+        if (part < 0 || part == 2) {
 #pragma unroll
-        for (int i = 0; i < WL; ++i)
-            __builtin_amdgcn_global_load_lds((gptr)(gw[i] + kt * BK * (W_U8 ? 1 : 2)), (lptr)(base + D_A + (wave * WL + i) * 1024), 16, 0, 0);
+            for (int i = 0; i < WL; ++i)
+                __builtin_amdgcn_global_load_lds((gptr)(gw[i] + kt * BK * (W_U8 ? 1 : 2)), (lptr)(base + D_A + (wave * WL + i) * 1024), 16, 0, 0);
+        }
     };
 
     f32x16 acc[MI][NI];
@@ -401,35 +405,44 @@ DEV void gemm_dma_body(int T, int N, int M, const h16 *__restrict__ A, int64_t l
 
     // Every wave issues exactly LOADS loads per tile, so "vmcnt(LOADS n)" means "all but my newest n tiles have
     // landed".  Past the last tile the loads repeat it into a stage nobody reads any more, which keeps the counts static.
-    issue(0, 0);
-    issue(min(1, nk - 1), D_STAGE);
-    if (D_NST > 2) issue(min(2, nk - 1), 2 * D_STAGE);
-    __builtin_amdgcn_s_waitcnt(vm_only((D_NST - 1) * Cfg::LOADS));   // tile 0 has landed
+    // Three stages: while tile kt multiplies, tile kt + 1 has landed or is landing and the loads of tile kt + 2 are
+    // issued in three parts between the MFMA steps, into the stage tile kt - 1 was read from (a burst of all of
+    // them right after the barrier measured 2 % slower).  Two stages: tile kt + 2 can only go where tile kt is, so
+    // its loads follow the barrier in one go.
+    constexpr bool SPREAD = D_NST == 3;
+    issue(0, 0, -1);
+    issue(min(1, nk - 1), D_STAGE, -1);
+    __builtin_amdgcn_s_waitcnt(vm_only(Cfg::LOADS));   // tile 0 has landed
     __builtin_amdgcn_s_barrier();
     ldfrag(0, 0, 0);
-    int so = 0;
+    int so = 0, sp = 2 * D_STAGE;   // the stage being read and (three stages) the one read before it
     for (int kt = 0; kt < nk; ++kt) {
         const int sn = so + D_STAGE >= D_NST * D_STAGE ? 0 : so + D_STAGE;
+        const int kl = min(kt + 2, nk - 1);
         ldfrag(1, so, 1);
+        if (SPREAD) issue(kl, sp, 0);
         __builtin_amdgcn_sched_barrier(0);
         older_reads_done();
         multiply(0);
         ldfrag(0, so, 2);
+        if (SPREAD) issue(kl, sp, 1);
         __builtin_amdgcn_sched_barrier(0);
         older_reads_done();
         multiply(1);
         ldfrag(1, so, 3);
+        if (SPREAD) issue(kl, sp, 2);
         __builtin_amdgcn_sched_barrier(0);
         older_reads_done();
         multiply(0);
         // all my reads of this stage have returned and my part of tile kt + 1 has landed (with three stages tile
-        // kt + 2 may be in flight)
-        __builtin_amdgcn_s_waitcnt(vm_lgkm0((D_NST - 2) * Cfg::LOADS));
+        // kt + 2 is in flight)
+        __builtin_amdgcn_s_waitcnt(vm_lgkm0(SPREAD ? Cfg::LOADS : 0));
         __builtin_amdgcn_s_barrier();
-        issue(min(kt + D_NST, nk - 1), so);
+        if (!SPREAD) issue(kl, so, -1);
         ldfrag(0, sn, 0);
         __builtin_amdgcn_sched_barrier(0);
         multiply(1);
+        sp = so;
         so = sn;
     }
     __builtin_amdgcn_s_waitcnt(0x0070);   // vmcnt(0) lgkmcnt(0): nothing may land in LDS after the workgroup has gone
