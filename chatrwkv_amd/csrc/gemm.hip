@@ -611,15 +611,16 @@ struct PrepGroup {
     float *s0[4], *s2[4];
 };
 
-// xs[t, j] = fp16(x[t, j] * ry[j]);  s0[t] = sum_j x[t, j];  s2[t] = sum_j x[t, j] * my[j].  One wave per row.
+// xs[t, j] = fp16(x[t, j] * ry[j]);  s0[t] = sum_j x[t, j];  s2[t] = sum_j x[t, j] * my[j].  One workgroup (four
+// waves) per row: a 16384-wide row per wave left the memory system with four waves per CU to draw from.
 __global__ __launch_bounds__(256) void mm8_prepare_kernel(int T, int N, const rwkv_half *__restrict__ x, int64_t ldx,
                                                           const rwkv_half *__restrict__ ry,
                                                           const rwkv_half *__restrict__ my, rwkv_half *__restrict__ xs,
                                                           float *__restrict__ s0, float *__restrict__ s2) {
-    const int t = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
-    if (t >= T) return;
+    __shared__ float red[8];
+    const int t = blockIdx.x, lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
     float a0 = 0.f, a2 = 0.f;
-    for (int j = lane * 8; j < N; j += 64 * 8) {
+    for (int j = threadIdx.x * 8; j < N; j += 256 * 8) {
         const u32x4 xv = *(const u32x4 *)(x + (size_t)t * ldx + j);
         const u32x4 rv = *(const u32x4 *)(ry + j);
         const u32x4 mv = *(const u32x4 *)(my + j);
@@ -637,7 +638,12 @@ __global__ __launch_bounds__(256) void mm8_prepare_kernel(int T, int N, const rw
     }
     a0 = wave_sum(a0);
     a2 = wave_sum(a2);
-    if (lane == 0) { s0[t] = a0; s2[t] = a2; }
+    if (lane == 0) { red[wid] = a0; red[4 + wid] = a2; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        s0[t] = (red[0] + red[1]) + (red[2] + red[3]);
+        s2[t] = (red[4] + red[5]) + (red[6] + red[7]);
+    }
 }
 
 // the same for up to four (x, matrix) pairs in one launch: blockIdx.y picks the pair
@@ -832,8 +838,7 @@ int gemm_launch(bool w_u8, int64_t T, int64_t N, int64_t M, const rwkv_half *A, 
 
 int mm8_prepare_launch(int64_t T, int64_t N, const rwkv_half *x, int64_t ldx, const rwkv_half *ry,
                        const rwkv_half *my, rwkv_half *xs, float *s0, float *s2, hipStream_t st) {
-    hipLaunchKernelGGL(mm8_prepare_kernel, dim3((unsigned)((T + 3) / 4)), dim3(256), 0, st, (int)T, (int)N, x, ldx, ry,
-                       my, xs, s0, s2);
+    hipLaunchKernelGGL(mm8_prepare_kernel, dim3((unsigned)T), dim3(256), 0, st, (int)T, (int)N, x, ldx, ry, my, xs, s0, s2);
     RWKV_LAUNCH_CHECK();
     return RWKV_OK;
 }
