@@ -50,6 +50,7 @@ struct SeqMixArgs {
     const rwkv_half *ln_w, *ln_b;
     const rwkv_half *sx;       // state (previous token's normalised activation), NULL = no token shift
     rwkv_half *xx_last;        // scratch [C]: normalised activation of the last row (new state)
+    rwkv_half *state_out;      // or: the state itself (may be sx): written by row 0's workgroup after it has read sx
     const rwkv_half *mix[6];   // NULL entry = consumer sees LN(x)
     const rwkv_half *ry[6], *my[6];  // NULL ry = no scaling / sums (fp16 weights)
     rwkv_half *xs[6];          // [T, C] outputs

@@ -112,6 +112,21 @@ __global__ __launch_bounds__(256) void lnmix_seq_kernel(SeqMixArgs a) {
         const float v0 = block_sum(acc[2 * j], red), v2 = block_sum(acc[2 * j + 1], red);
         if (threadIdx.x == 0) { a.s0[j][t] = v0; a.s2[j][t] = v2; }
     }
+    // The new token-shift state is LN(x[T-1]).  Only row 0 reads the old one, so row 0's workgroup writes the new
+    // one once its own reads are done (each thread overwrites exactly the chunks it has read): no second launch.
+    if (a.state_out && t == 0) {
+        const rwkv_half *xl = a.x + (size_t)(a.T - 1) * C;
+        if (a.T > 1) row_stats(xl, C, red, mean, rstd);
+        for (int j8 = threadIdx.x; j8 < (C >> 3); j8 += blockDim.x) {
+            const h16x8 xv = *(const h16x8 *)(xl + 8 * j8);
+            const h16x8 wv = *(const h16x8 *)(a.ln_w + 8 * j8);
+            const h16x8 bv = *(const h16x8 *)(a.ln_b + 8 * j8);
+            h16x8 xx;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) xx[e] = (h16)(((float)xv[e] - mean) * rstd * (float)wv[e] + (float)bv[e]);
+            *(h16x8 *)(a.state_out + 8 * j8) = xx;
+        }
+    }
 }
 
 __global__ __launch_bounds__(256) void ln_f32_f16_kernel(int C, const float *__restrict__ x_, const float *__restrict__ w,
@@ -273,7 +288,6 @@ extern "C" int rwkv_v4_forward_seq(const rwkv_v4_model *m, const rwkv_v4_layer_s
     float *s0[3] = {ws.sums, ws.sums + 2 * T, ws.sums + 4 * T};
     float *s2[3] = {ws.sums + T, ws.sums + 3 * T, ws.sums + 5 * T};
     float *s0v = ws.sums + 6 * T, *s2v = ws.sums + 7 * T;
-    const int n16 = C >> 3;
 
     hipLaunchKernelGGL(gather_emb_kernel, dim3((unsigned)T), dim3(256), 0, st, (int)T, C, tokens, m->emb, ws.x);
     SideStreams *ss = T >= 256 ? side_streams() : nullptr;
@@ -286,7 +300,7 @@ extern "C" int rwkv_v4_forward_seq(const rwkv_v4_model *m, const rwkv_v4_layer_s
         {
             SeqMixArgs a{};
             a.T = (int)T; a.C = C; a.x = ws.x; a.ln_w = l.ln1_w; a.ln_b = l.ln1_b; a.sx = s.att_xx;
-            a.xx_last = ws.xx_att;
+            a.xx_last = nullptr; a.state_out = s.att_xx;
             const rwkv_half *mix[3] = {l.att_mix_k, l.att_mix_v, l.att_mix_r};
             const rwkv_mat *mt[3] = {&l.att_key, &l.att_value, &l.att_receptance};
             for (int j = 0; j < 3; ++j) {
@@ -295,8 +309,6 @@ extern "C" int rwkv_v4_forward_seq(const rwkv_v4_model *m, const rwkv_v4_layer_s
             }
             if ((rc = lnmix_seq_launch(a, 3, st))) return rc;
         }
-        hipLaunchKernelGGL(copy16_kernel, dim3((n16 + 255) / 256), dim3(256), 0, st, n16, (const u32x4 *)ws.xx_att,
-                           (u32x4 *)s.att_xx);
         GemmEpi e{};
         e.out_scale = 1.f;
         // k, v: uint8 weights return fp16 (widened by the consumer); fp16 weights return fp32 directly
@@ -339,7 +351,7 @@ extern "C" int rwkv_v4_forward_seq(const rwkv_v4_model *m, const rwkv_v4_layer_s
         {
             SeqMixArgs a{};
             a.T = (int)T; a.C = C; a.x = ws.x; a.ln_w = l.ln2_w; a.ln_b = l.ln2_b; a.sx = s.ffn_xx;
-            a.xx_last = ws.xx_ffn;
+            a.xx_last = nullptr; a.state_out = s.ffn_xx;
             const rwkv_half *mix[2] = {l.ffn_mix_r, l.ffn_mix_k};
             const rwkv_mat *mt[2] = {&l.ffn_receptance, &l.ffn_key};
             for (int j = 0; j < 2; ++j) {
@@ -348,8 +360,6 @@ extern "C" int rwkv_v4_forward_seq(const rwkv_v4_model *m, const rwkv_v4_layer_s
             }
             if ((rc = lnmix_seq_launch(a, 2, st))) return rc;
         }
-        hipLaunchKernelGGL(copy16_kernel, dim3((n16 + 255) / 256), dim3(256), 0, st, n16, (const u32x4 *)ws.xx_ffn,
-                           (u32x4 *)s.ffn_xx);
         e = GemmEpi{};
         e.out_scale = 1.f; e.out_dtype = RWKV_DT_F16;
         e.act = ACT_SIGMOID;

@@ -19,7 +19,7 @@ constexpr float LN_EPS56 = 1e-5f;
 struct Mix1Args {
     int T, C;
     const rwkv_half *x, *ln_w, *ln_b, *sx, *maa_x;
-    rwkv_half *xx, *sxd, *xxx, *xx_last;
+    rwkv_half *xx, *sxd, *xxx, *state_out;   // state_out: the token-shift state (may be sx)
 };
 
 // grid T x 256 threads: xx = LN1(x[t]); sxd = prev - xx; xxx = xx + sxd * maa_x.
@@ -65,7 +65,20 @@ __global__ __launch_bounds__(256) void v6_mix1_kernel(Mix1Args a) {
         *(h16x8 *)(a.xx + o) = xx;
         *(h16x8 *)(a.sxd + o) = sd;
         *(h16x8 *)(a.xxx + o) = xo;
-        if (t == a.T - 1) *(h16x8 *)(a.xx_last + 8 * j8) = xx;
+    }
+    // the new token-shift state LN1(x[T-1]): written by row 0's workgroup, the only one that reads the old state,
+    // after its own reads (each thread overwrites exactly the chunks it has read)
+    if (t == 0) {
+        const rwkv_half *xl = a.x + (size_t)(a.T - 1) * C;
+        if (a.T > 1) stats(xl, mean, rstd);
+        for (int j8 = threadIdx.x; j8 < (C >> 3); j8 += blockDim.x) {
+            const h16x8 xv = *(const h16x8 *)(xl + 8 * j8);
+            const h16x8 wv = *(const h16x8 *)(a.ln_w + 8 * j8), bv = *(const h16x8 *)(a.ln_b + 8 * j8);
+            h16x8 xx;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) xx[e] = (h16)(((float)xv[e] - mean) * rstd * (float)wv[e] + (float)bv[e]);
+            *(h16x8 *)(a.state_out + 8 * j8) = xx;
+        }
     }
 }
 
@@ -249,7 +262,7 @@ extern "C" int rwkv_v56_forward(const rwkv_v56_model *m, const rwkv_v56_layer_st
                 lnmix1_small_launch(a, st);
                 b.xx = ws.xx_att; b.sxd = nullptr; b.prev = s.att_xx;
             } else {
-                Mix1Args a{(int)T, C, ws.x, l.ln1_w, l.ln1_b, s.att_xx, l.att_mix[0], ws.xx, ws.sxd, ws.xxx, ws.xx_att};
+                Mix1Args a{(int)T, C, ws.x, l.ln1_w, l.ln1_b, s.att_xx, l.att_mix[0], ws.xx, ws.sxd, ws.xxx, s.att_xx};
                 hipLaunchKernelGGL(v6_mix1_kernel, dim3((unsigned)T), dim3(256), 0, st, a);
                 if ((rc = mm(c, lora_mat(l.tm_w1, C, 5 * lm), false, ws.xxx, ACT_TANH, nullptr, nullptr, 1.f, ws.t1))) return rc;
                 b.xx = ws.xx; b.sxd = ws.sxd; b.prev = nullptr;
@@ -266,7 +279,8 @@ extern "C" int rwkv_v56_forward(const rwkv_v56_model *m, const rwkv_v56_layer_st
         } else {
             SeqMixArgs a{};
             a.T = (int)T; a.C = C; a.x = ws.x; a.ln_w = l.ln1_w; a.ln_b = l.ln1_b; a.sx = s.att_xx;
-            a.xx_last = ws.xx_att;
+            // sequence calls: row 0's workgroup commits the new state; one token: the r / k / v launch below does
+            if (T == 1) a.xx_last = ws.xx_att; else a.state_out = s.att_xx;
             const int nj = gated ? 4 : 3;
             for (int j = 0; j < nj; ++j) { a.mix[j] = l.att_mix[j]; a.ry[j] = nullptr; a.my[j] = nullptr; a.xs[j] = ws.mix[j]; }
             if ((rc = lnmix_seq_launch(a, nj, st))) return rc;
@@ -301,14 +315,13 @@ extern "C" int rwkv_v56_forward(const rwkv_v56_model *m, const rwkv_v56_layer_st
                     ep[j].act = j == 3 ? ACT_SILU : ACT_NONE; ep[j].out_scale = 1.f; ep[j].out_dtype = RWKV_DT_F16;
                     ep[j].ldres = C; ep[j].ldgate = C;
                 }
-                if ((rc = copy_h16_launch(C, ws.xx_att, s.att_xx, st))) return rc;
                 if ((rc = gemm_group_launch(u8, n, T, C, xin, mats, outs, ep, xsc, sm, ws.splitk, st))) return rc;
             } else {
             // receptance (then gate) on the caller's stream, key and value on the side streams
             const bool par = ss && !dma_seq && fork_streams(ss, st, 2);
             Ctx cr = c;
             if (par) cr.splitk = nullptr;
-            if ((rc = mm(cr, l.att_receptance, u8, rx, ACT_NONE, nullptr, nullptr, 1.f, ws.r, ws.xx_att, s.att_xx, C))) return rc;
+            if ((rc = mm(cr, l.att_receptance, u8, rx, ACT_NONE, nullptr, nullptr, 1.f, ws.r))) return rc;
             if ((rc = mm(par ? cs[0] : c, l.att_key, u8, kx, ACT_NONE, nullptr, nullptr, 1.f, ws.k))) return rc;
             if ((rc = mm(par ? cs[1] : c, l.att_value, u8, vx, ACT_NONE, nullptr, nullptr, 1.f, ws.v))) return rc;
             if (gated && (rc = mm(c, l.att_gate, u8, gx, ACT_SILU, nullptr, nullptr, 1.f, ws.g))) return rc;
@@ -340,7 +353,7 @@ extern "C" int rwkv_v56_forward(const rwkv_v56_model *m, const rwkv_v56_layer_st
         {
             SeqMixArgs a{};
             a.T = (int)T; a.C = C; a.x = ws.x; a.ln_w = l.ln2_w; a.ln_b = l.ln2_b; a.sx = s.ffn_xx;
-            a.xx_last = ws.xx_ffn; a.maa_form = v6 ? 1 : 0;
+            a.xx_last = nullptr; a.state_out = s.ffn_xx; a.maa_form = v6 ? 1 : 0;
             a.mix[0] = l.ffn_mix_r; a.mix[1] = l.ffn_mix_k;
             for (int j = 0; j < 2; ++j) { a.ry[j] = nullptr; a.my[j] = nullptr; a.xs[j] = ws.mix[j]; }
             if ((rc = lnmix_seq_launch(a, 2, st))) return rc;
@@ -355,15 +368,13 @@ extern "C" int rwkv_v56_forward(const rwkv_v56_model *m, const rwkv_v56_layer_st
             GemmEpi ep[2] = {};
             ep[0].act = ACT_SIGMOID; ep[1].act = ACT_RELU_SQ;
             for (int j = 0; j < 2; ++j) { ep[j].out_scale = 1.f; ep[j].out_dtype = RWKV_DT_F16; }
-            if ((rc = copy_h16_launch(C, ws.xx_ffn, s.ffn_xx, st))) return rc;
             if ((rc = gemm_group_launch(u8, 2, T, C, xin, mats, outs, ep, xsc, sm, ws.splitk, st))) return rc;
         } else {
             // channel-mix receptance beside the key product
             const bool par = ss && !dma_seq && fork_streams(ss, st, 1);
-            if (par && (rc = copy_h16_launch(C, ws.xx_ffn, s.ffn_xx, st))) return rc;
             if (par) {
                 if ((rc = mm(cs[0], l.ffn_receptance, u8, ws.mix[0], ACT_SIGMOID, nullptr, nullptr, 1.f, ws.r))) return rc;
-            } else if ((rc = mm(c, l.ffn_receptance, u8, ws.mix[0], ACT_SIGMOID, nullptr, nullptr, 1.f, ws.r, ws.xx_ffn, s.ffn_xx, C))) {
+            } else if ((rc = mm(c, l.ffn_receptance, u8, ws.mix[0], ACT_SIGMOID, nullptr, nullptr, 1.f, ws.r))) {
                 return rc;
             }
             Ctx ck = c;

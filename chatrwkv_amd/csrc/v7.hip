@@ -573,7 +573,7 @@ extern "C" int rwkv_v7_forward(const rwkv_v7_model *m, const rwkv_v56_layer_stat
         {
             SeqMixArgs a{};
             a.T = (int)T; a.C = C; a.x = ws.x; a.ln_w = l.ln1_w; a.ln_b = l.ln1_b; a.sx = s.att_xx;
-            a.xx_last = ws.xx_att; a.maa_form = 1;
+            a.xx_last = nullptr; a.state_out = s.att_xx; a.maa_form = 1;   // row 0's workgroup commits the new state
             for (int j = 0; j < 6; ++j) { a.mix[j] = l.x_mix[j]; a.xs[j] = ws.mix[j]; }
             if ((rc = lnmix_seq_launch(a, 6, st))) return rc;
         }
@@ -588,7 +588,6 @@ extern "C" int rwkv_v7_forward(const rwkv_v7_model *m, const rwkv_v56_layer_stat
         const bool par = ss && dma_seq && 3 * ((T + 255) / 256) * ((C + 255) / 256) >= 192 && fork_streams(ss, st, 1);
         Ctx cm = c, cv = c, cl = c;
         if (par) cl.st = ss->s[0];
-        // the first matrix call also commits the new token-shift state (all readers of the old one are done)
         if (dma_seq && !(C & 7)) {
             // receptance, key and value as one grouped launch
             const rwkv_half *xin[3] = {xr, xk, xv};
@@ -596,10 +595,9 @@ extern "C" int rwkv_v7_forward(const rwkv_v7_model *m, const rwkv_v56_layer_stat
             void *outs[3] = {ws.r, ws.k, v};
             GemmEpi ep[3] = {};
             for (int j = 0; j < 3; ++j) { ep[j].act = ACT_NONE; ep[j].out_scale = 1.f; ep[j].out_dtype = RWKV_DT_F16; }
-            if ((rc = copy_h16_launch(C, ws.xx_att, s.att_xx, st))) return rc;
             if ((rc = gemm_group_launch(false, 3, T, C, xin, mats, outs, ep, nullptr, nullptr, ws.splitk, st))) return rc;
         } else {
-        if ((rc = mm(cm, l.att_receptance, false, xr, ACT_NONE, nullptr, nullptr, 1.f, ws.r, ws.xx_att, s.att_xx, C))) return rc;
+        if ((rc = mm(cm, l.att_receptance, false, xr, ACT_NONE, nullptr, nullptr, 1.f, ws.r))) return rc;
         if ((rc = mm(cm, l.att_key, false, xk, ACT_NONE, nullptr, nullptr, 1.f, ws.k))) return rc;
         if ((rc = mm(cv, l.att_value, false, xv, ACT_NONE, nullptr, nullptr, 1.f, v))) return rc;
         }
@@ -633,11 +631,11 @@ extern "C" int rwkv_v7_forward(const rwkv_v7_model *m, const rwkv_v56_layer_stat
         {
             SeqMixArgs a{};
             a.T = (int)T; a.C = C; a.x = ws.x; a.ln_w = l.ln2_w; a.ln_b = l.ln2_b; a.sx = s.ffn_xx;
-            a.xx_last = ws.xx_ffn; a.maa_form = 1;
+            a.xx_last = nullptr; a.state_out = s.ffn_xx; a.maa_form = 1;
             a.mix[0] = l.ffn_x_k; a.xs[0] = ws.mix[0];
             if ((rc = lnmix_seq_launch(a, 1, st))) return rc;
         }
-        if ((rc = mm(c, l.ffn_key, false, ws.mix[0], ACT_RELU_SQ, nullptr, nullptr, 1.f, ws.vx, ws.xx_ffn, s.ffn_xx, C))) return rc;
+        if ((rc = mm(c, l.ffn_key, false, ws.mix[0], ACT_RELU_SQ, nullptr, nullptr, 1.f, ws.vx))) return rc;
         if ((rc = mm(c, l.ffn_value, false, ws.vx, ACT_RESIDUAL, ws.x, nullptr, 1.f, ws.x))) return rc;
         RWKV_LAUNCH_CHECK();
     }
