@@ -117,16 +117,15 @@ def gemm_roofline(T, N, M, u8, reps=10):
             lib.check(L.rwkv_mm8_seq_f16(T, N, M, x.data_ptr(), N, w.data_ptr(), 1, N, mx.data_ptr(), rx.data_ptr(),
                                          my.data_ptr(), ry.data_ptr(), y.data_ptr(), M, ws.data_ptr(), nbytes, st),
                       "rwkv_mm8_seq_f16")
-        name = ("gemm_dma_kernel<uint8 weights> (256x256 tile, direct-to-LDS loads)" if T >= 512 else
-                "gemm_kernel<uint8 weights, 128x128 tile>") + " + mm8_prepare_kernel"
+        name = ("gemm_dma_kernel<uint8 weights> (direct-to-LDS loads; 256x256 or 128x128 tile by the launch cost model)"
+                + " + mm8_prepare_kernel")
     else:
         w = torch.randn(M, N, device=dev).half()
 
         def run():
             lib.check(L.rwkv_gemm_f16(T, N, M, x.data_ptr(), N, w.data_ptr(), 1, N, y.data_ptr(), M, lib.RWKV_DT_F16, st),
                       "rwkv_gemm_f16")
-        name = ("gemm_dma_kernel<fp16 weights> (256x256 tile, direct-to-LDS loads)" if T >= 512 else
-                "gemm_kernel<fp16 weights, 128x128 tile>")
+        name = "gemm_dma_kernel<fp16 weights> (direct-to-LDS loads; 256x256 or 128x128 tile by the launch cost model)"
     for _ in range(3):
         run()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
