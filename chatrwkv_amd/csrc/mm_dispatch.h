@@ -60,6 +60,21 @@ inline int mm(const Ctx &c, const rwkv_mat &m, bool mat_u8, const rwkv_half *x, 
     return gemm_launch(mat_u8, c.T, N, M, A, N, m.w, m.ld, out, M, e, c.st);
 }
 
+// Sequence calls only: the same product for an activation that the producing kernel has already scaled by the
+// matrix's ry (uint8 matrices; s0 / s2 = its row sums of x and x * my) -- no scaling pass.  fp16 matrices: xs is
+// the plain activation and the sums are not read.
+inline int mm_scaled(const Ctx &c, const rwkv_mat &m, bool mat_u8, const rwkv_half *xs, const float *s0, const float *s2,
+                     int act, const rwkv_half *res, const rwkv_half *gate, float out_scale, rwkv_half *out) {
+    const int N = (int)m.N, M = (int)m.M;
+    if (c.T <= 1) return RWKV_E_SHAPE;
+    GemmEpi e{};
+    e.act = act; e.res = res; e.ldres = M; e.gate = gate; e.ldgate = M; e.out_scale = out_scale;
+    e.out_dtype = RWKV_DT_F16; e.splitk_ws = c.splitk; e.splitk_bytes = RWKV_SPLITK_WS_BYTES;
+    e.small_tiles = c.small_tiles;
+    if (mat_u8) { e.mx = m.mx; e.rx = m.rx; e.s0 = s0; e.s2 = s2; }
+    return gemm_launch(mat_u8, c.T, N, M, xs, N, m.w, m.ld, out, M, e, c.st);
+}
+
 inline size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
 inline rwkv_mat lora_mat(const rwkv_half *w, int64_t N, int64_t M) {

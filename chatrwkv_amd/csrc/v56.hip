@@ -250,7 +250,8 @@ extern "C" int rwkv_v56_forward(const rwkv_v56_model *m, const rwkv_v56_layer_st
         // CU, so products side by side on several streams gain nothing)
         const bool dma_seq = T >= 512;
         const rwkv_half *kx, *vx, *rx, *gx = nullptr, *wx = nullptr;
-        bool fuse_d1 = false;
+        bool fuse_d1 = false, att_scaled = false;
+        float *att_sums[4] = {ws.sums, ws.sums_side[0], ws.sums_side[1], ws.sums_side[2]};   // of kx, vx, rx, gx
         if (v6) {
             Mix2Args b{};
             if (T == 1) {
@@ -282,7 +283,14 @@ extern "C" int rwkv_v56_forward(const rwkv_v56_model *m, const rwkv_v56_layer_st
             // sequence calls: row 0's workgroup commits the new state; one token: the r / k / v launch below does
             if (T == 1) a.xx_last = ws.xx_att; else a.state_out = s.att_xx;
             const int nj = gated ? 4 : 3;
-            for (int j = 0; j < nj; ++j) { a.mix[j] = l.att_mix[j]; a.ry[j] = nullptr; a.my[j] = nullptr; a.xs[j] = ws.mix[j]; }
+            // sequence calls with uint8 matrices: the same launch scales each mix by its matrix's ry and sums the rows
+            att_scaled = T > 1 && u8;
+            const rwkv_mat *mt[4] = {&l.att_key, &l.att_value, &l.att_receptance, &l.att_gate};
+            for (int j = 0; j < nj; ++j) {
+                a.mix[j] = l.att_mix[j]; a.xs[j] = ws.mix[j];
+                a.ry[j] = att_scaled ? mt[j]->ry : nullptr; a.my[j] = att_scaled ? mt[j]->my : nullptr;
+                a.s0[j] = att_sums[j]; a.s2[j] = att_sums[j] + T;
+            }
             if ((rc = lnmix_seq_launch(a, nj, st))) return rc;
             kx = ws.mix[0]; vx = ws.mix[1]; rx = ws.mix[2]; gx = gated ? ws.mix[3] : nullptr;
         }
@@ -315,7 +323,17 @@ extern "C" int rwkv_v56_forward(const rwkv_v56_model *m, const rwkv_v56_layer_st
                     ep[j].act = j == 3 ? ACT_SILU : ACT_NONE; ep[j].out_scale = 1.f; ep[j].out_dtype = RWKV_DT_F16;
                     ep[j].ldres = C; ep[j].ldgate = C;
                 }
-                if ((rc = gemm_group_launch(u8, n, T, C, xin, mats, outs, ep, xsc, sm, ws.splitk, st))) return rc;
+                float *smx[4] = {att_sums[2], att_sums[0], att_sums[1], att_sums[3]};
+                if ((rc = gemm_group_launch(u8, n, T, C, xin, mats, outs, ep, att_scaled ? nullptr : xsc, att_scaled ? smx : sm,
+                                            ws.splitk, st)))
+                    return rc;
+            } else if (att_scaled) {
+                if ((rc = mm_scaled(c, l.att_receptance, u8, rx, att_sums[2], att_sums[2] + T, ACT_NONE, nullptr, nullptr, 1.f, ws.r)) ||
+                    (rc = mm_scaled(c, l.att_key, u8, kx, att_sums[0], att_sums[0] + T, ACT_NONE, nullptr, nullptr, 1.f, ws.k)) ||
+                    (rc = mm_scaled(c, l.att_value, u8, vx, att_sums[1], att_sums[1] + T, ACT_NONE, nullptr, nullptr, 1.f, ws.v)))
+                    return rc;
+                if (gated && (rc = mm_scaled(c, l.att_gate, u8, gx, att_sums[3], att_sums[3] + T, ACT_SILU, nullptr, nullptr, 1.f, ws.g)))
+                    return rc;
             } else {
             // receptance (then gate) on the caller's stream, key and value on the side streams
             const bool par = ss && !dma_seq && fork_streams(ss, st, 2);
@@ -350,36 +368,40 @@ extern "C" int rwkv_v56_forward(const rwkv_v56_model *m, const rwkv_v56_layer_st
             RWKV_LAUNCH_CHECK();
             continue;
         }
+        // LN2 + token shift + the two mixes; for uint8 matrices the same launch scales each mix by its matrix's ry and
+        // sums the rows, so the two products below need no scaling pass
+        rwkv_half *fx[2] = {u8 ? ws.xs_side[0] : ws.mix[0], u8 ? ws.xs_side[1] : ws.mix[1]};
+        float *fs[2] = {ws.sums_side[0], ws.sums_side[1]};
         {
             SeqMixArgs a{};
             a.T = (int)T; a.C = C; a.x = ws.x; a.ln_w = l.ln2_w; a.ln_b = l.ln2_b; a.sx = s.ffn_xx;
             a.xx_last = nullptr; a.state_out = s.ffn_xx; a.maa_form = v6 ? 1 : 0;
             a.mix[0] = l.ffn_mix_r; a.mix[1] = l.ffn_mix_k;
-            for (int j = 0; j < 2; ++j) { a.ry[j] = nullptr; a.my[j] = nullptr; a.xs[j] = ws.mix[j]; }
+            const rwkv_mat *mt[2] = {&l.ffn_receptance, &l.ffn_key};
+            for (int j = 0; j < 2; ++j) {
+                a.ry[j] = u8 ? mt[j]->ry : nullptr; a.my[j] = u8 ? mt[j]->my : nullptr;
+                a.xs[j] = fx[j]; a.s0[j] = fs[j]; a.s2[j] = fs[j] + T;
+            }
             if ((rc = lnmix_seq_launch(a, 2, st))) return rc;
         }
         if (T <= 128 && !(C & 127) && !(F & 127)) {
             // short calls: receptance and key in one grouped launch (measured: +7 % at 64 rows, -5 % at 256)
-            const rwkv_half *xin[2] = {ws.mix[0], ws.mix[1]};
+            const rwkv_half *xin[2] = {fx[0], fx[1]};
             const rwkv_mat *mats[2] = {&l.ffn_receptance, &l.ffn_key};
             void *outs[2] = {ws.r, ws.vx};
-            rwkv_half *xsc[2] = {ws.xs, ws.xs_side[0]};
-            float *sm[2] = {ws.sums, ws.sums_side[0]};
             GemmEpi ep[2] = {};
             ep[0].act = ACT_SIGMOID; ep[1].act = ACT_RELU_SQ;
             for (int j = 0; j < 2; ++j) { ep[j].out_scale = 1.f; ep[j].out_dtype = RWKV_DT_F16; }
-            if ((rc = gemm_group_launch(u8, 2, T, C, xin, mats, outs, ep, xsc, sm, ws.splitk, st))) return rc;
+            if ((rc = gemm_group_launch(u8, 2, T, C, xin, mats, outs, ep, nullptr, fs, ws.splitk, st))) return rc;
         } else {
             // channel-mix receptance beside the key product
             const bool par = ss && !dma_seq && fork_streams(ss, st, 1);
-            if (par) {
-                if ((rc = mm(cs[0], l.ffn_receptance, u8, ws.mix[0], ACT_SIGMOID, nullptr, nullptr, 1.f, ws.r))) return rc;
-            } else if ((rc = mm(c, l.ffn_receptance, u8, ws.mix[0], ACT_SIGMOID, nullptr, nullptr, 1.f, ws.r))) {
+            if ((rc = mm_scaled(par ? cs[0] : c, l.ffn_receptance, u8, fx[0], fs[0], fs[0] + T, ACT_SIGMOID, nullptr, nullptr,
+                                1.f, ws.r)))
                 return rc;
-            }
             Ctx ck = c;
             ck.small_tiles = par ? 1 : 0;
-            if ((rc = mm(ck, l.ffn_key, u8, ws.mix[1], ACT_RELU_SQ, nullptr, nullptr, 1.f, ws.vx))) return rc;
+            if ((rc = mm_scaled(ck, l.ffn_key, u8, fx[1], fs[1], fs[1] + T, ACT_RELU_SQ, nullptr, nullptr, 1.f, ws.vx))) return rc;
             if (par && !join_streams(ss, st, 1)) return (int)hipErrorUnknown;
         }
         if ((rc = mm(c, l.ffn_value, u8, ws.vx, ACT_GATED_RESIDUAL, ws.x, ws.r, scale, ws.x))) return rc;
