@@ -88,6 +88,79 @@ __global__ __launch_bounds__(256) void splitk_epilogue_kernel(int T, int M, int 
     }
 }
 
+// The same pass for the direct-to-LDS launches, whose operands are all laid out for 16-byte accesses (dma_ok):
+// eight consecutive outputs per thread, all slab loads of a thread in flight together, 16-byte loads of the
+// residual / gate rows and 16-byte stores.  Same slab order and the same arithmetic per element as above.
+template <int KS>
+DEV void splitk_rows8(int T, int M, int ks_rt, const float *__restrict__ part, void *Y, int64_t ldy, const GemmEpi &ep,
+                      int64_t first, int64_t stride) {
+    const int64_t n8 = (int64_t)T * M / 8, n = (int64_t)T * M;
+    const int m8 = M / 8, ks = KS ? KS : ks_rt;
+    for (int64_t i = first; i < n8; i += stride) {
+        const int t = (int)(i / m8), col = (int)(i - (int64_t)t * m8) * 8;
+        f32x4 lo = *(const f32x4 *)(part + 8 * i), hi = *(const f32x4 *)(part + 8 * i + 4);
+        if constexpr (KS > 0) {
+            f32x4 pl[KS], ph[KS];
+#pragma unroll
+            for (int k = 1; k < KS; ++k) {
+                pl[k] = *(const f32x4 *)(part + (size_t)k * n + 8 * i);
+                ph[k] = *(const f32x4 *)(part + (size_t)k * n + 8 * i + 4);
+            }
+#pragma unroll
+            for (int k = 1; k < KS; ++k) { lo += pl[k]; hi += ph[k]; }
+        } else {
+            for (int k = 1; k < ks; ++k) {
+                lo += *(const f32x4 *)(part + (size_t)k * n + 8 * i);
+                hi += *(const f32x4 *)(part + (size_t)k * n + 8 * i + 4);
+            }
+        }
+        float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        if (ep.rx) {
+            const h16x8 rx8 = *(const h16x8 *)(ep.rx + col), mx8 = *(const h16x8 *)(ep.mx + col);
+            const float s0t = ep.s0[t], s2t = ep.s2[t];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[e] = epi_affine(v[e], (float)rx8[e], (float)mx8[e], s0t, s2t);
+        }
+        if (ep.raw_f32) {
+            float *yo = (float *)Y + (size_t)t * ldy + col;
+            *(f32x4 *)yo = f32x4{v[0], v[1], v[2], v[3]};
+            *(f32x4 *)(yo + 4) = f32x4{v[4], v[5], v[6], v[7]};
+            continue;
+        }
+        h16x8 res8 = {}, gate8 = {};
+        if (ep.act == ACT_RESIDUAL || ep.act == ACT_GATED_RESIDUAL) res8 = *(const h16x8 *)(ep.res + (size_t)t * ep.ldres + col);
+        if (ep.act == ACT_GATED_RESIDUAL) gate8 = *(const h16x8 *)(ep.gate + (size_t)t * ep.ldgate + col);
+        float o[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) o[e] = epi_act(v[e], (float)res8[e], (float)gate8[e], ep);
+        if (ep.out_dtype == RWKV_DT_F32) {
+            float *yo = (float *)Y + (size_t)t * ldy + col;
+            *(f32x4 *)yo = f32x4{round_h(o[0]), round_h(o[1]), round_h(o[2]), round_h(o[3])};
+            *(f32x4 *)(yo + 4) = f32x4{round_h(o[4]), round_h(o[5]), round_h(o[6]), round_h(o[7])};
+        } else {
+            h16x8 y8;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) y8[e] = (h16)o[e];
+            *(h16x8 *)((rwkv_half *)Y + (size_t)t * ldy + col) = y8;
+        }
+    }
+}
+
+DEV void splitk_rows8_any(int T, int M, int KS, const float *__restrict__ part, void *Y, int64_t ldy, const GemmEpi &ep,
+                          int64_t first, int64_t stride) {
+    switch (KS) {
+        case 2: splitk_rows8<2>(T, M, KS, part, Y, ldy, ep, first, stride); break;
+        case 4: splitk_rows8<4>(T, M, KS, part, Y, ldy, ep, first, stride); break;
+        case 8: splitk_rows8<8>(T, M, KS, part, Y, ldy, ep, first, stride); break;
+        default: splitk_rows8<0>(T, M, KS, part, Y, ldy, ep, first, stride); break;
+    }
+}
+
+__global__ __launch_bounds__(256) void splitk_epilogue8_kernel(int T, int M, int KS, const float *__restrict__ part, void *Y,
+                                                               int64_t ldy, GemmEpi ep) {
+    splitk_rows8_any(T, M, KS, part, Y, ldy, ep, (int64_t)blockIdx.x * 256 + threadIdx.x, (int64_t)gridDim.x * 256);
+}
+
 template <bool W_U8, int BT, int BM, int WT, int WM, int PF, bool SPLIT>
 DEV void gemm_body(int T, int N, int M, const h16 *__restrict__ A, int64_t lda, const void *__restrict__ Wv, int64_t ldw,
                    void *__restrict__ Y, int64_t ldy, const GemmEpi &ep, int nk_split, float *__restrict__ part) {
@@ -586,23 +659,11 @@ int launch_dma_group(const GemmGroup &g, int n, int64_t T, int64_t N, int64_t gr
     return RWKV_OK;
 }
 
-// second pass of a split group: member blockIdx.y, as splitk_epilogue_kernel
-__global__ __launch_bounds__(256) void splitk_group_epilogue_kernel(int T, int KS, GemmGroup g) {
-    const int gi = blockIdx.y, M = g.M[gi];
-    const float *__restrict__ part = g.part[gi];
-    const int64_t n4 = (int64_t)T * M / 4, n = (int64_t)T * M;
-    const int m4 = M / 4;
-    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n4; i += (int64_t)gridDim.x * 256) {
-        const int t = (int)(i / m4), m = (int)(i - (int64_t)t * m4) * 4;
-        f32x4 v = *(const f32x4 *)(part + 4 * i);
-        for (int k = 1; k < KS; ++k) v += *(const f32x4 *)(part + (size_t)k * n + 4 * i);
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            float rxm = 1.f, mxm = 0.f;
-            if (g.ep[gi].rx) { rxm = h2f(g.ep[gi].rx[m + e]); mxm = h2f(g.ep[gi].mx[m + e]); }
-            gemm_epilogue(v[e], t, m + e, rxm, mxm, g.ep[gi], g.Y[gi], M);
-        }
-    }
+// second pass of a split group launch: member blockIdx.y, as splitk_epilogue8_kernel
+__global__ __launch_bounds__(256) void splitk_group_epilogue8_kernel(int T, int KS, GemmGroup g) {
+    const int gi = blockIdx.y;
+    splitk_rows8_any(T, g.M[gi], KS, g.part[gi], g.Y[gi], g.M[gi], g.ep[gi], (int64_t)blockIdx.x * 256 + threadIdx.x,
+                     (int64_t)gridDim.x * 256);
 }
 
 struct PrepGroup {
@@ -783,8 +844,8 @@ int launch_dma(int64_t T, int64_t N, int64_t M, const rwkv_half *A, int64_t lda,
         hipLaunchKernelGGL((gemm_dma_kernel<W_U8, true, TM, TN>), dim3((unsigned)tiles, (unsigned)ks), dim3(512), lds, st, (int)T, (int)N,
                            (int)M, (const h16 *)A, lda, W, ldw, Y, ldy, ep, nk / ks, ep.splitk_ws);
         const int64_t n = T * M;
-        const unsigned blocks = (unsigned)((n + 1023) / 1024 < 16384 ? (n + 1023) / 1024 : 16384);
-        hipLaunchKernelGGL(splitk_epilogue_kernel, dim3(blocks), dim3(256), 0, st, (int)T, (int)M, ks, ep.splitk_ws, Y, ldy, ep);
+        const unsigned blocks = (unsigned)((n + 2047) / 2048 < 16384 ? (n + 2047) / 2048 : 16384);
+        hipLaunchKernelGGL(splitk_epilogue8_kernel, dim3(blocks), dim3(256), 0, st, (int)T, (int)M, ks, ep.splitk_ws, Y, ldy, ep);
     } else {
         hipLaunchKernelGGL((gemm_dma_kernel<W_U8, false, TM, TN>), dim3((unsigned)tiles), dim3(512), lds, st, (int)T, (int)N, (int)M,
                            (const h16 *)A, lda, W, ldw, Y, ldy, ep, nk, (float *)nullptr);
@@ -904,8 +965,8 @@ int gemm_group_launch(bool w_u8, int n, int64_t T, int64_t N, const rwkv_half *c
         else rc = w_u8 ? launch_dma_group<true, 128, 128>(g, n, T, N, tiles, ks, st) : launch_dma_group<false, 128, 128>(g, n, T, N, tiles, ks, st);
         if (rc) return rc;
         if (ks > 1) {
-            const unsigned blocks = (unsigned)std::min<int64_t>((max_out + 1023) / 1024, 16384);
-            hipLaunchKernelGGL(splitk_group_epilogue_kernel, dim3(blocks, (unsigned)n), dim3(256), 0, st, (int)T, ks, g);
+            const unsigned blocks = (unsigned)std::min<int64_t>((max_out + 2047) / 2048, 16384);
+            hipLaunchKernelGGL(splitk_group_epilogue8_kernel, dim3(blocks, (unsigned)n), dim3(256), 0, st, (int)T, ks, g);
         }
         RWKV_LAUNCH_CHECK();
         return RWKV_OK;
