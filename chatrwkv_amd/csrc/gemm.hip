@@ -799,13 +799,13 @@ bool dma_ok(bool w_u8, int64_t N, int64_t M, const void *A, int64_t lda, const v
 // `tiles` tiles of nk k-tiles split c ways run in whole rounds over the 256 CUs; a k-tile step takes 1.75 us with
 // the 256 x 256 tile and 0.573 us with the 128 x 128 one (a quarter of the work in a third of the time); every
 // round adds its fill, drain and epilogue (10 steps; 4.3 for a split launch, whose epilogue is the reduction pass;
-// 12.8 for the small tile, 5.5 where two workgroups per CU overlap); the reduction pass of a split takes 5.3 us
-// per slab and 16 MB of fp32 output.
+// 12.8 for the small tile, 5.5 where two workgroups per CU overlap); the reduction pass of a split takes 2.5 us
+// + 3.6 us per slab and 16 MB of fp32 output, at least 4.5 us.
 double dma_cost(int64_t tiles, int nk, int c, bool small_tile, size_t out_bytes) {
     const int64_t rounds = (tiles * c + 255) / 256;
     const double step = small_tile ? 0.573 : 1.75;
     const double extra = small_tile ? (rounds > 1 ? 5.5 : 12.8) : (c > 1 ? 4.3 : 10.0);
-    return (double)rounds * (nk / c + extra) * step + (c > 1 ? 5.3 * c * (double)out_bytes / (16 << 20) : 0.0);
+    return (double)rounds * (nk / c + extra) * step + (c > 1 ? std::max(4.5, 2.5 + 3.6 * c * (double)out_bytes / (16 << 20)) : 0.0);
 }
 
 // the K split (1..8, whole k-tiles, at least 8 per split, slabs within ws_bytes) of least cost
