@@ -97,12 +97,12 @@ struct Mix2Args {
 // and reused for every token of the tile; the sum runs in index order.
 template <int MIX2_TT>
 __global__ __launch_bounds__(256) void v6_mix2_kernel(Mix2Args a) {
-    __shared__ float st1[MIX2_TT][64];
+    __shared__ __align__(16) float st1[64][MIX2_TT];   // [i][token]: the tokens of one i are read with 16-byte LDS loads
     const int t0 = blockIdx.x * MIX2_TT, c = blockIdx.y * 256 + threadIdx.x, j = blockIdx.z, R = a.R, C = a.C;
     const int nt = min(MIX2_TT, a.T - t0);
     for (int i = threadIdx.x; i < nt * R; i += 256) {
         const int tt = i / R, r = i - tt * R;
-        st1[tt][r] = h2f(a.t1[(size_t)(t0 + tt) * 5 * R + j * R + r]);
+        st1[r][tt] = h2f(a.t1[(size_t)(t0 + tt) * 5 * R + j * R + r]);
     }
     __syncthreads();
     if (c >= C) return;
@@ -120,7 +120,7 @@ __global__ __launch_bounds__(256) void v6_mix2_kernel(Mix2Args a) {
             if (i0 + i < R) {
                 const float wf = h2f(wv[i]);
 #pragma unroll
-                for (int tt = 0; tt < MIX2_TT; ++tt) m[tt] += st1[tt][i0 + i] * wf;
+                for (int tt = 0; tt < MIX2_TT; ++tt) m[tt] += st1[i0 + i][tt] * wf;
             }
     }
 #pragma unroll
