@@ -412,7 +412,8 @@ __global__ __launch_bounds__(256) void wkv56_split_kernel(Wkv56Args a) {
             q.w4 = WMODE == 2 ? *(const f32x4 *)&sw[tt][4 * g] : f32x4{};
             return q;
         };
-        auto step = [&](const Tok &q, int tt) {
+        // this thread's share of y for one token (before the sum over the 16 key groups), and the state update
+        auto partial = [&](const Tok &q) {
             float y = 0.f;
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
@@ -420,16 +421,28 @@ __global__ __launch_bounds__(256) void wkv56_split_kernel(Wkv56Args a) {
                 y += q.r4[e] * (u4[e] * x + s[e]);
                 s[e] = s[e] * (WMODE == 2 ? q.w4[e] : wc[e]) + x;
             }
-            y = row16_sum(y);
+            return y;
+        };
+        auto step = [&](const Tok &q, int tt) {
+            const float y = row16_sum(partial(q));
             if (g == 0) a.y[(size_t)(t0 + tt) * C + h * HS + i] = y;
         };
-        // four tokens per pass: their LDS reads are issued together, so the read latency is paid once per four
+        // four tokens per pass: their LDS reads are issued together, so the read latency is paid once per four, and
+        // in a full pass the four row sums (independent of the state chain) run interleaved
         for (int tt = 0; tt < nt; tt += 4) {
             const Tok q0 = ldtok(tt), q1 = ldtok(tt + 1), q2 = ldtok(tt + 2), q3 = ldtok(tt + 3);
-            step(q0, tt);
-            if (tt + 1 < nt) step(q1, tt + 1);
-            if (tt + 2 < nt) step(q2, tt + 2);
-            if (tt + 3 < nt) step(q3, tt + 3);
+            if (tt + 3 < nt) {
+                float y0 = partial(q0), y1 = partial(q1), y2 = partial(q2), y3 = partial(q3);
+                y0 = row16_sum(y0); y1 = row16_sum(y1); y2 = row16_sum(y2); y3 = row16_sum(y3);
+                if (g == 0) {
+                    float *yo = a.y + (size_t)(t0 + tt) * C + h * HS + i;
+                    yo[0] = y0; yo[(size_t)C] = y1; yo[2 * (size_t)C] = y2; yo[3 * (size_t)C] = y3;
+                }
+            } else {
+                step(q0, tt);
+                if (tt + 1 < nt) step(q1, tt + 1);
+                if (tt + 2 < nt) step(q2, tt + 2);
+            }
         }
     }
 #pragma unroll
