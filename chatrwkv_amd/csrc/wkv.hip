@@ -427,21 +427,27 @@ __global__ __launch_bounds__(256) void wkv56_split_kernel(Wkv56Args a) {
             const float y = row16_sum(partial(q));
             if (g == 0) a.y[(size_t)(t0 + tt) * C + h * HS + i] = y;
         };
-        // four tokens per pass: their LDS reads are issued together, so the read latency is paid once per four, and
-        // in a full pass the four row sums (independent of the state chain) run interleaved
-        for (int tt = 0; tt < nt; tt += 4) {
-            const Tok q0 = ldtok(tt), q1 = ldtok(tt + 1), q2 = ldtok(tt + 2), q3 = ldtok(tt + 3);
-            if (tt + 3 < nt) {
-                float y0 = partial(q0), y1 = partial(q1), y2 = partial(q2), y3 = partial(q3);
-                y0 = row16_sum(y0); y1 = row16_sum(y1); y2 = row16_sum(y2); y3 = row16_sum(y3);
+        // eight tokens per pass (TS2 % 8 == 0): their LDS reads are issued together, so the read latency is paid once per
+        // eight, and in a full pass the eight row sums (independent of the state chain) run interleaved
+        for (int tt = 0; tt < nt; tt += 8) {
+            Tok q[8];
+#pragma unroll
+            for (int p = 0; p < 8; ++p) q[p] = ldtok(tt + p);
+            if (tt + 7 < nt) {
+                float y[8];
+#pragma unroll
+                for (int p = 0; p < 8; ++p) y[p] = partial(q[p]);
+#pragma unroll
+                for (int p = 0; p < 8; ++p) y[p] = row16_sum(y[p]);
                 if (g == 0) {
                     float *yo = a.y + (size_t)(t0 + tt) * C + h * HS + i;
-                    yo[0] = y0; yo[(size_t)C] = y1; yo[2 * (size_t)C] = y2; yo[3 * (size_t)C] = y3;
+#pragma unroll
+                    for (int p = 0; p < 8; ++p) yo[p * (size_t)C] = y[p];
                 }
             } else {
-                step(q0, tt);
-                if (tt + 1 < nt) step(q1, tt + 1);
-                if (tt + 2 < nt) step(q2, tt + 2);
+#pragma unroll
+                for (int p = 0; p < 7; ++p)
+                    if (tt + p < nt) step(q[p], tt + p);
             }
         }
     }
