@@ -188,16 +188,19 @@ __global__ __launch_bounds__(256) void wkv7_kernel(Wkv7Args a) {
             q.b4 = *(const f32x4 *)&sb[tt][4 * g];
             return q;
         };
-        auto step = [&](const Tok &q, int tt) {
-            float p = (q.a4[0] * s[0] + q.a4[1] * s[1]) + (q.a4[2] * s[2] + q.a4[3] * s[3]);
-            float yw = (q.wr4[0] * s[0] + q.wr4[1] * s[1]) + (q.wr4[2] * s[2] + q.wr4[3] * s[3]);
+        // state update of one token; returns this thread's share of the read-out sum, p = the summed sa term
+        auto advance = [&](const Tok &q, float &p) {
+            p = (q.a4[0] * s[0] + q.a4[1] * s[1]) + (q.a4[2] * s[2] + q.a4[3] * s[3]);
+            const float yw = (q.wr4[0] * s[0] + q.wr4[1] * s[1]) + (q.wr4[2] * s[2] + q.wr4[3] * s[3]);
             f32x4 kv;
 #pragma unroll
             for (int e = 0; e < 4; ++e) kv[e] = s[e] * q.w4[e] + q.k4[e] * q.vi;
             p = row16_sum(p);
-            yw = row16_sum(yw);
 #pragma unroll
             for (int e = 0; e < 4; ++e) s[e] = kv[e] + p * q.b4[e];
+            return yw;
+        };
+        auto store = [&](const Tok &q, int tt, float yw, float p) {
             if (g == 0) {
                 const float y = yw + q.vi * q.kr + p * q.br;
                 const size_t o = (size_t)(t0 + tt) * C + h * HS7 + i;
@@ -205,13 +208,26 @@ __global__ __launch_bounds__(256) void wkv7_kernel(Wkv7Args a) {
                 else ((rwkv_half *)a.y)[o] = f2h(y);
             }
         };
-        // four tokens per pass: their LDS reads are issued together, so the read latency is paid once per four
+        // four tokens per pass: their LDS reads are issued together, so the read latency is paid once per four; in a
+        // full pass the four read-out row sums, which are not on the state chain, run interleaved after the updates
         for (int tt = 0; tt < nt; tt += 4) {
-            const Tok q0 = ldtok(tt), q1 = ldtok(tt + 1), q2 = ldtok(tt + 2), q3 = ldtok(tt + 3);
-            step(q0, tt);
-            if (tt + 1 < nt) step(q1, tt + 1);
-            if (tt + 2 < nt) step(q2, tt + 2);
-            if (tt + 3 < nt) step(q3, tt + 3);
+            const Tok q[4] = {ldtok(tt), ldtok(tt + 1), ldtok(tt + 2), ldtok(tt + 3)};
+            float yw[4], p[4];
+            if (tt + 3 < nt) {
+#pragma unroll
+                for (int u = 0; u < 4; ++u) yw[u] = advance(q[u], p[u]);
+#pragma unroll
+                for (int u = 0; u < 4; ++u) yw[u] = row16_sum(yw[u]);
+#pragma unroll
+                for (int u = 0; u < 4; ++u) store(q[u], tt + u, yw[u], p[u]);
+            } else {
+#pragma unroll
+                for (int u = 0; u < 3; ++u)
+                    if (tt + u < nt) {
+                        yw[u] = row16_sum(advance(q[u], p[u]));
+                        store(q[u], tt + u, yw[u], p[u]);
+                    }
+            }
         }
     }
     *(f32x4 *)S = s;
