@@ -559,7 +559,7 @@ DEV void gemm_dma_body(int T, int N, int M, const h16 *__restrict__ A, int64_t l
     };
 
     if constexpr (SPLIT) {
-        // partial sums go to this split's fp32 slab; splitk_epilogue_kernel adds the slabs and finishes
+        // partial sums go to this split's fp32 slab; splitk_epilogue8_kernel adds the slabs and finishes
         float *slab = part + (size_t)split * T * M;
 #pragma unroll
         for (int b = 0; b < NI; ++b) {

@@ -208,21 +208,25 @@ __global__ __launch_bounds__(256) void wkv7_kernel(Wkv7Args a) {
                 else ((rwkv_half *)a.y)[o] = f2h(y);
             }
         };
-        // four tokens per pass: their LDS reads are issued together, so the read latency is paid once per four; in a
-        // full pass the four read-out row sums, which are not on the state chain, run interleaved after the updates
-        for (int tt = 0; tt < nt; tt += 4) {
-            const Tok q[4] = {ldtok(tt), ldtok(tt + 1), ldtok(tt + 2), ldtok(tt + 3)};
-            float yw[4], p[4];
-            if (tt + 3 < nt) {
+        // PASS tokens per pass (TS7 % PASS == 0): their LDS reads are issued together, so the read latency is paid once
+        // per pass; in a full pass the read-out row sums, which are not on the state chain, run interleaved after the
+        // state updates
+        constexpr int PASS = 4;   // 8 was slower here (138 against 128 us per 1024 tokens): 23 operand registers per token
+        for (int tt = 0; tt < nt; tt += PASS) {
+            Tok q[PASS];
 #pragma unroll
-                for (int u = 0; u < 4; ++u) yw[u] = advance(q[u], p[u]);
+            for (int u = 0; u < PASS; ++u) q[u] = ldtok(tt + u);
+            float yw[PASS], p[PASS];
+            if (tt + PASS - 1 < nt) {
 #pragma unroll
-                for (int u = 0; u < 4; ++u) yw[u] = row16_sum(yw[u]);
+                for (int u = 0; u < PASS; ++u) yw[u] = advance(q[u], p[u]);
 #pragma unroll
-                for (int u = 0; u < 4; ++u) store(q[u], tt + u, yw[u], p[u]);
+                for (int u = 0; u < PASS; ++u) yw[u] = row16_sum(yw[u]);
+#pragma unroll
+                for (int u = 0; u < PASS; ++u) store(q[u], tt + u, yw[u], p[u]);
             } else {
 #pragma unroll
-                for (int u = 0; u < 3; ++u)
+                for (int u = 0; u < PASS - 1; ++u)
                     if (tt + u < nt) {
                         yw[u] = row16_sum(advance(q[u], p[u]));
                         store(q[u], tt + u, yw[u], p[u]);
