@@ -403,6 +403,33 @@ def test_v56_side_stream_path(ver):
         assert np.abs(_np(s) - _np(s2)).max() <= 1e-2 * scale, i
 
 
+@pytest.mark.parametrize("ver", [5, 5.2, 6])
+def test_v56_width_not_a_multiple_of_128(ver):
+    """n_embd 192 / ffn 704: the square products of a sequence call cannot share a grouped launch (its tiles are
+    128 wide), so each runs alone on the activation that the LN / mix launch has already scaled and summed
+    (RWKV-5 time mix, RWKV-5/6 channel mix).  Against the oracle, and against the same prompt in calls of 1, 5
+    and 7 tokens."""
+    cfg = dict(n_layer=2, n_embd=192, n_ffn=704, vocab=300)
+    ck = synth.make_checkpoint(version=ver, seed=192 + int(ver * 10), **cfg)
+    m, o = _rwkv()(ck, "cuda fp16i8", verbose=False), OracleRWKV(ck, "cuda fp16i8")
+    toks = synth.random_tokens(40, cfg["vocab"], seed=9)
+    out, st = m.forward(toks, None, full_output=True)
+    torch.cuda.synchronize()
+    oo, ost = o.forward(toks, None, full_output=True)
+    d = float(np.abs(_np(out) - oo).max())
+    assert d <= LOGIT_TOL, d
+    assert _argmax_agree(_np(out), oo, d)
+    st2, a = None, 0
+    for n in (1, 5, 7, 1, 26):
+        out2, st2 = m.forward(toks[a:a + n], st2)
+        a += n
+    assert a == 40 and np.abs(_np(out2) - _np(out)[-1]).max() <= LOGIT_TOL
+    for i, (s, s2, ref) in enumerate(zip(st, st2, ost)):
+        scale = max(float(np.abs(ref.astype(np.float32)).max()), 1.0)
+        assert np.abs(_np(s) - ref.astype(np.float32)).max() <= 1e-2 * scale, i
+        assert np.abs(_np(s) - _np(s2)).max() <= 1e-2 * scale, i
+
+
 @pytest.mark.parametrize("ver", [4, 5.2, 6])
 @pytest.mark.parametrize("strat", ["cuda fp16i8 *2 -> cuda fp16", "cuda fp16 *1 -> cuda fp16i8"])
 def test_mixed_weight_types_on_one_gpu(ver, strat):
