@@ -143,9 +143,169 @@ __global__ __launch_bounds__(256) void ln_f32_f16_kernel(int C, const float *__r
     for (int j = threadIdx.x; j < C; j += blockDim.x) y[j] = f2h((x[j] - mean) * rstd * w[j] + b[j]);
 }
 
+// N workgroup sums with one pair of barriers; each is formed exactly as block_sum forms it.  red: N * 4 floats.
+template <int N>
+DEV void block_sum_n(float (&v)[N], float *red) {
+    const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
+#pragma unroll
+    for (int i = 0; i < N; ++i) v[i] = wave_sum(v[i]);
+    __syncthreads();
+    if (lane == 0)
+#pragma unroll
+        for (int i = 0; i < N; ++i) red[i * 4 + wid] = v[i];
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+        float t = 0.f;
+        for (int w = 0; w < nw; ++w) t += red[i * 4 + w];
+        v[i] = t;
+    }
+}
+
+// lnmix_seq_kernel with a short dependent chain, for C <= 2048 CH: a thread's chunks of the row, of the previous row
+// and of the LayerNorm vectors are requested together at the top and kept in registers, the statistics of the two
+// rows share their barriers, and so do the 2 NJ sums at the end: two global round trips and three rounds of
+// barriers per workgroup instead of five and ten.  Every value is formed by the same thread with the same
+// operations in the same order as in lnmix_seq_kernel, so the two agree bit for bit.
+template <int NJ, int CH>
+__global__ __launch_bounds__(256) void lnmix_seq_fast_kernel(SeqMixArgs a) {
+    __shared__ float red[4 * 2 * NJ > 8 ? 4 * 2 * NJ : 8];
+    const int t = blockIdx.x, C = a.C, nch = C >> 3;
+    const rwkv_half *x = a.x + (size_t)t * C;
+    const bool shift = a.sx != nullptr, prev_row = shift && t > 0;
+    const rwkv_half *xp = prev_row ? x - C : x;
+    h16x8 xv[CH], pxv[CH], wv[CH], bv[CH];
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        const int j8 = min((int)threadIdx.x + c * 256, nch - 1);   // chunks past the end repeat the last one (unused)
+        xv[c] = *(const h16x8 *)(x + 8 * j8);
+        pxv[c] = *(const h16x8 *)(xp + 8 * j8);
+        wv[c] = *(const h16x8 *)(a.ln_w + 8 * j8);
+        bv[c] = *(const h16x8 *)(a.ln_b + 8 * j8);
+    }
+    float st[2] = {0.f, 0.f};
+#pragma unroll
+    for (int c = 0; c < CH; ++c)
+        if ((int)threadIdx.x + c * 256 < nch) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) { st[0] += (float)xv[c][e]; st[1] += (float)pxv[c][e]; }
+        }
+    block_sum_n<2>(st, red);
+    const float mean = st[0] / C, pmean = st[1] / C;
+    st[0] = st[1] = 0.f;
+#pragma unroll
+    for (int c = 0; c < CH; ++c)
+        if ((int)threadIdx.x + c * 256 < nch) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float d = (float)xv[c][e] - mean, pd = (float)pxv[c][e] - pmean;
+                st[0] += d * d;
+                st[1] += pd * pd;
+            }
+        }
+    block_sum_n<2>(st, red);
+    const float rstd = rsqrtf(st[0] / C + LN_EPS), prstd = rsqrtf(st[1] / C + LN_EPS);
+    float acc[2 * NJ];
+#pragma unroll
+    for (int i = 0; i < 2 * NJ; ++i) acc[i] = 0.f;
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        const int j8 = threadIdx.x + c * 256;
+        if (j8 >= nch) break;
+        h16x8 xx, pv;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) xx[e] = (h16)(((float)xv[c][e] - mean) * rstd * (float)wv[c][e] + (float)bv[c][e]);
+        pv = xx;
+        if (shift) {
+            if (t > 0) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    pv[e] = (h16)(((float)pxv[c][e] - pmean) * prstd * (float)wv[c][e] + (float)bv[c][e]);
+            } else {
+                pv = *(const h16x8 *)(a.sx + 8 * j8);
+            }
+        }
+        if (a.xx_last && t == a.T - 1) *(h16x8 *)(a.xx_last + 8 * j8) = xx;
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+            h16x8 kx = xx;
+            if (a.mix[j]) {
+                const h16x8 mv = *(const h16x8 *)(a.mix[j] + 8 * j8);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const float m = (float)mv[e];
+                    kx[e] = a.maa_form ? (h16)((float)xx[e] + (float)(h16)((float)(h16)((float)pv[e] - (float)xx[e]) * m))
+                                       : (h16)((float)xx[e] * m + (float)pv[e] * (1.f - m));
+                }
+            }
+            h16x8 o = kx;
+            if (a.ry[j]) {
+                const h16x8 rv = *(const h16x8 *)(a.ry[j] + 8 * j8);
+                const h16x8 yv = *(const h16x8 *)(a.my[j] + 8 * j8);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const float k = (float)kx[e];
+                    o[e] = (h16)(k * (float)rv[e]);
+                    acc[2 * j] += k;
+                    acc[2 * j + 1] += k * (float)yv[e];
+                }
+            }
+            *(h16x8 *)(a.xs[j] + (size_t)t * C + 8 * j8) = o;
+        }
+    }
+    bool any = false;
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) any = any || a.ry[j];
+    if (any) {
+        block_sum_n<2 * NJ>(acc, red);
+        if (threadIdx.x == 0)
+#pragma unroll
+            for (int j = 0; j < NJ; ++j)
+                if (a.ry[j]) { a.s0[j][t] = acc[2 * j]; a.s2[j][t] = acc[2 * j + 1]; }
+    }
+    // The new token-shift state is LN(x[T-1]).  Only row 0 reads the old one, so row 0's workgroup writes the new
+    // one once its own reads are done (each thread overwrites exactly the chunks it has read): no second launch.
+    if (a.state_out && t == 0) {
+        const rwkv_half *xl = a.x + (size_t)(a.T - 1) * C;
+        float lm = mean, lr = rstd;
+        if (a.T > 1) row_stats(xl, C, red, lm, lr);
+        for (int j8 = threadIdx.x; j8 < nch; j8 += blockDim.x) {
+            const h16x8 lv = *(const h16x8 *)(xl + 8 * j8);
+            const h16x8 lw = *(const h16x8 *)(a.ln_w + 8 * j8);
+            const h16x8 lb = *(const h16x8 *)(a.ln_b + 8 * j8);
+            h16x8 xx;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) xx[e] = (h16)(((float)lv[e] - lm) * lr * (float)lw[e] + (float)lb[e]);
+            *(h16x8 *)(a.state_out + 8 * j8) = xx;
+        }
+    }
+}
+
 }  // namespace
 
+template <int CH>
+static bool lnmix_seq_fast_launch(const SeqMixArgs &a, int nj, hipStream_t st) {
+    const dim3 grid((unsigned)a.T), block(256);
+    switch (nj) {
+        case 1: hipLaunchKernelGGL((lnmix_seq_fast_kernel<1, CH>), grid, block, 0, st, a); break;
+        case 2: hipLaunchKernelGGL((lnmix_seq_fast_kernel<2, CH>), grid, block, 0, st, a); break;
+        case 3: hipLaunchKernelGGL((lnmix_seq_fast_kernel<3, CH>), grid, block, 0, st, a); break;
+        case 4: hipLaunchKernelGGL((lnmix_seq_fast_kernel<4, CH>), grid, block, 0, st, a); break;
+        case 6: hipLaunchKernelGGL((lnmix_seq_fast_kernel<6, CH>), grid, block, 0, st, a); break;
+        default: return false;
+    }
+    return true;
+}
+
 int lnmix_seq_launch(const SeqMixArgs &a, int nj, hipStream_t st) {
+    // rows of up to 8192 channels: the register-resident kernel (1, 2 or 4 chunks of 8 channels per thread)
+    if (a.C <= 8192 && (nj == 1 || nj == 2 || nj == 3 || nj == 4 || nj == 6)) {
+        if (a.C <= 2048) lnmix_seq_fast_launch<1>(a, nj, st);
+        else if (a.C <= 4096) lnmix_seq_fast_launch<2>(a, nj, st);
+        else lnmix_seq_fast_launch<4>(a, nj, st);
+        RWKV_LAUNCH_CHECK();
+        return RWKV_OK;
+    }
     const dim3 grid((unsigned)a.T), block(256);
     switch (nj) {
         case 1: hipLaunchKernelGGL(lnmix_seq_kernel<1>, grid, block, 0, st, a); break;
