@@ -80,6 +80,26 @@ DEV float block_sum(float v, float *red) {
     return t;
 }
 
+// Sum K values over the workgroup at once (one pair of barriers); every thread gets all K totals, each formed
+// exactly as block_sum forms it.  `red` is LDS scratch of at least K * (blockDim.x / 64) floats.
+template <int K>
+DEV void block_sum_n(float (&v)[K], float *red) {
+    const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
+#pragma unroll
+    for (int k = 0; k < K; ++k) v[k] = wave_sum(v[k]);
+    __syncthreads();
+    if (lane == 0)
+#pragma unroll
+        for (int k = 0; k < K; ++k) red[k * nw + wid] = v[k];
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+        float t = 0.f;
+        for (int i = 0; i < nw; ++i) t += red[k * nw + i];
+        v[k] = t;
+    }
+}
+
 // ---- uint8 -> fp16 pairs -------------------------------------------------------------------
 // Bytes b0..b3 of `v` become the fp16 values (1024 + b): placing a byte under the exponent
 // byte 0x64 yields exactly 1024 + b.  lo = (b0, b1), hi = (b2, b3).

@@ -121,26 +121,6 @@ DEV void wave_rows_dot_f16(const h16 *const (&rows)[R], const h16 *const (&xs)[R
     for (int r = 0; r < R; ++r) acc[r] = wave_sum(acc[r]);
 }
 
-// Sum K values over the workgroup at once; every thread gets all K totals.
-// `red` is LDS scratch of at least K * (blockDim.x / 64) floats.
-template <int K>
-DEV void block_sum_n(float (&v)[K], float *red) {
-    const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
-#pragma unroll
-    for (int k = 0; k < K; ++k) v[k] = wave_sum(v[k]);
-    __syncthreads();
-    if (lane == 0)
-#pragma unroll
-        for (int k = 0; k < K; ++k) red[k * nw + wid] = v[k];
-    __syncthreads();
-#pragma unroll
-    for (int k = 0; k < K; ++k) {
-        float t = 0.f;
-        for (int i = 0; i < nw; ++i) t += red[k * nw + i];
-        v[k] = t;
-    }
-}
-
 // A register tile of weights: U 16-byte segments of R rows per lane.  Loading and consuming are
 // separate steps so that a kernel can put the loads of its first tile in flight *before* it
 // builds the activation vector (weights do not depend on activations).  A segment is 16 bytes

@@ -143,25 +143,6 @@ __global__ __launch_bounds__(256) void ln_f32_f16_kernel(int C, const float *__r
     for (int j = threadIdx.x; j < C; j += blockDim.x) y[j] = f2h((x[j] - mean) * rstd * w[j] + b[j]);
 }
 
-// N workgroup sums with one pair of barriers; each is formed exactly as block_sum forms it.  red: N * 4 floats.
-template <int N>
-DEV void block_sum_n(float (&v)[N], float *red) {
-    const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
-#pragma unroll
-    for (int i = 0; i < N; ++i) v[i] = wave_sum(v[i]);
-    __syncthreads();
-    if (lane == 0)
-#pragma unroll
-        for (int i = 0; i < N; ++i) red[i * 4 + wid] = v[i];
-    __syncthreads();
-#pragma unroll
-    for (int i = 0; i < N; ++i) {
-        float t = 0.f;
-        for (int w = 0; w < nw; ++w) t += red[i * 4 + w];
-        v[i] = t;
-    }
-}
-
 // lnmix_seq_kernel with a short dependent chain, for C <= 2048 CH: a thread's chunks of the row, of the previous row
 // and of the LayerNorm vectors are requested together at the top and kept in registers, the statistics of the two
 // rows share their barriers, and so do the 2 NJ sums at the end: two global round trips and three rounds of

@@ -23,9 +23,12 @@ struct Mix1Args {
 };
 
 // grid T x 256 threads: xx = LN1(x[t]); sxd = prev - xx; xxx = xx + sxd * maa_x.
+// Rows of up to 2048 CH channels keep a thread's chunks of the row and of the previous row in registers from one round
+// of loads, and the four sums of the two rows' statistics share one pair of barriers.
+template <int CH>
 __global__ __launch_bounds__(256) void v6_mix1_kernel(Mix1Args a) {
-    __shared__ float red[8];
-    const int t = blockIdx.x, C = a.C;
+    __shared__ float red[16];
+    const int t = blockIdx.x, C = a.C, nch = C >> 3;
     auto stats = [&](const rwkv_half *x, float &mean, float &rstd) {
         float s = 0.f, q = 0.f;
         for (int j8 = threadIdx.x; j8 < (C >> 3); j8 += blockDim.x) {
@@ -39,18 +42,39 @@ __global__ __launch_bounds__(256) void v6_mix1_kernel(Mix1Args a) {
         rstd = rsqrtf(fmaxf(q / C - mean * mean, 0.f) + LN_EPS56);
     };
     const rwkv_half *x = a.x + (size_t)t * C;
-    float mean, rstd, pmean = 0.f, prstd = 0.f;
-    stats(x, mean, rstd);
-    if (t > 0) stats(x - C, pmean, prstd);
-    for (int j8 = threadIdx.x; j8 < (C >> 3); j8 += blockDim.x) {
-        const h16x8 xv = *(const h16x8 *)(x + 8 * j8);
+    const rwkv_half *xp = t > 0 ? x - C : x;
+    h16x8 xr[CH], pr[CH];
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        const int j8 = min((int)threadIdx.x + c * 256, nch - 1);   // chunks past the end repeat the last one (unused)
+        xr[c] = *(const h16x8 *)(x + 8 * j8);
+        pr[c] = *(const h16x8 *)(xp + 8 * j8);
+    }
+    float sq[4] = {0.f, 0.f, 0.f, 0.f};   // sum and sum of squares of the row, of the previous row
+#pragma unroll
+    for (int c = 0; c < CH; ++c)
+        if ((int)threadIdx.x + c * 256 < nch) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float f = (float)xr[c][e], g = (float)pr[c][e];
+                sq[0] += f; sq[1] += f * f; sq[2] += g; sq[3] += g * g;
+            }
+        }
+    block_sum_n<4>(sq, red);
+    float mean = sq[0] / C, rstd = rsqrtf(fmaxf(sq[1] / C - mean * mean, 0.f) + LN_EPS56);
+    const float pmean = sq[2] / C, prstd = rsqrtf(fmaxf(sq[3] / C - pmean * pmean, 0.f) + LN_EPS56);
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        const int j8 = threadIdx.x + c * 256;
+        if (j8 >= nch) break;
+        const h16x8 xv = xr[c];
         const h16x8 wv = *(const h16x8 *)(a.ln_w + 8 * j8), bv = *(const h16x8 *)(a.ln_b + 8 * j8);
         const h16x8 mv = *(const h16x8 *)(a.maa_x + 8 * j8);
         h16x8 xx, pv, sd, xo;
 #pragma unroll
         for (int e = 0; e < 8; ++e) xx[e] = (h16)(((float)xv[e] - mean) * rstd * (float)wv[e] + (float)bv[e]);
         if (t > 0) {
-            const h16x8 pxv = *(const h16x8 *)(x - C + 8 * j8);
+            const h16x8 pxv = pr[c];
 #pragma unroll
             for (int e = 0; e < 8; ++e) pv[e] = (h16)(((float)pxv[e] - pmean) * prstd * (float)wv[e] + (float)bv[e]);
         } else {
@@ -264,7 +288,9 @@ extern "C" int rwkv_v56_forward(const rwkv_v56_model *m, const rwkv_v56_layer_st
                 b.xx = ws.xx_att; b.sxd = nullptr; b.prev = s.att_xx;
             } else {
                 Mix1Args a{(int)T, C, ws.x, l.ln1_w, l.ln1_b, s.att_xx, l.att_mix[0], ws.xx, ws.sxd, ws.xxx, s.att_xx};
-                hipLaunchKernelGGL(v6_mix1_kernel, dim3((unsigned)T), dim3(256), 0, st, a);
+                if (C <= 2048) hipLaunchKernelGGL(v6_mix1_kernel<1>, dim3((unsigned)T), dim3(256), 0, st, a);
+                else if (C <= 4096) hipLaunchKernelGGL(v6_mix1_kernel<2>, dim3((unsigned)T), dim3(256), 0, st, a);
+                else hipLaunchKernelGGL(v6_mix1_kernel<4>, dim3((unsigned)T), dim3(256), 0, st, a);
                 if ((rc = mm(c, lora_mat(l.tm_w1, C, 5 * lm), false, ws.xxx, ACT_TANH, nullptr, nullptr, 1.f, ws.t1))) return rc;
                 b.xx = ws.xx; b.sxd = ws.sxd; b.prev = nullptr;
             }
