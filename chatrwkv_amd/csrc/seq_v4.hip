@@ -146,46 +146,60 @@ __global__ __launch_bounds__(256) void ln_f32_f16_kernel(int C, const float *__r
 // lnmix_seq_kernel with a short dependent chain, for C <= 2048 CH: a thread's chunks of the row, of the previous row
 // and of the LayerNorm vectors are requested together at the top and kept in registers, the statistics of the two
 // rows share their barriers, and so do the 2 NJ sums at the end: two global round trips and three rounds of
-// barriers per workgroup instead of five and ten.  Every value is formed by the same thread with the same
+// barriers per workgroup instead of five and ten (and no longer chain in row 0's workgroup, which forms the new
+// token-shift state).  Every value is formed by the same thread with the same
 // operations in the same order as in lnmix_seq_kernel, so the two agree bit for bit.
 template <int NJ, int CH>
 __global__ __launch_bounds__(256) void lnmix_seq_fast_kernel(SeqMixArgs a) {
-    __shared__ float red[4 * 2 * NJ > 8 ? 4 * 2 * NJ : 8];
+    __shared__ float red[4 * 2 * NJ > 12 ? 4 * 2 * NJ : 12];
+    constexpr bool PRE = NJ * CH <= 8;   // the mix / scale vectors too are requested at the top (registers allow it)
     const int t = blockIdx.x, C = a.C, nch = C >> 3;
     const rwkv_half *x = a.x + (size_t)t * C;
     const bool shift = a.sx != nullptr, prev_row = shift && t > 0;
     const rwkv_half *xp = prev_row ? x - C : x;
-    h16x8 xv[CH], pxv[CH], wv[CH], bv[CH];
+    // Row 0's workgroup also forms the new token-shift state LN(x[T-1]): its statistics ride in the same barriers
+    const bool commit = a.state_out && t == 0;
+    const rwkv_half *xl = commit ? a.x + (size_t)(a.T - 1) * C : x;
+    h16x8 xv[CH], pxv[CH], lv[CH], wv[CH], bv[CH], mv[PRE ? NJ : 1][CH], rv[PRE ? NJ : 1][CH], yv[PRE ? NJ : 1][CH];
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
         const int j8 = min((int)threadIdx.x + c * 256, nch - 1);   // chunks past the end repeat the last one (unused)
         xv[c] = *(const h16x8 *)(x + 8 * j8);
         pxv[c] = *(const h16x8 *)(xp + 8 * j8);
+        lv[c] = *(const h16x8 *)(xl + 8 * j8);
         wv[c] = *(const h16x8 *)(a.ln_w + 8 * j8);
         bv[c] = *(const h16x8 *)(a.ln_b + 8 * j8);
+        if constexpr (PRE) {
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) {
+                if (a.mix[j]) mv[j][c] = *(const h16x8 *)(a.mix[j] + 8 * j8);
+                if (a.ry[j]) { rv[j][c] = *(const h16x8 *)(a.ry[j] + 8 * j8); yv[j][c] = *(const h16x8 *)(a.my[j] + 8 * j8); }
+            }
+        }
     }
-    float st[2] = {0.f, 0.f};
+    float st[3] = {0.f, 0.f, 0.f};
 #pragma unroll
     for (int c = 0; c < CH; ++c)
         if ((int)threadIdx.x + c * 256 < nch) {
 #pragma unroll
-            for (int e = 0; e < 8; ++e) { st[0] += (float)xv[c][e]; st[1] += (float)pxv[c][e]; }
+            for (int e = 0; e < 8; ++e) { st[0] += (float)xv[c][e]; st[1] += (float)pxv[c][e]; st[2] += (float)lv[c][e]; }
         }
-    block_sum_n<2>(st, red);
-    const float mean = st[0] / C, pmean = st[1] / C;
-    st[0] = st[1] = 0.f;
+    block_sum_n<3>(st, red);
+    const float mean = st[0] / C, pmean = st[1] / C, lmean = st[2] / C;
+    st[0] = st[1] = st[2] = 0.f;
 #pragma unroll
     for (int c = 0; c < CH; ++c)
         if ((int)threadIdx.x + c * 256 < nch) {
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-                const float d = (float)xv[c][e] - mean, pd = (float)pxv[c][e] - pmean;
+                const float d = (float)xv[c][e] - mean, pd = (float)pxv[c][e] - pmean, ld = (float)lv[c][e] - lmean;
                 st[0] += d * d;
                 st[1] += pd * pd;
+                st[2] += ld * ld;
             }
         }
-    block_sum_n<2>(st, red);
-    const float rstd = rsqrtf(st[0] / C + LN_EPS), prstd = rsqrtf(st[1] / C + LN_EPS);
+    block_sum_n<3>(st, red);
+    const float rstd = rsqrtf(st[0] / C + LN_EPS), prstd = rsqrtf(st[1] / C + LN_EPS), lrstd = rsqrtf(st[2] / C + LN_EPS);
     float acc[2 * NJ];
 #pragma unroll
     for (int i = 0; i < 2 * NJ; ++i) acc[i] = 0.f;
@@ -211,27 +225,37 @@ __global__ __launch_bounds__(256) void lnmix_seq_fast_kernel(SeqMixArgs a) {
         for (int j = 0; j < NJ; ++j) {
             h16x8 kx = xx;
             if (a.mix[j]) {
-                const h16x8 mv = *(const h16x8 *)(a.mix[j] + 8 * j8);
+                h16x8 m8;
+                if constexpr (PRE) m8 = mv[j][c]; else m8 = *(const h16x8 *)(a.mix[j] + 8 * j8);
 #pragma unroll
                 for (int e = 0; e < 8; ++e) {
-                    const float m = (float)mv[e];
+                    const float m = (float)m8[e];
                     kx[e] = a.maa_form ? (h16)((float)xx[e] + (float)(h16)((float)(h16)((float)pv[e] - (float)xx[e]) * m))
                                        : (h16)((float)xx[e] * m + (float)pv[e] * (1.f - m));
                 }
             }
             h16x8 o = kx;
             if (a.ry[j]) {
-                const h16x8 rv = *(const h16x8 *)(a.ry[j] + 8 * j8);
-                const h16x8 yv = *(const h16x8 *)(a.my[j] + 8 * j8);
+                h16x8 r8, y8;
+                if constexpr (PRE) { r8 = rv[j][c]; y8 = yv[j][c]; }
+                else { r8 = *(const h16x8 *)(a.ry[j] + 8 * j8); y8 = *(const h16x8 *)(a.my[j] + 8 * j8); }
 #pragma unroll
                 for (int e = 0; e < 8; ++e) {
                     const float k = (float)kx[e];
-                    o[e] = (h16)(k * (float)rv[e]);
+                    o[e] = (h16)(k * (float)r8[e]);
                     acc[2 * j] += k;
-                    acc[2 * j + 1] += k * (float)yv[e];
+                    acc[2 * j + 1] += k * (float)y8[e];
                 }
             }
             *(h16x8 *)(a.xs[j] + (size_t)t * C + 8 * j8) = o;
+        }
+        // Only row 0 reads the old state, so row 0's workgroup writes the new one, each thread exactly the chunk it
+        // has just read: no second launch.
+        if (commit) {
+            h16x8 ls;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) ls[e] = (h16)(((float)lv[c][e] - lmean) * lrstd * (float)wv[c][e] + (float)bv[c][e]);
+            *(h16x8 *)(a.state_out + 8 * j8) = ls;
         }
     }
     bool any = false;
@@ -243,22 +267,6 @@ __global__ __launch_bounds__(256) void lnmix_seq_fast_kernel(SeqMixArgs a) {
 #pragma unroll
             for (int j = 0; j < NJ; ++j)
                 if (a.ry[j]) { a.s0[j][t] = acc[2 * j]; a.s2[j][t] = acc[2 * j + 1]; }
-    }
-    // The new token-shift state is LN(x[T-1]).  Only row 0 reads the old one, so row 0's workgroup writes the new
-    // one once its own reads are done (each thread overwrites exactly the chunks it has read): no second launch.
-    if (a.state_out && t == 0) {
-        const rwkv_half *xl = a.x + (size_t)(a.T - 1) * C;
-        float lm = mean, lr = rstd;
-        if (a.T > 1) row_stats(xl, C, red, lm, lr);
-        for (int j8 = threadIdx.x; j8 < nch; j8 += blockDim.x) {
-            const h16x8 lv = *(const h16x8 *)(xl + 8 * j8);
-            const h16x8 lw = *(const h16x8 *)(a.ln_w + 8 * j8);
-            const h16x8 lb = *(const h16x8 *)(a.ln_b + 8 * j8);
-            h16x8 xx;
-#pragma unroll
-            for (int e = 0; e < 8; ++e) xx[e] = (h16)(((float)lv[e] - lm) * lr * (float)lw[e] + (float)lb[e]);
-            *(h16x8 *)(a.state_out + 8 * j8) = xx;
-        }
     }
 }
 
