@@ -27,42 +27,35 @@ struct Mix1Args {
 // of loads, and the four sums of the two rows' statistics share one pair of barriers.
 template <int CH>
 __global__ __launch_bounds__(256) void v6_mix1_kernel(Mix1Args a) {
-    __shared__ float red[16];
+    __shared__ float red[24];
     const int t = blockIdx.x, C = a.C, nch = C >> 3;
-    auto stats = [&](const rwkv_half *x, float &mean, float &rstd) {
-        float s = 0.f, q = 0.f;
-        for (int j8 = threadIdx.x; j8 < (C >> 3); j8 += blockDim.x) {
-            const h16x8 v = *(const h16x8 *)(x + 8 * j8);
-#pragma unroll
-            for (int e = 0; e < 8; ++e) { const float f = (float)v[e]; s += f; q += f * f; }
-        }
-        s = block_sum(s, red);
-        q = block_sum(q, red);
-        mean = s / C;
-        rstd = rsqrtf(fmaxf(q / C - mean * mean, 0.f) + LN_EPS56);
-    };
     const rwkv_half *x = a.x + (size_t)t * C;
     const rwkv_half *xp = t > 0 ? x - C : x;
-    h16x8 xr[CH], pr[CH];
+    // row 0's workgroup also forms the new token-shift state LN1(x[T-1]); its statistics ride in the same barriers
+    const bool commit = t == 0;
+    const rwkv_half *xl = commit ? a.x + (size_t)(a.T - 1) * C : x;
+    h16x8 xr[CH], pr[CH], lr[CH];
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
         const int j8 = min((int)threadIdx.x + c * 256, nch - 1);   // chunks past the end repeat the last one (unused)
         xr[c] = *(const h16x8 *)(x + 8 * j8);
         pr[c] = *(const h16x8 *)(xp + 8 * j8);
+        lr[c] = *(const h16x8 *)(xl + 8 * j8);
     }
-    float sq[4] = {0.f, 0.f, 0.f, 0.f};   // sum and sum of squares of the row, of the previous row
+    float sq[6] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f};   // sum and sum of squares of the row, the previous row, the last row
 #pragma unroll
     for (int c = 0; c < CH; ++c)
         if ((int)threadIdx.x + c * 256 < nch) {
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-                const float f = (float)xr[c][e], g = (float)pr[c][e];
-                sq[0] += f; sq[1] += f * f; sq[2] += g; sq[3] += g * g;
+                const float f = (float)xr[c][e], g = (float)pr[c][e], h = (float)lr[c][e];
+                sq[0] += f; sq[1] += f * f; sq[2] += g; sq[3] += g * g; sq[4] += h; sq[5] += h * h;
             }
         }
-    block_sum_n<4>(sq, red);
-    float mean = sq[0] / C, rstd = rsqrtf(fmaxf(sq[1] / C - mean * mean, 0.f) + LN_EPS56);
+    block_sum_n<6>(sq, red);
+    const float mean = sq[0] / C, rstd = rsqrtf(fmaxf(sq[1] / C - mean * mean, 0.f) + LN_EPS56);
     const float pmean = sq[2] / C, prstd = rsqrtf(fmaxf(sq[3] / C - pmean * pmean, 0.f) + LN_EPS56);
+    const float lmean = sq[4] / C, lrstd = rsqrtf(fmaxf(sq[5] / C - lmean * lmean, 0.f) + LN_EPS56);
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
         const int j8 = threadIdx.x + c * 256;
@@ -89,19 +82,13 @@ __global__ __launch_bounds__(256) void v6_mix1_kernel(Mix1Args a) {
         *(h16x8 *)(a.xx + o) = xx;
         *(h16x8 *)(a.sxd + o) = sd;
         *(h16x8 *)(a.xxx + o) = xo;
-    }
-    // the new token-shift state LN1(x[T-1]): written by row 0's workgroup, the only one that reads the old state,
-    // after its own reads (each thread overwrites exactly the chunks it has read)
-    if (t == 0) {
-        const rwkv_half *xl = a.x + (size_t)(a.T - 1) * C;
-        if (a.T > 1) stats(xl, mean, rstd);
-        for (int j8 = threadIdx.x; j8 < (C >> 3); j8 += blockDim.x) {
-            const h16x8 xv = *(const h16x8 *)(xl + 8 * j8);
-            const h16x8 wv = *(const h16x8 *)(a.ln_w + 8 * j8), bv = *(const h16x8 *)(a.ln_b + 8 * j8);
-            h16x8 xx;
+        // the new token-shift state: written by row 0's workgroup, the only one that reads the old state, each thread
+        // exactly the chunk it has just read
+        if (commit) {
+            h16x8 ls;
 #pragma unroll
-            for (int e = 0; e < 8; ++e) xx[e] = (h16)(((float)xv[e] - mean) * rstd * (float)wv[e] + (float)bv[e]);
-            *(h16x8 *)(a.state_out + 8 * j8) = xx;
+            for (int e = 0; e < 8; ++e) ls[e] = (h16)(((float)lr[c][e] - lmean) * lrstd * (float)wv[e] + (float)bv[e]);
+            *(h16x8 *)(a.state_out + 8 * j8) = ls;
         }
     }
 }
