@@ -149,10 +149,11 @@ __global__ __launch_bounds__(256) void ln_f32_f16_kernel(int C, const float *__r
 // barriers per workgroup instead of five and ten (and no longer chain in row 0's workgroup, which forms the new
 // token-shift state).  Every value is formed by the same thread with the same
 // operations in the same order as in lnmix_seq_kernel, so the two agree bit for bit.
-template <int NJ, int CH>
+// PRE: the mix / scale vectors too are requested at the top (3 NJ CH more registers per thread: shorter chain, fewer
+// workgroups per CU -- for short calls, where a CU has one or two rows anyway).
+template <int NJ, int CH, bool PRE>
 __global__ __launch_bounds__(256) void lnmix_seq_fast_kernel(SeqMixArgs a) {
     __shared__ float red[4 * 2 * NJ > 12 ? 4 * 2 * NJ : 12];
-    constexpr bool PRE = NJ * CH <= 8;   // the mix / scale vectors too are requested at the top (registers allow it)
     const int t = blockIdx.x, C = a.C, nch = C >> 3;
     const rwkv_half *x = a.x + (size_t)t * C;
     const bool shift = a.sx != nullptr, prev_row = shift && t > 0;
@@ -272,26 +273,28 @@ __global__ __launch_bounds__(256) void lnmix_seq_fast_kernel(SeqMixArgs a) {
 
 }  // namespace
 
-template <int CH>
+template <int CH, bool PRE>
 static bool lnmix_seq_fast_launch(const SeqMixArgs &a, int nj, hipStream_t st) {
     const dim3 grid((unsigned)a.T), block(256);
     switch (nj) {
-        case 1: hipLaunchKernelGGL((lnmix_seq_fast_kernel<1, CH>), grid, block, 0, st, a); break;
-        case 2: hipLaunchKernelGGL((lnmix_seq_fast_kernel<2, CH>), grid, block, 0, st, a); break;
-        case 3: hipLaunchKernelGGL((lnmix_seq_fast_kernel<3, CH>), grid, block, 0, st, a); break;
-        case 4: hipLaunchKernelGGL((lnmix_seq_fast_kernel<4, CH>), grid, block, 0, st, a); break;
-        case 6: hipLaunchKernelGGL((lnmix_seq_fast_kernel<6, CH>), grid, block, 0, st, a); break;
+        case 1: hipLaunchKernelGGL((lnmix_seq_fast_kernel<1, CH, PRE>), grid, block, 0, st, a); break;
+        case 2: hipLaunchKernelGGL((lnmix_seq_fast_kernel<2, CH, PRE>), grid, block, 0, st, a); break;
+        case 3: hipLaunchKernelGGL((lnmix_seq_fast_kernel<3, CH, PRE>), grid, block, 0, st, a); break;
+        case 4: hipLaunchKernelGGL((lnmix_seq_fast_kernel<4, CH, PRE && CH <= 2>), grid, block, 0, st, a); break;
+        case 6: hipLaunchKernelGGL((lnmix_seq_fast_kernel<6, CH, PRE && CH <= 1>), grid, block, 0, st, a); break;
         default: return false;
     }
     return true;
 }
 
 int lnmix_seq_launch(const SeqMixArgs &a, int nj, hipStream_t st) {
-    // rows of up to 8192 channels: the register-resident kernel (1, 2 or 4 chunks of 8 channels per thread)
+    // rows of up to 8192 channels: the register-resident kernel (1, 2 or 4 chunks of 8 channels per thread); calls of
+    // up to 512 rows also hold the mix and scale vectors in registers
     if (a.C <= 8192 && (nj == 1 || nj == 2 || nj == 3 || nj == 4 || nj == 6)) {
-        if (a.C <= 2048) lnmix_seq_fast_launch<1>(a, nj, st);
-        else if (a.C <= 4096) lnmix_seq_fast_launch<2>(a, nj, st);
-        else lnmix_seq_fast_launch<4>(a, nj, st);
+        const bool pre = a.T <= 512;
+        if (a.C <= 2048) pre ? lnmix_seq_fast_launch<1, true>(a, nj, st) : lnmix_seq_fast_launch<1, false>(a, nj, st);
+        else if (a.C <= 4096) pre ? lnmix_seq_fast_launch<2, true>(a, nj, st) : lnmix_seq_fast_launch<2, false>(a, nj, st);
+        else lnmix_seq_fast_launch<4, false>(a, nj, st);
         RWKV_LAUNCH_CHECK();
         return RWKV_OK;
     }
