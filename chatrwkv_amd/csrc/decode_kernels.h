@@ -19,9 +19,11 @@ constexpr int DWAVES = DTHREADS / 64;
 constexpr float LN_EPS = 1e-5f;
 constexpr int VP = 4;  // most 8-element groups per thread the vector prologue keeps in registers (N <= 32768)
 
-// x for this step: the embedding row of the token (first layer) or the running activation.
-DEV const rwkv_half *resolve_x(const rwkv_half *x, const rwkv_half *emb, const int32_t *token, int C) {
-    return token ? emb + (size_t)(*token) * C : x;
+// x for this step: the embedding row of the token (first layer) or the running activation.  The id comes
+// from device memory (it may be the output of a sampling kernel); one outside [0, vocab) is clamped to the
+// nearest valid row, so a bad id can never become an out-of-bounds read.
+DEV const rwkv_half *resolve_x(const rwkv_half *x, const rwkv_half *emb, const int32_t *token, int C, int vocab) {
+    return token ? emb + (size_t)min(max(*token, 0), vocab - 1) * C : x;
 }
 
 // LDS item (16 bytes = 8 halves) index of the 8-element group j8 of an activation vector.
@@ -275,7 +277,7 @@ DEV void stream_rows(int ngroups, int nseg, bool pro_wave, ProLoad pro_load, Pro
 struct AttArgs {
     const rwkv_half *x, *emb;
     const int32_t *token;
-    int C;
+    int C, vocab;
     const rwkv_half *ln_w, *ln_b, *sx;
     rwkv_half *xx_tmp;
     const rwkv_half *mix[3];  // k, v, r
@@ -299,7 +301,7 @@ __global__ __launch_bounds__(DTHREADS) void att_kernel(AttArgs a) {
     VecSums S[3];
     LnMixPro<U8, 3> pro;
     auto pro_load = [&]() {
-        pro.load(resolve_x(a.x, a.emb, a.token, C), C, a.ln_w, a.ln_b, a.sx, a.mix, a.mat);
+        pro.load(resolve_x(a.x, a.emb, a.token, C, a.vocab), C, a.ln_w, a.ln_b, a.sx, a.mix, a.mat);
     };
     auto pro_compute = [&]() { pro.compute(C, a.sx != nullptr, a.mix, xs, S, a.xx_tmp, red); };
     auto rowf = [&](int c, int k, const uint8_t *&row, const h16 *&xv) {
@@ -412,7 +414,7 @@ struct VecArgs {
     MatDev mat;
     const rwkv_half *x_in, *emb;  // residual source (emb row when token != NULL)
     const int32_t *token;
-    int C;
+    int C, vocab;
     const rwkv_half *gate;  // [M] or NULL
     rwkv_half *x_out;       // [M]
     float out_scale;
@@ -486,7 +488,7 @@ __global__ __launch_bounds__(DTHREADS) void vec_kernel(VecArgs a) {
     auto epi_load = [&](int m) {
         VecEpi e{};
         if (U8) { e.rx = a.mat.rx[m]; e.mx = a.mat.mx[m]; }
-        if (a.act == VACT_RESIDUAL) e.xin = resolve_x(a.x_in, a.emb, a.token, a.C)[m];
+        if (a.act == VACT_RESIDUAL) e.xin = resolve_x(a.x_in, a.emb, a.token, a.C, a.vocab)[m];
         if (a.gate) e.gate = a.gate[m];
         return e;
     };

@@ -132,7 +132,7 @@ static int v4_one_impl(const rwkv_v4_model *m, const rwkv_v4_layer_state *states
         const bool u8 = mat_is_u8(m->weights_u8, l.att_key);
         if (only_phase < 0 || only_phase == 0) {
             AttArgs a{};
-            a.x = ws.x; a.emb = m->emb; a.token = tok; a.C = C;
+            a.x = ws.x; a.emb = m->emb; a.token = tok; a.C = C; a.vocab = m->vocab;
             a.ln_w = l.ln1_w; a.ln_b = l.ln1_b; a.sx = s.att_xx; a.xx_tmp = ws.xx_att;
             a.mix[0] = l.att_mix_k; a.mix[1] = l.att_mix_v; a.mix[2] = l.att_mix_r;
             a.mat[0] = to_dev(l.att_key); a.mat[1] = to_dev(l.att_value); a.mat[2] = to_dev(l.att_receptance);
@@ -146,7 +146,7 @@ static int v4_one_impl(const rwkv_v4_model *m, const rwkv_v4_layer_state *states
         if (only_phase < 0 || only_phase == 1) {
             VecArgs a{};
             a.vin = ws.rwkv; a.N = C; a.M = C; a.mat = to_dev(l.att_output);
-            a.x_in = ws.x; a.emb = m->emb; a.token = tok; a.C = C; a.gate = nullptr; a.x_out = ws.x;
+            a.x_in = ws.x; a.emb = m->emb; a.token = tok; a.C = C; a.vocab = m->vocab; a.gate = nullptr; a.x_out = ws.x;
             a.out_scale = 1.f; a.commit_src = ws.xx_att; a.commit_dst = s.att_xx; a.act = VACT_RESIDUAL;
             vec_launch(u8, a, grid, st);
             mark();

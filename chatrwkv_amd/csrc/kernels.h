@@ -59,7 +59,7 @@ struct SeqMixArgs {
 };
 
 int lnmix_seq_launch(const SeqMixArgs &a, int nj, hipStream_t st);
-int gather_emb_launch(int64_t T, int C, const int32_t *tokens, const rwkv_half *emb, rwkv_half *x, hipStream_t st);
+int gather_emb_launch(int64_t T, int C, int vocab, const int32_t *tokens, const rwkv_half *emb, rwkv_half *x, hipStream_t st);
 int copy_h16_launch(int n, const rwkv_half *src, rwkv_half *dst, hipStream_t st);
 int v4_model_check(const rwkv_v4_model *m);
 int v4_head_launch(const rwkv_v4_model *m, const rwkv_half *x, float *logits, hipStream_t st);

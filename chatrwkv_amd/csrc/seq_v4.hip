@@ -10,11 +10,12 @@ namespace {
 
 constexpr float LN_EPS = 1e-5f;
 
-__global__ __launch_bounds__(256) void gather_emb_kernel(int T, int C, const int32_t *__restrict__ tokens,
+// ids outside [0, vocab) are clamped to the nearest valid row: a bad id never becomes an out-of-bounds read
+__global__ __launch_bounds__(256) void gather_emb_kernel(int T, int C, int vocab, const int32_t *__restrict__ tokens,
                                                          const rwkv_half *__restrict__ emb,
                                                          rwkv_half *__restrict__ x) {
     const int t = blockIdx.x;
-    const u32x4 *src = (const u32x4 *)(emb + (size_t)tokens[t] * C);
+    const u32x4 *src = (const u32x4 *)(emb + (size_t)min(max(tokens[t], 0), vocab - 1) * C);
     u32x4 *dst = (u32x4 *)(x + (size_t)t * C);
     for (int i = threadIdx.x; i < (C >> 3); i += blockDim.x) dst[i] = src[i];
 }
@@ -311,8 +312,8 @@ int lnmix_seq_launch(const SeqMixArgs &a, int nj, hipStream_t st) {
     return RWKV_OK;
 }
 
-int gather_emb_launch(int64_t T, int C, const int32_t *tokens, const rwkv_half *emb, rwkv_half *x, hipStream_t st) {
-    hipLaunchKernelGGL(gather_emb_kernel, dim3((unsigned)T), dim3(256), 0, st, (int)T, C, tokens, emb, x);
+int gather_emb_launch(int64_t T, int C, int vocab, const int32_t *tokens, const rwkv_half *emb, rwkv_half *x, hipStream_t st) {
+    hipLaunchKernelGGL(gather_emb_kernel, dim3((unsigned)T), dim3(256), 0, st, (int)T, C, vocab, tokens, emb, x);
     RWKV_LAUNCH_CHECK();
     return RWKV_OK;
 }
@@ -441,7 +442,7 @@ extern "C" int rwkv_v4_forward_seq(const rwkv_v4_model *m, const rwkv_v4_layer_s
     float *s2[3] = {ws.sums + T, ws.sums + 3 * T, ws.sums + 5 * T};
     float *s0v = ws.sums + 6 * T, *s2v = ws.sums + 7 * T;
 
-    hipLaunchKernelGGL(gather_emb_kernel, dim3((unsigned)T), dim3(256), 0, st, (int)T, C, tokens, m->emb, ws.x);
+    hipLaunchKernelGGL(gather_emb_kernel, dim3((unsigned)T), dim3(256), 0, st, (int)T, C, (int)m->vocab, tokens, m->emb, ws.x);
     SideStreams *ss = T >= 256 ? side_streams() : nullptr;
 
     for (int i = 0; i < m->n_layer; ++i) {

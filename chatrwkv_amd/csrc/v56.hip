@@ -252,7 +252,7 @@ extern "C" int rwkv_v56_forward(const rwkv_v56_model *m, const rwkv_v56_layer_st
             cs[j].splitk = nullptr;
         }
 
-    if ((rc = gather_emb_launch(T, C, tokens, m->emb, ws.x, st))) return rc;
+    if ((rc = gather_emb_launch(T, C, m->vocab, tokens, m->emb, ws.x, st))) return rc;
     for (int i = 0; i < m->n_layer; ++i) {
         const rwkv_v56_layer &l = m->layers[i];
         const rwkv_v56_layer_state &s = states[i];

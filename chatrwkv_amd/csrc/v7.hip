@@ -551,7 +551,7 @@ extern "C" int rwkv_v7_forward(const rwkv_v7_model *m, const rwkv_v56_layer_stat
 
     SideStreams *ss = T >= 256 ? side_streams() : nullptr;
 
-    if ((rc = gather_emb_launch(T, C, tokens, m->emb, ws.x, st))) return rc;
+    if ((rc = gather_emb_launch(T, C, m->vocab, tokens, m->emb, ws.x, st))) return rc;
     for (int i = 0; i < m->n_layer; ++i) {
         const rwkv_v7_layer &l = m->layers[i];
         const rwkv_v56_layer_state &s = states[i];

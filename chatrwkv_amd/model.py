@@ -17,7 +17,8 @@ Differences a caller can observe, all deliberate:
     this for aa, bb, pp); ``copy.deepcopy(state)`` snapshots a state as in v2/chat.py:166-179;
   * ``model`` may also be an in-memory ``{name: tensor}`` dict (tensors on CPU or GPU), and
     ``tokens`` of a one-token call may be a 1-element integer tensor on the GPU, which keeps a
-    greedy decode loop free of host synchronisation.
+    greedy decode loop free of host synchronisation; such an id cannot be checked without one, so the
+    kernels clamp it into [0, vocab) (ids given as Python ints raise IndexError when out of range).
 """
 import collections
 import ctypes
@@ -58,7 +59,7 @@ class RWKV:
             if not args.MODEL_NAME.endswith('.pth'):
                 args.MODEL_NAME += '.pth'
             prxxx(f'Loading {args.MODEL_NAME} ...')
-            w = torch.load(args.MODEL_NAME, map_location='cpu')
+            w = torch.load(args.MODEL_NAME, map_location='cpu', weights_only=True, mmap=True)
 
         converted = '_strategy' in w                                  # model.py:646-656
         if converted:

@@ -71,10 +71,15 @@ class _TorchGen:
 
 
 def make_checkpoint(version=4, n_layer=2, n_embd=64, n_ffn=None, vocab=97, seed=0,
-                    head_size=64, lora_maa=32, lora_decay=64, device=None, n_att=None):
+                    head_size=64, lora_maa=32, lora_decay=64, device=None, n_att=None, affine=False,
+                    time_state=False):
     """Return an OrderedDict checkpoint in the reference's raw (pre-conversion) layout.
 
     version: 4, 5 (v5.0), 5.1, 5.2 or 6.
+    affine: LayerNorm / GroupNorm weights U[0.8, 1.2] and biases N(0, 0.05) instead of 1 / 0, so that
+    every affine vector is told apart from every other one (parity tests); the benchmark shapes keep 1 / 0.
+    time_state: RWKV-5/6 only, adds a trained initial state ``att.time_state`` [H, N, N] per block
+    (model.py:1467-1468).
     Key order follows real checkpoints; for v6, ``time_maa_*`` precede
     ``time_faaaa`` inside a block because the reference's head-count
     detection depends on it (model.py:676-679).
@@ -84,6 +89,15 @@ def make_checkpoint(version=4, n_layer=2, n_embd=64, n_ffn=None, vocab=97, seed=
     V = int(vocab)
     A = int(n_att) if n_att is not None else C
     g = _NumpyGen(seed) if device is None else _TorchGen(seed, device)
+
+    def ln(name, n):
+        if affine:
+            w[name + ".weight"] = g.uniform(name + ".weight", (n,), 0.8, 1.2)
+            w[name + ".bias"] = g.normal(name + ".bias", (n,), 0.05)
+        else:
+            w[name + ".weight"] = g.const((n,), 1.0)
+            w[name + ".bias"] = g.const((n,), 0.0)
+
     w = OrderedDict()
     w["emb.weight"] = g.normal("emb.weight", (V, C), 0.02)
     v5 = int(version) == 5
@@ -93,9 +107,8 @@ def make_checkpoint(version=4, n_layer=2, n_embd=64, n_ffn=None, vocab=97, seed=
         H = A // head_size
     for i in range(n_layer):
         b = f"blocks.{i}."
-        for ln in (("ln1", "ln2", "ln0") if i == 0 else ("ln1", "ln2")):
-            w[b + ln + ".weight"] = g.const((C,), 1.0)
-            w[b + ln + ".bias"] = g.const((C,), 0.0)
+        for name in (("ln1", "ln2", "ln0") if i == 0 else ("ln1", "ln2")):
+            ln(b + name, C)
         a = b + "att."
         if version == 4:
             w[a + "time_decay"] = g.uniform(a + "time_decay", (A,), -6.0, -1.0)
@@ -127,8 +140,9 @@ def make_checkpoint(version=4, n_layer=2, n_embd=64, n_ffn=None, vocab=97, seed=
             w[a + "gate.weight"] = g.normal(a + "gate.weight", (A, C), 0.02)
         w[a + "output.weight"] = g.normal(a + "output.weight", (C, A), 0.02)
         if v5 or v6:
-            w[a + "ln_x.weight"] = g.const((A,), 1.0)
-            w[a + "ln_x.bias"] = g.const((A,), 0.0)
+            ln(a + "ln_x", A)
+            if time_state:
+                w[a + "time_state"] = g.normal(a + "time_state", (H, head_size, head_size), 0.3)
         f = b + "ffn."
         mixname = "time_maa_" if v6 else "time_mix_"
         for m in "kr":
@@ -136,8 +150,7 @@ def make_checkpoint(version=4, n_layer=2, n_embd=64, n_ffn=None, vocab=97, seed=
         w[f + "key.weight"] = g.normal(f + "key.weight", (F, C), 0.02)
         w[f + "receptance.weight"] = g.normal(f + "receptance.weight", (C, C), 0.02)
         w[f + "value.weight"] = g.normal(f + "value.weight", (C, F), 0.02)
-    w["ln_out.weight"] = g.const((C,), 1.0)
-    w["ln_out.bias"] = g.const((C,), 0.0)
+    ln("ln_out", C)
     w["head.weight"] = g.normal("head.weight", (V, C), 0.02)
     return w
 

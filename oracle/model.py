@@ -84,7 +84,10 @@ def _np(t):
 
 
 class OracleRWKV:
-    def __init__(self, checkpoint, strategy, rescale_layer=None, cache_dequant=None):
+    def __init__(self, checkpoint, strategy, rescale_layer=None, cache_dequant=None, exact=False):
+        """exact=True: the weights are converted as ``strategy`` says (same uint8 matrices, same stored scale
+        and mix vectors, same rescale), then every step of forward is evaluated in fp64 with no rounding:
+        the value both the reference's fp16 path and any emulation of it approximate."""
         self.strategy = strategy
         n_layer = 1 + max(int(k.split('.')[1]) for k in checkpoint if k.startswith('blocks.'))
         self.device, at, self.slot_u8 = plan_wtypes(strategy, n_layer)
@@ -98,6 +101,9 @@ class OracleRWKV:
         # the CPU baseline path dequantises per call; the emulation may cache
         self.cache = (self.device != 'cpu') if cache_dequant is None else cache_dequant
         self._convert({k: _np(v) for k, v in checkpoint.items()})
+        if exact:
+            self.atype = np.float64
+            self.w = {k: (v if v.dtype == np.uint8 else v.astype(np.float64)) for k, v in self.w.items()}
 
     @classmethod
     def random_converted_v4(cls, n_layer, n_embd, n_ffn, vocab, seed=0):
@@ -243,7 +249,10 @@ class OracleRWKV:
                        np.full(self.n_att, -1e30, f32), np.zeros(C, A)]
             else:
                 N = self.n_att // self.n_head
-                st += [np.zeros(C, A), np.zeros((self.n_head, N, N), f32), np.zeros(C, A)]
+                ts = self.w.get(f'blocks.{i}.att.time_state')            # model.py:765-768, 1467-1468
+                kv = (np.zeros((self.n_head, N, N), f32) if ts is None else
+                      np.ascontiguousarray(ts.reshape(self.n_head, N, N).transpose(0, 2, 1)).astype(f32))
+                st += [np.zeros(C, A), kv, np.zeros(C, A)]
         return st
 
     # ------------------------------------------------------------------ blocks
@@ -294,6 +303,7 @@ class OracleRWKV:
         w, p = self.w, f'blocks.{i}.'
         a = p + 'att.'
         A = self.atype
+        f32 = np.float64 if A == np.float64 else np.float32          # exact evaluation: nothing narrower than fp64
         one = A(1)
         T = x.shape[0]
         H = self.n_head

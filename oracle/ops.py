@@ -23,6 +23,11 @@ f16, f32, f64 = np.float16, np.float32, np.float64
 def layer_norm(x, w, b, eps=1e-5):
     """F.layer_norm over the last axis (model.py:985, 1035, 1668).  Statistics in
     high precision, affine applied before the single rounding to x.dtype."""
+    if x.ndim == 2 and x.shape[0] > 4096:             # a whole embedding table: row blocks that stay in cache
+        out = np.empty_like(x)
+        for r in range(0, x.shape[0], 2048):
+            out[r:r + 2048] = layer_norm(x[r:r + 2048], w, b, eps)
+        return out
     x64 = x.astype(f64)
     mu = x64.mean(axis=-1, keepdims=True)
     var = ((x64 - mu) ** 2).mean(axis=-1, keepdims=True)
@@ -70,16 +75,17 @@ class Mat:
     def quantized(self):
         return self.w.dtype == np.uint8
 
-    def dense_f32(self, cache):
+    def dense_f32(self, cache, dtype=f32):
         """fp32 matrix used by the contraction.  For uint8 weights this is the dequantised
         matrix evaluated in fp32 (model.py:93 order; cuda/operators.cu:130-134 is the same
-        expression with the factors commuted)."""
-        if self._deq is not None:
+        expression with the factors commuted).  dtype=f64: the same stored values (uint8 matrix and
+        its stored scale vectors) expanded without rounding, for the exact evaluation."""
+        if self._deq is not None and self._deq.dtype == dtype:
             return self._deq
         if self.quantized:
-            d = quant.dequant(self.w, self.mx, self.rx, self.my, self.ry, dtype=f32)
+            d = quant.dequant(self.w, self.mx, self.rx, self.my, self.ry, dtype=dtype)
         else:
-            d = self.w.astype(f32)
+            d = self.w.astype(dtype)
         if cache:
             self._deq = d
         return d
@@ -98,6 +104,8 @@ def matmul(a, m, atype, output_dtype=None, cache=False, via_atype=False):
     """
     if output_dtype is None:
         output_dtype = atype
+    if atype == f64:                                  # exact evaluation: no rounding anywhere
+        return a @ m.dense_f32(cache, f64)
     acc = a.astype(f32) @ m.dense_f32(cache)
     if m.quantized or via_atype:
         return acc.astype(atype).astype(output_dtype)
@@ -107,6 +115,8 @@ def matmul(a, m, atype, output_dtype=None, cache=False, via_atype=False):
 def small_matmul(a, b, out_dtype):
     """Plain ``a @ b`` / ``torch.bmm`` on float operands with fp32 accumulation (RWKV-6 LoRA,
     model.py:1268-1269, 1286)."""
+    if out_dtype == f64:
+        return a.astype(f64) @ b.astype(f64)
     return (a.astype(f32) @ b.astype(f32)).astype(out_dtype)
 
 
@@ -121,8 +131,9 @@ def wkv4(k, v, t_first, t_decay, aa, bb, pp):
     Returns y [T, C] fp32 and the new state.
     """
     T, C = k.shape
-    aa, bb, pp = aa.astype(f32), bb.astype(f32), pp.astype(f32)
-    y = np.empty((T, C), dtype=f32)
+    ft = f64 if k.dtype == f64 else f32               # f64 only in the exact evaluation
+    aa, bb, pp = aa.astype(ft), bb.astype(ft), pp.astype(ft)
+    y = np.empty((T, C), dtype=ft)
     for t in range(T):
         kk, vv = k[t], v[t]
         ww = t_first + kk
@@ -152,13 +163,14 @@ def wkv56(r, k, v, w, u, S):
     Returns out [T, H, N] fp32 and the new S.
     """
     T, H, N = r.shape
-    S = S.astype(f32).copy()
-    out = np.empty((T, H, N), dtype=f32)
-    u3 = np.broadcast_to(u.astype(f32).reshape(H, -1), (H, N))[:, :, None]
+    ft = f64 if r.dtype == f64 else f32               # f64 only in the exact evaluation
+    S = S.astype(ft).copy()
+    out = np.empty((T, H, N), dtype=ft)
+    u3 = np.broadcast_to(u.astype(ft).reshape(H, -1), (H, N))[:, :, None]
     for t in range(T):
         wt = w[t] if w.ndim == 3 else w
-        w3 = np.broadcast_to(wt.astype(f32).reshape(H, -1), (H, N))[:, :, None]
+        w3 = np.broadcast_to(wt.astype(ft).reshape(H, -1), (H, N))[:, :, None]
         a = k[t][:, :, None] * v[t][:, None, :]
-        out[t] = np.einsum('hj,hji->hi', r[t], u3 * a + S, dtype=f32)
+        out[t] = np.einsum('hj,hji->hi', r[t], u3 * a + S, dtype=ft)
         S = a + w3 * S
     return out, S

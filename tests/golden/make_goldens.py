@@ -20,6 +20,8 @@ RWKV_CUDA_ON=0 (no native build), feeds it synthetic checkpoints from
                             the rescale (x / 2 after layer 6, matrices of layers >= 6 halved) to act
   e2e_<ver>_mixed_cpu.npz   RWKV-4 / RWKV-6 under 'cpu fp32i8 *2 -> cpu fp32': uint8 weights for two layers, float
                             weights for the third and the head
+  e2e_<ver>_state_<strategy>.npz  RWKV-5.2 / RWKV-6 checkpoints that carry a trained initial state
+                            (att.time_state, model.py:765-768, 1467-1468) under 'cpu fp32' and 'cpu fp16'
   planner.json              the per-slot plan the reference prints for a list of strategy strings
   e2e_v4_169m_cpu_fp32i8.npz  the 169M-shape model: 128-token prefill + 32 greedy steps;
                             argmax per position, 256 fixed logits per position, state sums
@@ -40,8 +42,10 @@ REF_SRC = "/root/reference/rwkv_pip_package/src"
 
 from chatrwkv_amd import synth  # noqa: E402
 
-TINY = dict(n_layer=3, n_embd=128, n_ffn=512, vocab=211)
-TINY8 = dict(n_layer=8, n_embd=64, n_ffn=256, vocab=100)
+# affine=True: random LayerNorm / GroupNorm weights and biases, so a swapped, dropped or mis-indexed affine
+# vector shows in every fixture below
+TINY = dict(n_layer=3, n_embd=128, n_ffn=512, vocab=211, affine=True)
+TINY8 = dict(n_layer=8, n_embd=64, n_ffn=256, vocab=100, affine=True)
 PROMPT_SEED = 11
 
 
@@ -175,6 +179,31 @@ def e2e_tiny(tmp, which_strats=None):
             print("wrote", name, "version", m.version)
 
 
+def e2e_time_state(tmp):
+    """Checkpoints with att.time_state: forward(tokens, None) starts from it (transposed) instead of zeros."""
+    RWKV = _ref()
+    for ver, tag in ((5.2, "v5_2"), (6, "v6_0")):
+        ck = synth.make_checkpoint(version=ver, seed=500 + int(ver * 10), time_state=True, **TINY)
+        p = os.path.join(tmp, f"ts_{tag}.pth")
+        _save_ckpt(ck, p)
+        toks = synth.random_tokens(9, TINY["vocab"], seed=PROMPT_SEED)
+        for strat in ("cpu fp32", "cpu fp16"):
+            m = RWKV(p, strat, verbose=False)
+            assert m.args.time_state
+            full, st_full = m.forward(toks, None, full_output=True)
+            outs, st = [], None
+            for a, b in ((0, 1), (1, 4), (4, 5), (5, 9)):
+                o, st = m.forward(toks[a:b], st)
+                outs.append(o.detach().float().cpu().numpy())
+            d = {"tokens": np.array(toks), "full_logits": full.detach().float().cpu().numpy(),
+                 "chunk_logits": np.stack(outs)}
+            d.update({"full_" + k: v for k, v in _state_np(st_full).items()})
+            d.update({"chunk_" + k: v for k, v in _state_np(st).items()})
+            name = f"e2e_{tag}_state_{strat.replace(' ', '_')}.npz"
+            np.savez_compressed(os.path.join(HERE, name), **d)
+            print("wrote", name)
+
+
 def e2e_169m(tmp):
     RWKV = _ref()
     ck = synth.make_named("v4-169m", seed=0)
@@ -251,7 +280,7 @@ def planner(tmp):
 if __name__ == "__main__":
     torch.manual_seed(0)
     with tempfile.TemporaryDirectory() as tmp:
-        which = sys.argv[1:] or ["quant_cpu", "quant_cuda", "tiny", "fp16", "mixed", "169m", "planner"]
+        which = sys.argv[1:] or ["quant_cpu", "quant_cuda", "tiny", "fp16", "mixed", "state", "169m", "planner"]
         if "planner" in which:
             planner(tmp)
         if "fp16" in which and "tiny" not in which:
@@ -266,5 +295,7 @@ if __name__ == "__main__":
             quant_cuda_convert(tmp)
         if "tiny" in which:
             e2e_tiny(tmp)
+        if "state" in which:
+            e2e_time_state(tmp)
         if "169m" in which:
             e2e_169m(tmp)

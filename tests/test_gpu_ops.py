@@ -97,7 +97,7 @@ def test_mm8_one(N, M):
 
 
 @pytest.mark.parametrize("N,M,B", [(768, 768, 2), (768, 3072, 5), (3072, 768, 128), (768, 50277, 3),
-                                   (2560, 2560, 200), (4096, 4096, 1024), (4096, 16384, 256), (16384, 4096, 130),
+                                   (2560, 2560, 200), (4096, 4096, 1024), (4096, 16384, 256), (16384, 4096, 130), (4096, 16384, 1024),
                                    # long calls: 256 x 256 tiles loaded straight into LDS; whole, ragged and split-K
                                    (4096, 8192, 1000), (16384, 4096, 520), (2560, 10240, 768),
                                    # ragged tiles of the direct-to-LDS kernel: widths and row counts that end inside a tile

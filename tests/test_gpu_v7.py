@@ -254,6 +254,11 @@ def test_v7_api_errors(tiny7):
         m.forward([TINY7["vocab"]], None)
     with pytest.raises(IndexError):
         m.forward([1, -1], None)
+    # an id that is already on the device cannot be range-checked without a synchronisation: clamped in the gather
+    V = TINY7["vocab"]
+    bad, _ = m.forward(torch.tensor([V + 5], device="cuda"), None)
+    ok, _ = m.forward([V - 1], None)
+    assert torch.equal(bad, ok)
     with pytest.raises(ValueError):
         m.forward([1], [torch.zeros(1)])
     with pytest.raises(NotImplementedError):

@@ -168,3 +168,34 @@ def test_mixed_weight_types_match_reference(ver, tag):
     np.testing.assert_allclose(np.stack(outs), ref["chunk_logits"], rtol=2e-4, atol=2e-5)
     for i, s in enumerate(st):
         np.testing.assert_allclose(s, ref[f"chunk_state_{i}"], rtol=2e-4, atol=2e-5, err_msg=str(i))
+
+
+@pytest.mark.parametrize("ver,tag", [(5.2, "v5_2"), (6, "v6_0")])
+def test_time_state_matches_reference(ver, tag):
+    """Checkpoints with a trained initial state (att.time_state): forward(tokens, None) starts from its
+    transpose (model.py:1467-1468); against the reference's 'cpu fp32' run exactly and its 'cpu fp16' run
+    within the half-precision bound.  Dropping the transpose, or starting from zeros, fails this."""
+    ck = synth.make_checkpoint(version=ver, seed=500 + int(ver * 10), time_state=True, **TINY)
+    ref = _load(f"e2e_{tag}_state_cpu_fp32.npz")
+    o = OracleRWKV(ck, "cpu fp32")
+    toks = [int(t) for t in ref["tokens"]]
+    full, st_full = o.forward(toks, None, full_output=True)
+    np.testing.assert_allclose(full, ref["full_logits"], rtol=2e-4, atol=2e-5)
+    st, outs = None, []
+    for a, b in ((0, 1), (1, 4), (4, 5), (5, 9)):
+        out, st = o.forward(toks[a:b], st)
+        outs.append(out)
+    np.testing.assert_allclose(np.stack(outs), ref["chunk_logits"], rtol=2e-4, atol=2e-5)
+    for prefix, state in (("full_", st_full), ("chunk_", st)):
+        for i, s in enumerate(state):
+            np.testing.assert_allclose(s, ref[f"{prefix}state_{i}"], rtol=2e-4, atol=2e-5, err_msg=f"{prefix}{i}")
+    # the initial state matters: the same tokens from a zero state give visibly different logits
+    zero = OracleRWKV(ck, "cpu fp32")
+    zero.w = {k: v for k, v in zero.w.items() if "time_state" not in k}
+    zfull, _ = zero.forward(toks, None, full_output=True)
+    assert np.abs(zfull - ref["full_logits"]).max() > 1e-2
+    ref16 = _load(f"e2e_{tag}_state_cpu_fp16.npz")
+    for strat in ("cpu fp16", "cuda fp16"):
+        o16 = OracleRWKV(ck, strat)
+        f16full, _ = o16.forward(toks, None, full_output=True)
+        assert np.abs(f16full - ref16["full_logits"]).max() <= 1.5e-3 * max(float(np.abs(ref16["full_logits"]).max()), 1.0)
