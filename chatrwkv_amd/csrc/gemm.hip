@@ -20,6 +20,7 @@
 #include <algorithm>
 #include "kernels.h"
 #include <cstdlib>
+#include <mutex>
 
 namespace {
 
@@ -875,13 +876,13 @@ int launch_pick(int cfg, int64_t T, int64_t N, int64_t M, const rwkv_half *A, in
 //    9       uint8 weights otherwise, where 256 x 256 tiles of the register-staged kernel fill the chip: one per CU
 //            and round, the last round at least 70 % full
 //    3       everything else: 128 x 128 tiles, 4 k-tiles of prefetch
-int pick_cfg(int64_t T, int64_t N, int64_t M, bool w_u8, bool alone, bool dma, bool can_split) {
+int pick_cfg(int64_t T, int64_t N, int64_t M, bool w_u8, bool alone, bool dma, size_t split_bytes) {
     const char *e = getenv("RWKV_GEMM_CFG");  // tuning override
     if (e && *e) return atoi(e);
     if (!alone) return dma ? 15 : 3;   // a 256 x 256 tile's LDS leaves no room beside it on the CU, two small ones fit
     if (dma) {
         const int nk = (int)(N / BK);
-        const size_t out_bytes = (size_t)T * M * sizeof(float), ws = can_split && !(M & 3) ? RWKV_SPLITK_WS_BYTES : 0;
+        const size_t out_bytes = (size_t)T * M * sizeof(float), ws = !(M & 3) ? split_bytes : 0;
         double c14, c15;
         dma_split(((T + 255) / 256) * ((M + 255) / 256), nk, false, out_bytes, ws, &c14);
         dma_split(((T + 127) / 128) * ((M + 127) / 128), nk, true, out_bytes, ws, &c15);
@@ -895,7 +896,8 @@ int pick_cfg(int64_t T, int64_t N, int64_t M, bool w_u8, bool alone, bool dma, b
 
 int gemm_launch(bool w_u8, int64_t T, int64_t N, int64_t M, const rwkv_half *A, int64_t lda, const void *W,
                 int64_t ldw, void *Y, int64_t ldy, const GemmEpi &ep, hipStream_t st) {
-    const int cfg = pick_cfg(T, N, M, w_u8, !ep.small_tiles, dma_ok(w_u8, N, M, A, lda, W, ldw, Y, ldy, ep), ep.splitk_ws != nullptr);
+    const int cfg = pick_cfg(T, N, M, w_u8, !ep.small_tiles, dma_ok(w_u8, N, M, A, lda, W, ldw, Y, ldy, ep),
+                             ep.splitk_ws ? ep.splitk_bytes : 0);
     return w_u8 ? launch_pick<true>(cfg, T, N, M, A, lda, W, ldw, Y, ldy, ep, st)
                 : launch_pick<false>(cfg, T, N, M, A, lda, W, ldw, Y, ldy, ep, st);
 }
@@ -1005,6 +1007,69 @@ extern "C" int rwkv_mm8_seq_f16(int64_t B, int64_t N, int64_t M, const rwkv_half
     ep.mx = mx; ep.rx = rx; ep.s0 = s0; ep.s2 = s2; ep.act = ACT_NONE; ep.out_scale = 1.f; ep.out_dtype = RWKV_DT_F16;
     ep.splitk_ws = (float *)((unsigned char *)workspace + xs_bytes + (((size_t)B * 8 + 255) & ~(size_t)255));
     ep.splitk_bytes = RWKV_SPLITK_WS_BYTES;
+    return gemm_launch(true, B, N, M, xs, N, w, w_stride_m, y, y_stride, ep, st);
+}
+
+// ---- rwkv_mm8_seq_f16 without a caller workspace ------------------------------------------------------------
+// The scratch of the product (the ry-scaled copy of x, its two row sums, split-K slabs) in a file-scope device
+// array instead of a workspace argument.  The array's name is only a host-side handle: the device address of each
+// GPU's copy comes from hipGetSymbolAddress, once per device, and that pointer is what the kernels get.
+constexpr size_t STATIC_XS_BYTES = (size_t)8 << 20;       // B * N <= 4 Mi elements
+constexpr size_t STATIC_SUMS_BYTES = (size_t)64 << 10;    // B <= 8192
+constexpr size_t STATIC_SPLITK_BYTES = (size_t)16 << 20;  // the K split is limited to slabs that fit here
+constexpr size_t STATIC_SCRATCH_BYTES = STATIC_XS_BYTES + STATIC_SUMS_BYTES + STATIC_SPLITK_BYTES;
+static __device__ __align__(256) unsigned char scratch[STATIC_SCRATCH_BYTES];
+
+constexpr int STATIC_MAX_DEVICES = 64;
+static void *g_scratch_ptr[STATIC_MAX_DEVICES];
+static std::mutex g_scratch_mutex;
+
+// device address of the current device's copy of `scratch` (looked up on the first call on that device)
+static int static_scratch(unsigned char **out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= STATIC_MAX_DEVICES) return RWKV_E_SHAPE;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void *p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return (int)e;
+        if (!p) return RWKV_E_NULL;
+        g_scratch_ptr[dev] = p;
+    }
+    *out = (unsigned char *)g_scratch_ptr[dev];
+    return RWKV_OK;
+}
+
+extern "C" size_t rwkv_mm8_seq_static_max_elems(void) { return STATIC_XS_BYTES / 2; }
+extern "C" size_t rwkv_mm8_seq_static_max_rows(void) { return STATIC_SUMS_BYTES / 8; }
+
+extern "C" int rwkv_mm8_seq_f16_static(int64_t B, int64_t N, int64_t M, const rwkv_half *x, int64_t x_stride,
+                                       const uint8_t *w, int64_t w_stride_n, int64_t w_stride_m, const rwkv_half *mx,
+                                       const rwkv_half *rx, const rwkv_half *my, const rwkv_half *ry, rwkv_half *y,
+                                       int64_t y_stride, void *stream) {
+    if (!x || !w || !mx || !rx || !my || !ry || !y) return RWKV_E_NULL;
+    if (B <= 0 || N <= 0 || M <= 0 || (N % BK) != 0 || B > (1 << 24) || M > (1 << 24)) return RWKV_E_SHAPE;
+    if (w_stride_n != 1 || w_stride_m < N || (w_stride_m & 15) || !aligned16(w)) return RWKV_E_LAYOUT;
+    if (x_stride < N || (x_stride & 7) || !aligned16(x) || y_stride < M || !aligned16(my) || !aligned16(ry))
+        return RWKV_E_LAYOUT;
+    if ((size_t)B * (size_t)N * 2 > STATIC_XS_BYTES || (size_t)B * 8 > STATIC_SUMS_BYTES) return RWKV_E_SCRATCH;
+    unsigned char *base = nullptr;
+    int rc = static_scratch(&base);
+    if (rc) return rc;
+    hipStream_t st = (hipStream_t)stream;
+    rwkv_half *xs = (rwkv_half *)base;
+    float *s0 = (float *)(base + STATIC_XS_BYTES);
+    float *s2 = s0 + B;
+    // every row of xs / s0 / s2 and every slab element the product reads is written by this call first:
+    // nothing in the array has to start at zero
+    rc = mm8_prepare_launch(B, N, x, x_stride, ry, my, xs, s0, s2, st);
+    if (rc) return rc;
+    GemmEpi ep{};
+    ep.mx = mx; ep.rx = rx; ep.s0 = s0; ep.s2 = s2; ep.act = ACT_NONE; ep.out_scale = 1.f; ep.out_dtype = RWKV_DT_F16;
+    ep.splitk_ws = (float *)(base + STATIC_XS_BYTES + STATIC_SUMS_BYTES);
+    ep.splitk_bytes = STATIC_SPLITK_BYTES;
     return gemm_launch(true, B, N, M, xs, N, w, w_stride_m, y, y_stride, ep, st);
 }
 

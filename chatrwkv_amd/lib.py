@@ -18,6 +18,7 @@ _ERR = {
     -3: "RWKV_E_NULL: required pointer is NULL",
     -4: "RWKV_E_WORKSPACE: workspace too small or misaligned",
     -5: "RWKV_E_DTYPE: unknown dtype / mode code",
+    -6: "RWKV_E_SCRATCH: size beyond what the library's built-in scratch holds",
 }
 
 _i64, _int, _vp, _sz = ctypes.c_int64, ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t
@@ -31,6 +32,9 @@ SIGNATURES = {
     "rwkv_mm8_one_f16": (_int, [_i64, _i64, _vp, _vp, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _int, _vp]),
     "rwkv_mm8_seq_workspace": (_sz, [_i64, _i64]),
     "rwkv_mm8_seq_f16": (_int, [_i64, _i64, _i64, _vp, _i64, _vp, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _i64, _vp, _sz, _vp]),
+    "rwkv_mm8_seq_static_max_elems": (_sz, []),
+    "rwkv_mm8_seq_static_max_rows": (_sz, []),
+    "rwkv_mm8_seq_f16_static": (_int, [_i64, _i64, _i64, _vp, _i64, _vp, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _i64, _vp]),
     "rwkv_gemm_f16": (_int, [_i64, _i64, _i64, _vp, _i64, _vp, _i64, _i64, _vp, _i64, _int, _vp]),
     "rwkv_wkv4_forward": (_int, [_i64, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _int, _vp, _vp, _vp, _vp]),
     "rwkv_wkv5_forward": (_int, [_i64, _i64, _i64, _i64, _vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),

@@ -39,6 +39,7 @@ typedef uint16_t rwkv_half;
 #define RWKV_E_NULL (-3)      /* required pointer is NULL */
 #define RWKV_E_WORKSPACE (-4) /* workspace too small */
 #define RWKV_E_DTYPE (-5)     /* unknown dtype / mode code */
+#define RWKV_E_SCRATCH (-6)   /* size beyond what the library's built-in scratch holds */
 
 #define RWKV_DT_F16 0
 #define RWKV_DT_F32 1
@@ -88,6 +89,22 @@ int rwkv_mm8_seq_f16(int64_t B, int64_t N, int64_t M, const rwkv_half *x, int64_
                      const uint8_t *w, int64_t w_stride_n, int64_t w_stride_m,
                      const rwkv_half *mx, const rwkv_half *rx, const rwkv_half *my, const rwkv_half *ry,
                      rwkv_half *y, int64_t y_stride, void *workspace, size_t workspace_bytes, void *stream);
+
+/* rwkv_mm8_seq_f16 for callers that cannot allocate (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc): no workspace argument, and no hipMalloc / hipFree or other allocating call
+ * inside.  It has no counterpart in the reference.  The scratch of the product lives in a device array built
+ * into the library (24 MiB + 64 KiB per GPU, held until the process ends), which bounds the size:
+ *   B * N <= rwkv_mm8_seq_static_max_elems() (4 Mi) and B <= rwkv_mm8_seq_static_max_rows() (8192),
+ * otherwise RWKV_E_SCRATCH and nothing is enqueued.  Same kernels and arguments as rwkv_mm8_seq_f16; the K split
+ * is chosen within 16 MiB of slabs instead of 64, so a result can differ from rwkv_mm8_seq_f16's in the order of
+ * its fp32 sums (at most one fp16 rounding step).  All calls on one GPU share that GPU's array: calls that may
+ * overlap there (different streams, different host threads) race; calls on one stream are safe. */
+size_t rwkv_mm8_seq_static_max_elems(void);
+size_t rwkv_mm8_seq_static_max_rows(void);
+int rwkv_mm8_seq_f16_static(int64_t B, int64_t N, int64_t M, const rwkv_half *x, int64_t x_stride,
+                            const uint8_t *w, int64_t w_stride_n, int64_t w_stride_m,
+                            const rwkv_half *mx, const rwkv_half *rx, const rwkv_half *my, const rwkv_half *ry,
+                            rwkv_half *y, int64_t y_stride, void *stream);
 
 /* gemm_fp16: c[B, M] = a[B, N] @ b[N, M], fp16 operands, fp32 accumulation, c written
  * directly as fp16 or fp32 (c_dtype) with no intermediate fp16 rounding.  Replaces
