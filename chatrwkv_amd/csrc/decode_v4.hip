@@ -18,6 +18,7 @@
 // workgroup, so its new value goes to a scratch vector and is committed to the state by
 // workgroup 0 of the *next* launch.
 #include "decode_kernels.h"
+#include "../../include/rwkv_hip_bench.h"
 
 namespace {
 

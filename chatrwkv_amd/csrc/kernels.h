@@ -69,13 +69,36 @@ int num_cu();
 // the presence of the scale vectors -- a strategy such as 'cuda fp16i8 *20 -> cuda fp16'.
 inline bool mat_is_u8(int weights_u8, const rwkv_mat &m) { return weights_u8 == 2 ? m.mx != nullptr : weights_u8 != 0; }
 
-// Two extra streams (default priority, created once per process) for contractions that are independent and each
-// too small to fill the chip; fork / join by events around them (seq_v4.hip).
+// Two extra streams (default priority) for contractions that are independent and each too small to fill the chip;
+// fork / join by events around them (seq_v4.hip).  Every (device, caller stream) pair gets its own set, created on
+// its first use and kept until the process ends, so calls on different streams never share an event; calls on
+// ONE stream must come from one host thread at a time, as for any stream-ordered API.
 struct SideStreams {
     hipStream_t s[2];
     hipEvent_t fork, join[2];
     bool ok;
 };
-SideStreams *side_streams();                                   // NULL when the streams could not be created
+SideStreams *side_streams(hipStream_t caller);                 // NULL: none available (creation failed, table full)
 bool fork_streams(SideStreams *ss, hipStream_t st, int n);     // side stream j < n then sees everything queued on st so far
 bool join_streams(SideStreams *ss, hipStream_t st, int n);     // st then sees everything queued on the side streams
+
+// A fork that is always joined: by join(), or by the destructor on an early (error) return, so that work queued on
+// a side stream never outlives the call that queued it.
+struct ForkScope {
+    SideStreams *ss;
+    hipStream_t st;
+    int n;
+    bool active;
+    ForkScope(SideStreams *ss_, hipStream_t st_, int n_, bool want) : ss(ss_), st(st_), n(n_), active(false) {
+        if (want && ss) active = fork_streams(ss, st, n);
+    }
+    ForkScope(const ForkScope &) = delete;
+    ForkScope &operator=(const ForkScope &) = delete;
+    explicit operator bool() const { return active; }
+    bool join() {
+        if (!active) return true;
+        active = false;
+        return join_streams(ss, st, n);
+    }
+    ~ForkScope() { if (active) (void)join_streams(ss, st, n); }
+};

@@ -4,6 +4,7 @@
 //   lnmix_seq (LN2, ...) -> GEMM Wr (sigmoid), GEMM Wk (relu^2) -> prepare -> GEMM Wv (gate, residual, /2)
 // and LN_out + head on the last row (GEMV) or on every row (GEMM) for full_output.
 #include <cstdlib>
+#include <mutex>
 #include "kernels.h"
 
 namespace {
@@ -375,17 +376,27 @@ int run_gemm(const rwkv_mat &m, bool u8, int64_t T, const rwkv_half *A, const fl
 // to fill the chip alone: k / v / r of the time mix and r / k of the channel mix run side by side.
 }  // namespace
 
-SideStreams *side_streams() {
-    static SideStreams ss{};
-    static bool tried = false;
-    if (!tried) {
-        tried = true;
-        ss.ok = hipStreamCreateWithFlags(&ss.s[0], hipStreamNonBlocking) == hipSuccess &&
-                hipStreamCreateWithFlags(&ss.s[1], hipStreamNonBlocking) == hipSuccess &&
-                hipEventCreateWithFlags(&ss.fork, hipEventDisableTiming) == hipSuccess &&
-                hipEventCreateWithFlags(&ss.join[0], hipEventDisableTiming) == hipSuccess &&
-                hipEventCreateWithFlags(&ss.join[1], hipEventDisableTiming) == hipSuccess;
-    }
+SideStreams *side_streams(hipStream_t caller) {
+    struct Slot { int dev; hipStream_t caller; SideStreams ss; };
+    constexpr int MAX_SLOTS = 32;
+    static Slot slots[MAX_SLOTS];
+    static int n_slots = 0;
+    static std::mutex mu;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return nullptr;
+    std::lock_guard<std::mutex> lock(mu);
+    for (int i = 0; i < n_slots; ++i)
+        if (slots[i].dev == dev && slots[i].caller == caller) return slots[i].ss.ok ? &slots[i].ss : nullptr;
+    if (n_slots == MAX_SLOTS) return nullptr;      // more caller streams than slots: those run without side streams
+    Slot &sl = slots[n_slots++];
+    sl.dev = dev;
+    sl.caller = caller;
+    SideStreams &ss = sl.ss;
+    ss.ok = hipStreamCreateWithFlags(&ss.s[0], hipStreamNonBlocking) == hipSuccess &&
+            hipStreamCreateWithFlags(&ss.s[1], hipStreamNonBlocking) == hipSuccess &&
+            hipEventCreateWithFlags(&ss.fork, hipEventDisableTiming) == hipSuccess &&
+            hipEventCreateWithFlags(&ss.join[0], hipEventDisableTiming) == hipSuccess &&
+            hipEventCreateWithFlags(&ss.join[1], hipEventDisableTiming) == hipSuccess;
     return ss.ok ? &ss : nullptr;
 }
 
@@ -443,7 +454,7 @@ extern "C" int rwkv_v4_forward_seq(const rwkv_v4_model *m, const rwkv_v4_layer_s
     float *s0v = ws.sums + 6 * T, *s2v = ws.sums + 7 * T;
 
     hipLaunchKernelGGL(gather_emb_kernel, dim3((unsigned)T), dim3(256), 0, st, (int)T, C, (int)m->vocab, tokens, m->emb, ws.x);
-    SideStreams *ss = T >= 256 ? side_streams() : nullptr;
+    SideStreams *ss = T >= 256 ? side_streams(st) : nullptr;
 
     for (int i = 0; i < m->n_layer; ++i) {
         const rwkv_v4_layer &l = m->layers[i];
@@ -471,7 +482,7 @@ extern "C" int rwkv_v4_forward_seq(const rwkv_v4_model *m, const rwkv_v4_layer_s
         // CU, so products side by side on several streams gain nothing); k, v, r as one group
         const bool dma_seq = T >= 512;
         const bool group_kvr = true;       // k, v, r as one grouped launch at every length (tile size and K split by cost)
-        const bool par = ss && !group_kvr && (T / 128) * (C / 128) > 128 && fork_streams(ss, st, 2);
+        ForkScope par(ss, st, 2, !group_kvr && (T / 128) * (C / 128) > 128);
         if (group_kvr) {
             const rwkv_half *xin[3] = {ws.xs[0], ws.xs[1], ws.xs[2]};
             const rwkv_mat *mats[3] = {&l.att_key, &l.att_value, &l.att_receptance};
@@ -487,7 +498,7 @@ extern "C" int rwkv_v4_forward_seq(const rwkv_v4_model *m, const rwkv_v4_layer_s
         if ((rc = run_gemm(l.att_value, u8, T, ws.xs[1], s0[1], s2[1], ws.v, C, e, sv, sk))) return rc;
         e.act = ACT_SIGMOID; e.out_dtype = RWKV_DT_F16; e.raw_f32 = 0;
         if ((rc = run_gemm(l.att_receptance, u8, T, ws.xs[2], s0[2], s2[2], ws.r, C, e, sr, sk))) return rc;
-        if (par && !join_streams(ss, st, 2)) return (int)hipErrorUnknown;
+        if (!par.join()) return (int)hipErrorUnknown;
         }
         if ((rc = wkv4_fused_launch((int)T, C, l.time_decay, l.time_first, ws.k, ws.v, u8 ? 0 : 1, ws.r, ws.rwkv, s.aa,
                                     s.bb, s.pp, st, ws.wkv)))
@@ -516,7 +527,7 @@ extern "C" int rwkv_v4_forward_seq(const rwkv_v4_model *m, const rwkv_v4_layer_s
         e = GemmEpi{};
         e.out_scale = 1.f; e.out_dtype = RWKV_DT_F16;
         e.act = ACT_SIGMOID;
-        const bool par2 = ss && !dma_seq && (T / 128) * (C / 128) > 128 && fork_streams(ss, st, 1);
+        ForkScope par2(ss, st, 1, !dma_seq && (T / 128) * (C / 128) > 128);
         float *sk2 = par2 ? nullptr : ws.splitk;
         if (T <= 128 && !(C & 127) && !(F & 127)) {
             // short calls: receptance and key in one grouped launch
@@ -532,7 +543,7 @@ extern "C" int rwkv_v4_forward_seq(const rwkv_v4_model *m, const rwkv_v4_layer_s
         e.small_tiles = par2 ? 1 : 0;   // the receptance product runs beside this one
         if ((rc = run_gemm(l.ffn_key, u8, T, ws.xs[1], s0[1], s2[1], ws.vx, F, e, st, sk2))) return rc;
         e.small_tiles = 0;
-        if (par2 && !join_streams(ss, st, 1)) return (int)hipErrorUnknown;
+        if (!par2.join()) return (int)hipErrorUnknown;
         }
         const rwkv_half *a_v = ws.vx;
         if (u8) {

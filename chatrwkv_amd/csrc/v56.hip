@@ -244,7 +244,7 @@ extern "C" int rwkv_v56_forward(const rwkv_v56_model *m, const rwkv_v56_layer_st
     // Sequence calls whose square products have more than 128 output tiles (none of them would split K) run
     // independent products side by side on two extra streams, each with its own activation scratch.  Shorter
     // calls are faster one product after the other with split-K (measured at 256 tokens, n_embd 4096).
-    SideStreams *ss = (T / 128) * (C / 128) > 128 ? side_streams() : nullptr;
+    SideStreams *ss = (T / 128) * (C / 128) > 128 ? side_streams(st) : nullptr;
     Ctx cs[2] = {c, c};
     if (ss)
         for (int j = 0; j < 2; ++j) {
@@ -349,14 +349,14 @@ extern "C" int rwkv_v56_forward(const rwkv_v56_model *m, const rwkv_v56_layer_st
                     return rc;
             } else {
             // receptance (then gate) on the caller's stream, key and value on the side streams
-            const bool par = ss && !dma_seq && fork_streams(ss, st, 2);
+            ForkScope par(ss, st, 2, !dma_seq);
             Ctx cr = c;
             if (par) cr.splitk = nullptr;
             if ((rc = mm(cr, l.att_receptance, u8, rx, ACT_NONE, nullptr, nullptr, 1.f, ws.r))) return rc;
             if ((rc = mm(par ? cs[0] : c, l.att_key, u8, kx, ACT_NONE, nullptr, nullptr, 1.f, ws.k))) return rc;
             if ((rc = mm(par ? cs[1] : c, l.att_value, u8, vx, ACT_NONE, nullptr, nullptr, 1.f, ws.v))) return rc;
             if (gated && (rc = mm(c, l.att_gate, u8, gx, ACT_SILU, nullptr, nullptr, 1.f, ws.g))) return rc;
-            if (par && !join_streams(ss, st, 2)) return (int)hipErrorUnknown;
+            if (!par.join()) return (int)hipErrorUnknown;
             }
         }
         // one token of v6: the second decay LoRA product is done inside the WKV kernel
@@ -408,14 +408,14 @@ extern "C" int rwkv_v56_forward(const rwkv_v56_model *m, const rwkv_v56_layer_st
             if ((rc = gemm_group_launch(u8, 2, T, C, xin, mats, outs, ep, nullptr, fs, ws.splitk, st))) return rc;
         } else {
             // channel-mix receptance beside the key product
-            const bool par = ss && !dma_seq && fork_streams(ss, st, 1);
+            ForkScope par(ss, st, 1, !dma_seq);
             if ((rc = mm_scaled(par ? cs[0] : c, l.ffn_receptance, u8, fx[0], fs[0], fs[0] + T, ACT_SIGMOID, nullptr, nullptr,
                                 1.f, ws.r)))
                 return rc;
             Ctx ck = c;
             ck.small_tiles = par ? 1 : 0;
             if ((rc = mm_scaled(ck, l.ffn_key, u8, fx[1], fs[1], fs[1] + T, ACT_RELU_SQ, nullptr, nullptr, 1.f, ws.vx))) return rc;
-            if (par && !join_streams(ss, st, 1)) return (int)hipErrorUnknown;
+            if (!par.join()) return (int)hipErrorUnknown;
         }
         if ((rc = mm(c, l.ffn_value, u8, ws.vx, ACT_GATED_RESIDUAL, ws.x, ws.r, scale, ws.x))) return rc;
         RWKV_LAUNCH_CHECK();

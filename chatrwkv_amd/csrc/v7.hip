@@ -549,7 +549,7 @@ extern "C" int rwkv_v7_forward(const rwkv_v7_model *m, const rwkv_v56_layer_stat
         return q;
     };
 
-    SideStreams *ss = T >= 256 ? side_streams() : nullptr;
+    SideStreams *ss = T >= 256 ? side_streams(st) : nullptr;
 
     if ((rc = gather_emb_launch(T, C, m->vocab, tokens, m->emb, ws.x, st))) return rc;
     for (int i = 0; i < m->n_layer; ++i) {
@@ -605,7 +605,7 @@ extern "C" int rwkv_v7_forward(const rwkv_v7_model *m, const rwkv_v56_layer_stat
         // of the chip without splitting K, the eight small LoRA products (which do split K: one user of the split-K
         // scratch at a time) run beside it on a side stream, on the CUs the group leaves free.
         const bool dma_seq = true;
-        const bool par = ss && dma_seq && 3 * ((T + 255) / 256) * ((C + 255) / 256) >= 192 && fork_streams(ss, st, 1);
+        ForkScope par(ss, st, 1, dma_seq && 3 * ((T + 255) / 256) * ((C + 255) / 256) >= 192);
         Ctx cm = c, cv = c, cl = c;
         if (par) cl.st = ss->s[0];
         if (dma_seq && !(C & 7)) {
@@ -631,7 +631,7 @@ extern "C" int rwkv_v7_forward(const rwkv_v7_model *m, const rwkv_v56_layer_stat
         }
         if ((rc = mm(cl, lora_first(l, o_g, m->lora_g), false, xg, ACT_SIGMOID, nullptr, nullptr, 1.f, ws.lg))) return rc;
         if ((rc = mm(cl, lora_second(l, o_g, m->lora_g), false, ws.lg, ACT_NONE, nullptr, nullptr, 1.f, ws.g))) return rc;
-        if (par && !join_streams(ss, st, 1)) return (int)hipErrorUnknown;
+        if (!par.join()) return (int)hipErrorUnknown;
         {
             Prep7Args a{};
             a.T = (int)T; a.C = C; a.H = H; a.r = ws.r; a.k = ws.k; a.v = v; a.w_raw = ws.w_raw; a.a_raw = ws.a_raw;

@@ -513,6 +513,13 @@ class RWKV:
 
     def forward(self, tokens, state, full_output=False):
         """model.py:1443-1677.  Returns (logits fp32 [vocab] or [T, vocab], state)."""
+        cur = _lib.stream_order.before()
+        try:
+            return self._forward(tokens, state, full_output)
+        finally:
+            _lib.stream_order.after(cur)
+
+    def _forward(self, tokens, state, full_output):
         with torch.no_grad():
             if state is None:
                 state = self._new_state()

@@ -250,6 +250,13 @@ class RWKV_x070:
 
     def forward(self, idx, state, full_output=False):
         """model.py:292-302."""
+        cur = _lib.stream_order.before()
+        try:
+            return self._forward(idx, state, full_output)
+        finally:
+            _lib.stream_order.after(cur)
+
+    def _forward(self, idx, state, full_output):
         with torch.no_grad():
             if state is None:
                 state = self.generate_zero_state()

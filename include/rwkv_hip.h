@@ -216,24 +216,6 @@ size_t rwkv_v4_one_workspace(const rwkv_v4_model *m);
 int rwkv_v4_forward_one(const rwkv_v4_model *m, const rwkv_v4_layer_state *states, const int32_t *token,
                         float *logits, void *workspace, size_t workspace_bytes, void *stream);
 
-/* Measurement aid: the same step as rwkv_v4_forward_one with a HIP event recorded on `stream`
- * around every kernel launch.  Blocks until the step has finished and writes the elapsed
- * milliseconds of the 4 * n_layer + 1 launches to ms[] in launch order: per layer (time-mix
- * k/v/r + WKV, time-mix output, channel-mix r/k, channel-mix value), then the head.
- * Not capturable (it synchronises). */
-int rwkv_v4_profile_one(const rwkv_v4_model *m, const rwkv_v4_layer_state *states, const int32_t *token,
-                        float *logits, void *workspace, size_t workspace_bytes, void *stream,
-                        float *ms, int64_t n_ms);
-
-/* Measurement aid: launches ONE phase of the step (0 time-mix k/v/r + WKV, 1 time-mix output,
- * 2 channel-mix r/k, 3 channel-mix value: once per layer, each layer streaming its own weights;
- * 4 head) `reps` times back to back between two HIP events on `stream`, blocks, and returns the
- * mean duration of one launch in milliseconds.  Results written to the state / logits are
- * meaningless: pass a scratch state. */
-int rwkv_v4_time_phase(const rwkv_v4_model *m, const rwkv_v4_layer_state *states, const int32_t *token,
-                       float *logits, void *workspace, size_t workspace_bytes, void *stream, int phase,
-                       int reps, float *ms_per_launch);
-
 /* Sequence mode (len(tokens) > 1): tokens is a device int32 [T].  logits: fp32 [vocab] for the
  * last token, or [T, vocab] when full_output != 0.  workspace: rwkv_v4_seq_workspace(m, T,
  * full_output) bytes. */

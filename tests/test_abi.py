@@ -10,10 +10,19 @@ from chatrwkv_amd import lib, synth
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
-def _declared():
-    text = open(os.path.join(ROOT, "include", "rwkv_hip.h")).read()
-    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(rwkv_[a-z0-9_]+)\s*\(", text)))
+def _declared(headers=("rwkv_hip.h", "rwkv_hip_bench.h")):
+    names = set()
+    for h in headers:
+        text = open(os.path.join(ROOT, "include", h)).read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        names |= set(re.findall(r"\b(rwkv_[a-z0-9_]+)\s*\(", text))
+    return sorted(names)
+
+
+def test_measurement_aids_are_not_in_the_product_header():
+    product = _declared(("rwkv_hip.h",))
+    assert not [n for n in product if "profile" in n or "time_phase" in n]
+    assert set(_declared(("rwkv_hip_bench.h",))) == {"rwkv_v4_profile_one", "rwkv_v4_time_phase"}
 
 
 def test_header_symbols_exported_and_bound():
