@@ -19,8 +19,9 @@ One JSON line is printed:
   isolated_mm8_op       the dequant-matmul operator alone at the 7B shapes: mm8_one GB/s, mm8_seq TFLOP/s
   prefill_roofline      the prefill contraction alone on the model's largest matrix shape: 2 T N M flops /
                         mean launch duration (HIP events), against the 2.5 PFLOP/s dense fp16 MFMA peak
-  cpu_baseline          the oracle's 'cpu fp32i8' path (numpy port of the reference's CPU arithmetic)
-                        timed on this host: a bounded sample at the 7B shape, extrapolated per token
+  cpu_baseline          the oracle's 'cpu fp32i8' path (numpy port of the reference's CPU arithmetic) timed on this
+                        host on configs[0] (169M shape, 128-token prefill + 32 greedy steps, all BLAS threads)
+  cpu_baseline_layer_sample   the same path on one layer + head of the benchmarked shape, extrapolated per token
 """
 import argparse
 import json
@@ -45,6 +46,61 @@ def u8_weight_bytes(L, C, F, V, version=4):
     v6 has 6; all have the two C x F channel-mix matrices; plus the head."""
     per_layer = (5 if version < 5.1 else 6) * C * C + 2 * C * F
     return L * per_layer + C * V
+
+
+def _cpu_info():
+    model = "unknown"
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.lower().startswith("model name"):
+                    model = line.split(":", 1)[1].strip()
+                    break
+    except OSError:
+        pass
+    try:
+        from threadpoolctl import threadpool_info
+        threads = max([p.get("num_threads", 1) for p in threadpool_info()] + [1])
+    except Exception:
+        threads = os.cpu_count() or 1
+    return model, int(threads)
+
+
+def cpu_baseline_cfg0():
+    """The reference's 'cpu fp32i8' path (oracle restatement: fp32 activations, every product dequantises its whole
+    uint8 matrix first, model.py:91-97) on BASELINE.json configs[0]: RWKV-4 169M shape, prefill of 128 tokens in
+    one call, then 32 greedy one-token steps, all BLAS threads of this host.  One warm-up pass (prefill + 2
+    steps), then the prefill three times (median) and the 32 steps once (median per step): about 20 s of CPU work.  Converted weights are random bytes and scales (the path's speed
+    does not depend on the values; the arithmetic is pinned by tests/golden/e2e_v4_169m_cpu_fp32i8.npz)."""
+    import numpy as np
+    from chatrwkv_amd import synth
+    from oracle.model import OracleRWKV
+    _, L, C, F, V = synth.SHAPES["v4-169m"]
+    o = OracleRWKV.random_converted_v4(L, C, F, V, seed=0, emb_rows=V)
+    toks = synth.random_tokens(128, V, seed=0)
+
+    out, st = o.forward(toks, None)
+    for _ in range(2):
+        out, st = o.forward([int(out.argmax())], st)
+    pre = []
+    for _ in range(3):
+        a = time.perf_counter()
+        out, st = o.forward(toks, None)
+        pre.append(time.perf_counter() - a)
+    dec = []
+    for _ in range(32):
+        a = time.perf_counter()
+        out, st = o.forward([int(out.argmax())], st)
+        dec.append(time.perf_counter() - a)
+    t_pre, t_dec = float(np.median(pre)), float(np.median(dec))
+    model, threads = _cpu_info()
+    return {
+        "value": 1.0 / t_dec, "unit": "tok/s", "cores": threads, "kind": "port",
+        "sample": (f"BASELINE.json configs[0]: RWKV-4 169M shape ({L} layers, n_embd {C}) 'cpu fp32i8', prefill 128 tokens in "
+                   f"one call (median of 3) + 32 greedy steps (median per step) after a warm-up pass, numpy oracle; value = decode tok/s"),
+        "prefill_tok_s": 128.0 / t_pre, "decode_tok_s": 1.0 / t_dec, "cpu_model": model,
+        "os_cpu_count": os.cpu_count(), "blas_threads": threads,
+    }
 
 
 def cpu_baseline(shape, budget_s=25.0):
@@ -343,7 +399,9 @@ def main():
     if args.shape == "v4-7b" and u8:
         res["isolated_mm8_op"] = isolated_mm8()
     if not args.no_cpu and version != 7:
-        res["cpu_baseline"] = cpu_baseline(args.shape)
+        # the CPU baseline proper: configs[0] in full; beside it one layer + head of the benchmarked shape
+        res["cpu_baseline"] = cpu_baseline_cfg0()
+        res["cpu_baseline_layer_sample"] = cpu_baseline(args.shape, budget_s=12.0)
     else:
         res["cpu_baseline"] = None
     print(json.dumps(res))

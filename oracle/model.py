@@ -106,7 +106,7 @@ class OracleRWKV:
             self.w = {k: (v if v.dtype == np.uint8 else v.astype(np.float64)) for k, v in self.w.items()}
 
     @classmethod
-    def random_converted_v4(cls, n_layer, n_embd, n_ffn, vocab, seed=0):
+    def random_converted_v4(cls, n_layer, n_embd, n_ffn, vocab, seed=0, emb_rows=16):
         """A 'cpu fp32i8' RWKV-4 oracle whose *converted* weights are filled directly with uniform
         random bytes and plausible scales, skipping the (slow, CPU) quantizer.  For timing the CPU
         path only: its speed does not depend on the weight values."""
@@ -117,7 +117,7 @@ class OracleRWKV:
         self.n_ffn, self.n_layer, self.version, self.n_head = n_ffn, n_layer, 4, 0
         rng = np.random.Generator(np.random.PCG64(seed))
         C, F, V = n_embd, n_ffn, vocab
-        w = {'emb.weight': rng.standard_normal((16, C), dtype=f32)}
+        w = {'emb.weight': rng.standard_normal((emb_rows, C), dtype=f32)}
 
         def qmat(name, N, M):
             w[name] = rng.integers(0, 256, size=(N, M), dtype=np.uint8)
