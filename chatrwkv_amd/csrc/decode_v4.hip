@@ -103,9 +103,12 @@ static int v4_one_impl(const rwkv_v4_model *m, const rwkv_v4_layer_state *states
                        int only_phase = -1) {
     int rc = v4_model_check(m);
     if (rc) return rc;
-    if (!states || !token || !logits || !workspace) return RWKV_E_NULL;
+    int lb, le;
+    if (!layer_range(m->n_layer, m->layer_begin, m->layer_end, lb, le)) return RWKV_E_SHAPE;
+    const bool with_head = le == m->n_layer;
+    if (!states || !token || (with_head && !logits) || !workspace) return RWKV_E_NULL;
     if (workspace_bytes < rwkv_v4_one_workspace(m) || !aligned16(workspace)) return RWKV_E_WORKSPACE;
-    for (int i = 0; i < m->n_layer; ++i) {
+    for (int i = lb; i < le; ++i) {
         const rwkv_v4_layer_state &s = states[i];
         if (!s.att_xx || !s.aa || !s.bb || !s.pp || !s.ffn_xx) return RWKV_E_NULL;
         if (!aligned16(s.att_xx) || !aligned16(s.ffn_xx)) return RWKV_E_LAYOUT;
@@ -126,7 +129,7 @@ static int v4_one_impl(const rwkv_v4_model *m, const rwkv_v4_layer_state *states
     auto mark = [&]() { if (ev) (void)hipEventRecord(ev[nev++], st); };
     mark();
 
-    for (int i = 0; i < m->n_layer; ++i) {
+    for (int i = lb; i < le; ++i) {
         const rwkv_v4_layer &l = m->layers[i];
         const rwkv_v4_layer_state &s = states[i];
         const int32_t *tok = (i == 0) ? token : nullptr;
@@ -173,7 +176,7 @@ static int v4_one_impl(const rwkv_v4_model *m, const rwkv_v4_layer_state *states
         }
         RWKV_LAUNCH_CHECK();
     }
-    if (only_phase < 0 || only_phase == 4) rc = v4_head_launch(m, ws.x, logits, st);
+    if (with_head && (only_phase < 0 || only_phase == 4)) rc = v4_head_launch(m, ws.x, logits, st);
     mark();
     return rc;
 }

@@ -67,6 +67,13 @@ int num_cu();
 
 // Is this matrix uint8?  weights_u8 0: no matrix is, 1: every matrix is, 2: decided per layer (and for the head) by
 // the presence of the scale vectors -- a strategy such as 'cuda fp16i8 *20 -> cuda fp16'.
+// The layer range [begin, end) of a model-level call (0 / 0 = all layers); false when it is not a range of the model.
+inline bool layer_range(int n_layer, int begin, int end, int &lb, int &le) {
+    lb = begin;
+    le = (begin == 0 && end == 0) ? n_layer : end;
+    return lb >= 0 && lb < le && le <= n_layer;
+}
+
 inline bool mat_is_u8(int weights_u8, const rwkv_mat &m) { return weights_u8 == 2 ? m.mx != nullptr : weights_u8 != 0; }
 
 // Two extra streams (default priority) for contractions that are independent and each too small to fill the chip;

@@ -437,11 +437,14 @@ extern "C" int rwkv_v4_forward_seq(const rwkv_v4_model *m, const rwkv_v4_layer_s
                                    size_t workspace_bytes, void *stream) {
     int rc = v4_model_check(m);
     if (rc) return rc;
-    if (!states || !tokens || !logits || !workspace) return RWKV_E_NULL;
+    int lb, le;
+    if (!layer_range(m->n_layer, m->layer_begin, m->layer_end, lb, le)) return RWKV_E_SHAPE;
+    const bool with_head = le == m->n_layer;
+    if (!states || !tokens || (with_head && !logits) || !workspace) return RWKV_E_NULL;
     if (T <= 0 || T > (1 << 20)) return RWKV_E_SHAPE;
     if (workspace_bytes < rwkv_v4_seq_workspace(m, T, full_output) || (((uintptr_t)workspace) & 255))
         return RWKV_E_WORKSPACE;
-    for (int i = 0; i < m->n_layer; ++i) {
+    for (int i = lb; i < le; ++i) {
         const rwkv_v4_layer_state &s = states[i];
         if (!s.att_xx || !s.aa || !s.bb || !s.pp || !s.ffn_xx) return RWKV_E_NULL;
         if (!aligned16(s.att_xx) || !aligned16(s.ffn_xx)) return RWKV_E_LAYOUT;
@@ -453,10 +456,11 @@ extern "C" int rwkv_v4_forward_seq(const rwkv_v4_model *m, const rwkv_v4_layer_s
     float *s2[3] = {ws.sums + T, ws.sums + 3 * T, ws.sums + 5 * T};
     float *s0v = ws.sums + 6 * T, *s2v = ws.sums + 7 * T;
 
-    hipLaunchKernelGGL(gather_emb_kernel, dim3((unsigned)T), dim3(256), 0, st, (int)T, C, (int)m->vocab, tokens, m->emb, ws.x);
+    if (lb == 0)
+        hipLaunchKernelGGL(gather_emb_kernel, dim3((unsigned)T), dim3(256), 0, st, (int)T, C, (int)m->vocab, tokens, m->emb, ws.x);
     SideStreams *ss = T >= 256 ? side_streams(st) : nullptr;
 
-    for (int i = 0; i < m->n_layer; ++i) {
+    for (int i = lb; i < le; ++i) {
         const rwkv_v4_layer &l = m->layers[i];
         const rwkv_v4_layer_state &s = states[i];
         const bool u8 = mat_is_u8(m->weights_u8, l.att_key);
@@ -555,6 +559,7 @@ extern "C" int rwkv_v4_forward_seq(const rwkv_v4_model *m, const rwkv_v4_layer_s
         if ((rc = run_gemm(l.ffn_value, u8, T, a_v, s0v, s2v, ws.x, C, e, st, ws.splitk))) return rc;
         RWKV_LAUNCH_CHECK();
     }
+    if (!with_head) return RWKV_OK;
     if (!full_output) return v4_head_launch(m, ws.x + (size_t)(T - 1) * C, logits, st);
     const bool u8 = mat_is_u8(m->weights_u8, m->head);
     {

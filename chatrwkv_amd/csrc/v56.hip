@@ -227,10 +227,13 @@ extern "C" int rwkv_v56_forward(const rwkv_v56_model *m, const rwkv_v56_layer_st
                                 void *stream) {
     int rc = v56_check(m);
     if (rc) return rc;
-    if (!states || !tokens || !logits || !workspace) return RWKV_E_NULL;
+    int lb, le;
+    if (!layer_range(m->n_layer, m->layer_begin, m->layer_end, lb, le)) return RWKV_E_SHAPE;
+    const bool with_head = le == m->n_layer;
+    if (!states || !tokens || (with_head && !logits) || !workspace) return RWKV_E_NULL;
     if (T <= 0 || T > (1 << 20)) return RWKV_E_SHAPE;
     if (workspace_bytes < rwkv_v56_workspace(m, T) || (((uintptr_t)workspace) & 255)) return RWKV_E_WORKSPACE;
-    for (int i = 0; i < m->n_layer; ++i) {
+    for (int i = lb; i < le; ++i) {
         const rwkv_v56_layer_state &s = states[i];
         if (!s.att_xx || !s.att_kv || !s.ffn_xx) return RWKV_E_NULL;
         if (!aligned16(s.att_xx) || !aligned16(s.ffn_xx)) return RWKV_E_LAYOUT;
@@ -252,8 +255,8 @@ extern "C" int rwkv_v56_forward(const rwkv_v56_model *m, const rwkv_v56_layer_st
             cs[j].splitk = nullptr;
         }
 
-    if ((rc = gather_emb_launch(T, C, m->vocab, tokens, m->emb, ws.x, st))) return rc;
-    for (int i = 0; i < m->n_layer; ++i) {
+    if (lb == 0 && (rc = gather_emb_launch(T, C, m->vocab, tokens, m->emb, ws.x, st))) return rc;
+    for (int i = lb; i < le; ++i) {
         const rwkv_v56_layer &l = m->layers[i];
         const rwkv_v56_layer_state &s = states[i];
         const bool u8 = mat_is_u8(m->weights_u8, l.att_key);
@@ -421,6 +424,7 @@ extern "C" int rwkv_v56_forward(const rwkv_v56_model *m, const rwkv_v56_layer_st
         RWKV_LAUNCH_CHECK();
     }
     // ---- head
+    if (!with_head) return RWKV_OK;
     const bool u8 = mat_is_u8(m->weights_u8, m->head);
     const bool all_rows = full_output && T > 1;
     const int64_t TH = all_rows ? T : 1;

@@ -64,7 +64,8 @@ class RwkvV4Model(ctypes.Structure):
     _fields_ = [("n_layer", ctypes.c_int32), ("n_embd", ctypes.c_int32), ("n_ffn", ctypes.c_int32),
                 ("vocab", ctypes.c_int32), ("rescale_layer", ctypes.c_int32), ("weights_u8", ctypes.c_int32),
                 ("emb", _vp), ("ln_out_w", _vp), ("ln_out_b", _vp), ("head", RwkvMat),
-                ("layers", ctypes.POINTER(RwkvV4Layer))]
+                ("layers", ctypes.POINTER(RwkvV4Layer)),
+                ("layer_begin", ctypes.c_int32), ("layer_end", ctypes.c_int32)]
 
 
 class RwkvV56Layer(ctypes.Structure):
@@ -88,7 +89,8 @@ class RwkvV56Model(ctypes.Structure):
                 ("lora_maa", ctypes.c_int32), ("lora_decay", ctypes.c_int32),
                 ("rescale_layer", ctypes.c_int32), ("weights_u8", ctypes.c_int32),
                 ("emb", _vp), ("ln_out_w", _vp), ("ln_out_b", _vp), ("head", RwkvMat),
-                ("layers", ctypes.POINTER(RwkvV56Layer))]
+                ("layers", ctypes.POINTER(RwkvV56Layer)),
+                ("layer_begin", ctypes.c_int32), ("layer_end", ctypes.c_int32)]
 
 
 class RwkvV7Layer(ctypes.Structure):

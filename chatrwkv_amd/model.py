@@ -34,6 +34,8 @@ from . import strategy as _strategy
 from .state import StateList
 
 _MATRIX_KEYS = ('key.weight', 'value.weight', 'receptance.weight', 'gate.weight', 'output.weight', 'head.weight')
+# the tensors a streamed slot keeps in pinned host memory (model.py:854)
+_STREAMED_KEYS = ('key.weight', 'value.weight', 'receptance.weight', 'output.weight')
 
 
 def _ptr(t):
@@ -117,6 +119,7 @@ class RWKV:
             if convert_and_save_and_exit:
                 self._save_converted(convert_and_save_and_exit, prxxx)
                 raise SystemExit(0)                                   # model.py:903
+            self._plan_staging()
             if self.version == 4:
                 self._build_descriptors()
             else:
@@ -160,6 +163,8 @@ class RWKV:
                 if is_matrix:
                     # reference device layout [in, out] with out contiguous -> input-contiguous
                     out[x] = _ops.to_input_contiguous(t.to(dev))
+                    if self.strategy[layer_id if 'blocks.' in x else args.n_layer].stream and x.endswith(_STREAMED_KEYS):
+                        out[x] = self._to_pinned(out[x])
                 elif x.endswith(('_mx', '_rx', '_my', '_ry')) or 'emb.' in x:
                     out[x] = t.to(dev).contiguous()
                 else:
@@ -180,6 +185,8 @@ class RWKV:
                 else:
                     out[x] = t.to(torch.float16).t()
                 del t
+                if slot.stream and x.endswith(_STREAMED_KEYS):            # model.py:854-858
+                    out[x] = self._to_pinned(out[x])
                 continue
             t = t.detach().to('cpu')
             if '.time_' in x:
@@ -208,6 +215,13 @@ class RWKV:
         torch.cuda.synchronize()
         return out
 
+    @staticmethod
+    def _to_pinned(t):
+        """An input-contiguous [N, M] device matrix as a pinned host tensor of the same shape and strides."""
+        host = torch.empty((t.shape[1], t.shape[0]), dtype=t.dtype, pin_memory=True)   # allocated pinned
+        host.copy_(t.t())
+        return host.t()
+
     def _save_converted(self, path, prxxx):
         """model.py:894-903: the converted dict in the reference's own layout ([in, out] matrices
         with the output index contiguous) so that either implementation can load the file."""
@@ -232,10 +246,54 @@ class RWKV:
         assert t.stride(0) == 1, name
         m = _lib.RwkvMat()
         m.w, m.ld, m.N, m.M = t.data_ptr(), t.stride(1), N, M
+        if not t.is_cuda:
+            m.w = self._stage_ptr[name]       # a streamed matrix: the kernels read its place in the staging buffer
         if t.dtype == torch.uint8:
             m.mx, m.rx = w[name + '_mx'].data_ptr(), w[name + '_rx'].data_ptr()
             m.my, m.ry = w[name + '_my'].data_ptr(), w[name + '_ry'].data_ptr()
         return m
+
+    def _plan_staging(self):
+        """Streamed layers (model.py:854-858, 1526-1530, 1617-1620): their key / value / receptance / output matrices
+        live in pinned host memory and are copied into ONE device staging buffer, sized for the largest such layer,
+        right before the layer runs; every streamed layer's descriptors point into that buffer."""
+        self._stage_ptr, self._stage_plan, sizes = {}, {}, {}
+        for name, t in self.w.items():
+            if isinstance(t, torch.Tensor) and not t.is_cuda and t.dim() == 2 and name.endswith(_STREAMED_KEYS):
+                layer = int(name.split('.')[1])
+                off = sizes.get(layer, 0)
+                nbytes = t.numel() * t.element_size()
+                self._stage_plan.setdefault(layer, []).append((name, t.t().reshape(-1).view(torch.uint8), off, nbytes))
+                sizes[layer] = off + ((nbytes + 255) & ~255)
+        self._staging = None
+        if sizes:
+            self._staging = torch.empty(max(sizes.values()), dtype=torch.uint8, device=self.device)
+            for layer, items in self._stage_plan.items():
+                for name, _, off, _ in items:
+                    self._stage_ptr[name] = self._staging.data_ptr() + off
+        # the calls one forward pass is made of: runs of resident layers, and every streamed layer alone
+        self._segments, i, L = [], 0, self.args.n_layer
+        while i < L:
+            if i in self._stage_plan:
+                self._segments.append((i, i + 1))
+                i += 1
+            else:
+                j = i
+                while j < L and j not in self._stage_plan:
+                    j += 1
+                self._segments.append((i, j))
+                i = j
+
+    def _run_segments(self, call):
+        """call() once per segment with the model's layer range set, the streamed layer's matrices copied first
+        (same stream: the copy follows the previous layer's kernels and precedes this layer's)."""
+        m = self._model
+        for lb, le in self._segments:
+            for _, host, off, nbytes in self._stage_plan.get(lb, ()):
+                self._staging[off:off + nbytes].copy_(host, non_blocking=True)
+            m.layer_begin, m.layer_end = lb, le
+            call()
+        m.layer_begin = m.layer_end = 0
 
     def _build_descriptors(self):
         a, w = self.args, self.w
@@ -417,16 +475,18 @@ class RWKV:
     # ------------------------------------------------------------------ forward
     def _launch_one(self, sdesc):
         L = _lib.load()
-        if self.version != 4:
-            rc = L.rwkv_v56_forward(ctypes.byref(self._model), sdesc, self._token_dev.data_ptr(), 1, 0,
-                                    self._logits.data_ptr(), self._one_ws.data_ptr(), self._one_ws.numel(),
-                                    torch.cuda.current_stream().cuda_stream)
-            _lib.check(rc, "rwkv_v56_forward")
-            return
-        rc = L.rwkv_v4_forward_one(ctypes.byref(self._model), sdesc, self._token_dev.data_ptr(),
-                                   self._logits.data_ptr(), self._one_ws.data_ptr(), self._one_ws.numel(),
-                                   torch.cuda.current_stream().cuda_stream)
-        _lib.check(rc, "rwkv_v4_forward_one")
+        st = torch.cuda.current_stream().cuda_stream
+
+        def call():
+            if self.version != 4:
+                rc = L.rwkv_v56_forward(ctypes.byref(self._model), sdesc, self._token_dev.data_ptr(), 1, 0,
+                                        self._logits.data_ptr(), self._one_ws.data_ptr(), self._one_ws.numel(), st)
+                _lib.check(rc, "rwkv_v56_forward")
+            else:
+                rc = L.rwkv_v4_forward_one(ctypes.byref(self._model), sdesc, self._token_dev.data_ptr(),
+                                           self._logits.data_ptr(), self._one_ws.data_ptr(), self._one_ws.numel(), st)
+                _lib.check(rc, "rwkv_v4_forward_one")
+        self._run_segments(call)
 
     def _forward_one(self, token, state):
         if isinstance(token, torch.Tensor):
@@ -437,7 +497,7 @@ class RWKV:
             self._token_dev.fill_(int(token))
         use_graph = os.environ.get("RWKV_HIP_GRAPH", "1") != "0"
         key = None
-        if use_graph and isinstance(state, StateList) and state.intact():
+        if use_graph and not self._stage_plan and isinstance(state, StateList) and state.intact():
             key = tuple(t.data_ptr() for t in state.flat)
         if key is None:
             self._launch_one(self._state_desc(state))
@@ -505,10 +565,13 @@ class RWKV:
         V = self._model.vocab
         logits = torch.empty((T, V) if full_output else (V,), dtype=torch.float32, device=self.device)
         fn = L.rwkv_v4_forward_seq if self.version == 4 else L.rwkv_v56_forward
-        rc = fn(ctypes.byref(self._model), self._state_desc(state), tok.data_ptr(), T,
-                int(full_output), logits.data_ptr(), self._seq_ws.data_ptr(),
-                self._seq_ws.numel(), torch.cuda.current_stream().cuda_stream)
-        _lib.check(rc, "forward (sequence mode)")
+        sdesc, st = self._state_desc(state), torch.cuda.current_stream().cuda_stream
+
+        def call():
+            rc = fn(ctypes.byref(self._model), sdesc, tok.data_ptr(), T, int(full_output), logits.data_ptr(),
+                    self._seq_ws.data_ptr(), self._seq_ws.numel(), st)
+            _lib.check(rc, "forward (sequence mode)")
+        self._run_segments(call)
         return logits, state
 
     def forward(self, tokens, state, full_output=False):

@@ -4,10 +4,12 @@ Restates the planner of RWKV.__init__ (rwkv_pip_package/src/rwkv/model.py:620-75
 strategy is a chain of segments ``device dtype[i8] [*N | *N+]`` joined by ``->``; the
 n_layer + 1 slots (the last one holds ln_out + head, model.py:776-778) are dealt to the
 segments in order.  This package then runs only plans that put every slot on one ROCm
-GPU with fp16 activations and uint8 or fp16 weights: 'cuda fp16i8', 'cuda fp16', and chains of the
+GPU with fp16 activations and uint8 or fp16 weights: 'cuda fp16i8', 'cuda fp16', chains of the
 two on the same GPU such as 'cuda fp16i8 *20 -> cuda fp16' (uint8 weights for the first 20 layers,
-fp16 for the rest and the head).  Any other valid strategy raises NotImplementedError, an invalid
-string raises ValueError as the reference does (model.py:621-622).
+fp16 for the rest and the head), and streamed segments ('cuda fp16i8 *10+': the big matrices of the layers
+after the first 10 stay in pinned host memory and are copied to the GPU for every call, model.py:854-858,
+1526-1530).  Any other valid strategy raises NotImplementedError, an invalid string raises ValueError as the
+reference does (model.py:621-622).
 """
 import re
 import types
@@ -94,10 +96,10 @@ def require_single_gpu(slots):
     for s in slots:
         if s is None:
             raise NotImplementedError("strategy leaves layers unassigned")
-        if not str(s.device).startswith("cuda") or s.stream:
+        if not str(s.device).startswith("cuda"):
             raise NotImplementedError(
-                "chatrwkv_amd runs single-GPU strategies only ('cuda fp16i8', 'cuda fp16' and chains of the two); "
-                f"got device {s.device!r}{' with streaming' if s.stream else ''}")
+                "chatrwkv_amd runs single-GPU strategies only ('cuda fp16i8', 'cuda fp16', chains of the two, "
+                f"streamed or not); got device {s.device!r}")
         if s.device not in ("cuda", "cuda:0"):
             raise NotImplementedError("chatrwkv_amd uses GPU 0 only")
         if s.atype != torch.float16 or s.wtype not in (torch.uint8, torch.float16):

@@ -44,7 +44,7 @@ typedef uint16_t rwkv_half;
 #define RWKV_DT_F16 0
 #define RWKV_DT_F32 1
 
-/* Library / device identification.  Returns the ABI version (currently 1). */
+/* Library / device identification.  Returns the ABI version (currently 2). */
 int rwkv_abi_version(void);
 
 /* ---------------------------------------------------------------------------------------
@@ -205,6 +205,12 @@ typedef struct {
     const rwkv_half *ln_out_w, *ln_out_b;
     rwkv_mat head;          /* [C -> vocab] */
     const rwkv_v4_layer *layers; /* host array [n_layer] */
+    /* Layer range of this call: [layer_begin, layer_end), 0 / 0 = the whole model.  The embedding gather runs when
+     * layer_begin == 0 and ln_out + head when layer_end reaches n_layer (logits may be NULL otherwise); between
+     * the calls of one forward pass the running activation stays in the workspace, so they must share it (and
+     * T).  This is how a streamed strategy ('cuda fp16i8 *10+', model.py:854-858, 1526-1530) runs: the caller
+     * copies the matrices of one streamed layer to the device, then calls for that layer alone. */
+    int32_t layer_begin, layer_end;
 } rwkv_v4_model;
 
 /* One-token step (len(tokens) == 1).  `token` is a device int32: the kernels read the id from
@@ -262,6 +268,7 @@ typedef struct {
     const rwkv_half *emb, *ln_out_w, *ln_out_b;
     rwkv_mat head;
     const rwkv_v56_layer *layers;
+    int32_t layer_begin, layer_end;   /* as in rwkv_v4_model */
 } rwkv_v56_model;
 
 size_t rwkv_v56_workspace(const rwkv_v56_model *m, int64_t T);

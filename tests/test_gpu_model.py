@@ -769,3 +769,37 @@ def test_calls_from_two_streams_are_ordered(tiny_models):
     torch.cuda.synchronize()
     for a, b in zip(outs, refs):
         assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("ver", [4, 5.2, 6])
+@pytest.mark.parametrize("strat,same_as,first", [("cuda fp16i8 *1+", "cuda fp16i8", 1), ("cuda fp16 *0+", "cuda fp16", 0),
+                                                 ("cuda fp16i8 *1 -> cuda fp16 *1+", "cuda fp16i8 *1 -> cuda fp16", 2)])
+def test_streamed_strategy(ver, strat, same_as, first):
+    """'*N+' (model.py:686-747, 854-858, 1526-1530): the key / value / receptance / output matrices of the streamed
+    layers live in pinned host memory and are copied to the GPU for every call, layer by layer.  Same kernels on the
+    same bytes: logits and states equal those of the strategy without the '+', bit for bit."""
+    ck = synth.make_checkpoint(version=ver, seed=610 + int(ver * 10), **TINY)
+    m, ref = _rwkv()(ck, strat, verbose=False), _rwkv()(ck, same_as, verbose=False)
+    streamed = [i for i in range(TINY["n_layer"]) if m.strategy[i].stream]
+    assert streamed == list(range(first, TINY["n_layer"]))
+    for i in range(TINY["n_layer"]):
+        for name in ("att.key.weight", "att.output.weight", "ffn.value.weight"):
+            t = m.w[f"blocks.{i}.{name}"]
+            assert t.is_cuda != (i in streamed) and (t.is_cuda or t.is_pinned()), (i, name)
+            assert torch.equal(t.cpu(), ref.w[f"blocks.{i}.{name}"].cpu())
+        if ver != 4:
+            assert m.w[f"blocks.{i}.att.gate.weight"].is_cuda        # not among the streamed tensors (model.py:854)
+    assert m.w["head.weight"].is_cuda
+    toks = synth.random_tokens(48, TINY["vocab"], seed=PROMPT_SEED)
+    a, sa = m.forward(toks[:40], None, full_output=True)
+    b, sb = ref.forward(toks[:40], None, full_output=True)
+    assert torch.equal(a, b)
+    for t in toks[40:]:
+        a, sa = m.forward([t], sa)
+        b, sb = ref.forward([t], sb)
+        assert torch.equal(a, b)
+    a, sa = m.forward(toks[:3], sa)
+    b, sb = ref.forward(toks[:3], sb)
+    assert torch.equal(a, b)
+    for x, y in zip(sa, sb):
+        assert torch.equal(x, y)

@@ -37,7 +37,11 @@ def test_only_single_gpu_plans_are_accepted():
     assert strategy.require_single_gpu(strategy.plan("cuda fp16i8 *1 -> cuda fp16", 4)) == "mixed"
     assert strategy.require_single_gpu(strategy.plan("cuda:0 fp16 *2 -> cuda fp16i8", 4)) == "mixed"
     assert strategy.require_single_gpu(strategy.plan("cuda fp16i8 *9 -> cuda fp16", 4)) == "u8"   # the first segment takes all
-    for s in ("cpu fp32", "cpu fp32i8", "cuda fp32", "cuda bf16", "cuda fp16i8 -> cpu fp32 *1", "cuda fp16 *2+",
+    # streamed segments on the one GPU: the slots after the first two stream (the head slot among them)
+    slots = strategy.plan("cuda fp16 *2+", 4)
+    assert strategy.require_single_gpu(slots) == "f16" and [s.stream for s in slots] == [False, False, True, True, True]
+    assert strategy.require_single_gpu(strategy.plan("cuda fp16i8 *1 -> cuda fp16 *1+", 4)) == "mixed"
+    for s in ("cpu fp32", "cpu fp32i8", "cuda fp32", "cuda bf16", "cuda fp16i8 -> cpu fp32 *1", "cuda fp16 *2+ -> cpu fp32 *1",
               "cuda fp16 -> cuda:1 fp16", "cuda:1 fp16", "cuda fp16i8 *1 -> cuda fp32"):
         with pytest.raises(NotImplementedError):
             strategy.require_single_gpu(strategy.plan(s, 4))
