@@ -8,7 +8,8 @@ import ctypes
 import os
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(HERE, "librwkv_hip.so")
+# RWKV_HIP_LIB: another build of the same library (kernel tuning: two builds side by side)
+LIB_PATH = os.environ.get("RWKV_HIP_LIB") or os.path.join(HERE, "librwkv_hip.so")
 
 RWKV_DT_F16, RWKV_DT_F32 = 0, 1
 
