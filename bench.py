@@ -35,9 +35,13 @@ if ROOT not in sys.path:
 
 HBM_PEAK = 8.0e12      # bytes/s, MI355X HBM3E
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by a 1 GiB copy
-# kernel: x2.0 / x1.0); profiles/decode_7b_fp16i8_hbm_traffic.md has the commands and the table
-MEASURED_TRAFFIC = {("v4-7b", "cuda fp16i8", 32, "ffn_rk"): 85068800 + 49254,
-                    ("v4-7b", "cuda fp16i8", 32, "att_kvr_wkv"): 52143309 + 65536}
+# kernel: x2.0 / x1.0).  Counter figures, not read in this run: TRAFFIC_SOURCE has the commands and the table, and
+# every roofline object names it next to the number so that a stale value can be told from a fresh one.
+TRAFFIC_SOURCE = "profiles/decode_7b_fp16i8_hbm_traffic.md"
+MEASURED_TRAFFIC = {("v4-7b", "cuda fp16i8", 32, "ffn_rk"): 85082112 + 49254,
+                    ("v4-7b", "cuda fp16i8", 32, "att_kvr_wkv"): 52142694 + 65536,
+                    # the prefill contraction [1024 x 4096] x [4096 x 16384], uint8 weights, 256 x 256 tiles
+                    ("gemm", 1024, 4096, 16384, True): 134557082 + 33554432}
 MFMA_F16_PEAK = 2.5e15  # flop/s dense fp16
 
 
@@ -194,7 +198,9 @@ def gemm_roofline(T, N, M, u8, reps=10):
     t = e0.elapsed_time(e1) * 1e-3 / reps
     flops = 2.0 * T * N * M
     return {"bound": "mfma", "kernel": f"{name}, [{T} x {N}] x [{N} x {M}]", "achieved": flops / t / 1e12,
-            "peak": MFMA_F16_PEAK / 1e12, "unit": "TFLOP/s", "frac": flops / t / MFMA_F16_PEAK, "traffic": None,
+            "peak": MFMA_F16_PEAK / 1e12, "unit": "TFLOP/s", "frac": flops / t / MFMA_F16_PEAK,
+            "traffic": MEASURED_TRAFFIC.get(("gemm", T, N, M, bool(u8))),
+            "traffic_source": TRAFFIC_SOURCE if ("gemm", T, N, M, bool(u8)) in MEASURED_TRAFFIC else None,
             "flops_per_launch": flops, "ms_per_launch": t * 1e3}
 
 
@@ -358,6 +364,7 @@ def main():
         roof = {"bound": "hbm", "kernel": kname, "achieved": kbytes[dom] / (kms[dom] * 1e-3) / 1e9,
                 "peak": HBM_PEAK / 1e9, "unit": "GB/s", "frac": kbytes[dom] / (kms[dom] * 1e-3) / HBM_PEAK,
                 "traffic": MEASURED_TRAFFIC.get((args.shape, args.strategy, L, dom)),
+                "traffic_source": TRAFFIC_SOURCE if (args.shape, args.strategy, L, dom) in MEASURED_TRAFFIC else None,
                 "bytes_per_launch": kbytes[dom], "ms_per_launch": kms[dom]}
     else:
         # RWKV-5/6 one-token steps are a chain of the same streaming GEMV launches with no per-phase timing
