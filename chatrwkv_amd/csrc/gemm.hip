@@ -734,6 +734,161 @@ __global__ __launch_bounds__(256) void mm8_prepare_group_kernel(int T, int N, Pr
 }
 
 
+
+// ---- calls of 2 .. 16 rows: every weight row streamed once ---------------------------------------------------
+// A ragged last prompt chunk (rwkv/utils.py:98-101) or a short chat turn has a handful of tokens: with 128-row
+// tiles the contraction kernels spend their time on empty rows and a call costs several one-token steps.  Here
+// a workgroup of 16 waves takes 16 output rows at a time and splits K over its waves: wave w owns the k-chunks
+// w, w + 16, ... (64 wide for uint8 rows, 32 for fp16 rows); per chunk a lane loads 16 bytes of one weight row
+// (lane = row + 16 q: the four lanes of a row cover 64 contiguous bytes) and the matching 16 / 8 activation values
+// of one token (lane = token + 16 q, rows past T repeat the last one), widens uint8 to the exact fp16 value b + 1/2
+// and issues v_mfma_f32_16x16x32_f16 with the weights as the first and the activations as the second operand, so
+// that lane (token j, q) ends with rows 4 q .. 4 q + 3 of token j.  The 16 partial 16 x 16 blocks are added in wave
+// order through LDS (deterministic), and 256 threads run the same epilogue as the large kernels.  Activations come
+// from L2 (T x N values, re-read per row group); weights from HBM, each byte once.
+struct SkinnyGroup {
+    const h16 *A[4];
+    const void *W[4];
+    void *Y[4];
+    int64_t lda, ldw[4], ldy[4];
+    int M[4];
+    GemmEpi ep[4];
+};
+
+// NCI > 0: a wave owns at most NCI chunks and keeps their activation values in registers for all its row groups
+// (rows of up to 16 * NCI chunks: the loop then issues weight loads only); NCI == 0: any row length, activations
+// re-read from L2 for every row group.
+template <bool W_U8, int NCI>
+__global__ __launch_bounds__(1024) void skinny_kernel(int T, int N, SkinnyGroup g) {
+    __shared__ float red[16][64][4];
+    const int gi = blockIdx.y, M = g.M[gi];
+    const h16 *__restrict__ A = g.A[gi];
+    const unsigned char *__restrict__ W = (const unsigned char *)g.W[gi];
+    const int64_t lda = g.lda, ldw = g.ldw[gi];
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int sub = lane & 15, q = lane >> 4;
+    constexpr int CK = W_U8 ? 64 : 32;               // k values per chunk
+    const int nchunks = N / CK;
+    const int ngroups = (M + 15) >> 4;
+    const h16 *arow = A + (size_t)min(sub, T - 1) * lda;   // this lane's token
+    const h16x2 off = {(h16)1023.5f, (h16)1023.5f};
+    constexpr int NB = NCI > 0 ? NCI : 4;            // chunks loaded before any is multiplied
+    auto load_x = [&](int c, h16x8 &x0, h16x8 &x1) {
+        if (W_U8) {
+            x0 = *(const h16x8 *)(arow + (size_t)c * 64 + 16 * q);
+            x1 = *(const h16x8 *)(arow + (size_t)c * 64 + 16 * q + 8);
+        } else {
+            x0 = *(const h16x8 *)(arow + (size_t)c * 32 + 8 * q);
+            x1 = x0;
+        }
+    };
+    auto load_w = [&](const unsigned char *wrow, int c) {
+        if (W_U8) return __builtin_nontemporal_load((const u32x4 *)(wrow + (size_t)c * 64 + 16 * q));
+        return __builtin_nontemporal_load((const u32x4 *)(wrow + ((size_t)c * 32 + 8 * q) * 2));
+    };
+    auto multiply = [&](u32x4 wv, h16x8 x0, h16x8 x1, f32x4 &acc) {
+        if (W_U8) {
+            const h16x2 a0 = u8pair_lo_1024(wv.x) - off, a1 = u8pair_hi_1024(wv.x) - off;
+            const h16x2 a2 = u8pair_lo_1024(wv.y) - off, a3 = u8pair_hi_1024(wv.y) - off;
+            const h16x2 b0 = u8pair_lo_1024(wv.z) - off, b1 = u8pair_hi_1024(wv.z) - off;
+            const h16x2 b2 = u8pair_lo_1024(wv.w) - off, b3 = u8pair_hi_1024(wv.w) - off;
+            const h16x8 wa = {a0.x, a0.y, a1.x, a1.y, a2.x, a2.y, a3.x, a3.y};
+            const h16x8 wb = {b0.x, b0.y, b1.x, b1.y, b2.x, b2.y, b3.x, b3.y};
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(wa, x0, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(wb, x1, acc, 0, 0, 0);
+        } else {
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h16x8, wv), x0, acc, 0, 0, 0);
+        }
+    };
+    // chunks past the end of the row repeat the last one and multiply zeros: no branch sits between the loads and
+    // their use (loads would be sunk behind it, one chunk in flight at a time)
+    h16x8 rx0[NB], rx1[NB];
+    if (NCI > 0) {
+#pragma unroll
+        for (int i = 0; i < NB; ++i) {
+            load_x(min(wave + 16 * i, nchunks - 1), rx0[i], rx1[i]);
+            if (wave + 16 * i >= nchunks) { rx0[i] = h16x8{}; rx1[i] = h16x8{}; }
+        }
+    }
+    for (int grp = blockIdx.x; grp < ngroups; grp += gridDim.x) {
+        const int m0 = grp << 4;
+        const unsigned char *wrow = W + (size_t)min(m0 + sub, M - 1) * ldw * (W_U8 ? 1 : 2);
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+        if (NCI > 0) {
+            u32x4 wv[NB];
+#pragma unroll
+            for (int i = 0; i < NB; ++i) wv[i] = load_w(wrow, min(wave + 16 * i, nchunks - 1));
+#pragma unroll
+            for (int i = 0; i < NB; ++i) multiply(wv[i], rx0[i], rx1[i], acc);
+        } else {
+            for (int c0 = wave; c0 < nchunks; c0 += 16 * NB) {
+                u32x4 wv[NB];
+                h16x8 x0[NB], x1[NB];
+#pragma unroll
+                for (int i = 0; i < NB; ++i) {
+                    const int c = min(c0 + 16 * i, nchunks - 1);
+                    wv[i] = load_w(wrow, c);
+                    load_x(c, x0[i], x1[i]);
+                }
+#pragma unroll
+                for (int i = 0; i < NB; ++i) {
+                    if (c0 + 16 * i >= nchunks) { x0[i] = h16x8{}; x1[i] = h16x8{}; }
+                    multiply(wv[i], x0[i], x1[i], acc);
+                }
+            }
+        }
+        __syncthreads();                                          // the previous group's sums have been read
+        *(f32x4 *)&red[wave][lane][0] = acc;
+        __syncthreads();
+        if (threadIdx.x < 256) {
+            const int l = threadIdx.x & 63, r = threadIdx.x >> 6;
+            float v = 0.f;
+#pragma unroll
+            for (int w = 0; w < 16; ++w) v += red[w][l][r];
+            const int m = m0 + 4 * (l >> 4) + r, t = l & 15;
+            if (m < M && t < T) {
+                const GemmEpi &ep = g.ep[gi];
+                float rxm = 1.f, mxm = 0.f;
+                if (ep.rx) { rxm = h2f(ep.rx[m]); mxm = h2f(ep.mx[m]); }
+                gemm_epilogue(v, t, m, rxm, mxm, ep, g.Y[gi], g.ldy[gi]);
+            }
+        }
+    }
+}
+
+constexpr int SKINNY_MAX_ROWS = 16;
+
+// what skinny_kernel assumes of one product: whole chunks, 16-byte aligned rows for its 16-byte loads
+bool skinny_ok(bool w_u8, int64_t T, int64_t N, const void *A, int64_t lda, const void *W, int64_t ldw, const GemmEpi &ep) {
+    auto a16 = [](const void *p) { return (((uintptr_t)p) & 15) == 0; };
+    if (T < 2 || T > SKINNY_MAX_ROWS || N < 64 || (N % 64)) return false;
+    if ((lda & 7) || (ldw & (w_u8 ? 15 : 7)) || !a16(A) || !a16(W)) return false;
+    if (w_u8 && (!ep.rx || !ep.mx || !ep.s0 || !ep.s2)) return false;
+    if (!w_u8 && ep.rx) return false;
+    const char *e = getenv("RWKV_NO_SKINNY");                     // tuning: send short calls through the tile kernels
+    return !(e && *e == '1');
+}
+
+int skinny_launch(bool w_u8, int n, int64_t T, int64_t N, const SkinnyGroup &g, hipStream_t st) {
+    int maxg = 1;
+    for (int i = 0; i < n; ++i) maxg = std::max(maxg, (g.M[i] + 15) / 16);
+    const dim3 grid((unsigned)std::min(maxg, 2 * num_cu()), (unsigned)n);
+    const int64_t per_wave = (N / (w_u8 ? 64 : 32) + 15) / 16;    // chunks a wave owns
+#define RWKV_SKINNY(NCI)                                                                                         \
+    do {                                                                                                         \
+        if (w_u8) hipLaunchKernelGGL((skinny_kernel<true, NCI>), grid, dim3(1024), 0, st, (int)T, (int)N, g);   \
+        else hipLaunchKernelGGL((skinny_kernel<false, NCI>), grid, dim3(1024), 0, st, (int)T, (int)N, g);       \
+    } while (0)
+    if (per_wave <= 1) RWKV_SKINNY(1);
+    else if (per_wave <= 2) RWKV_SKINNY(2);
+    else if (per_wave <= 4) RWKV_SKINNY(4);
+    else if (per_wave <= 8) RWKV_SKINNY(8);
+    else RWKV_SKINNY(0);
+#undef RWKV_SKINNY
+    RWKV_LAUNCH_CHECK();
+    return RWKV_OK;
+}
+
 }  // namespace
 
 namespace {
@@ -896,6 +1051,11 @@ int pick_cfg(int64_t T, int64_t N, int64_t M, bool w_u8, bool alone, bool dma, s
 
 int gemm_launch(bool w_u8, int64_t T, int64_t N, int64_t M, const rwkv_half *A, int64_t lda, const void *W,
                 int64_t ldw, void *Y, int64_t ldy, const GemmEpi &ep, hipStream_t st) {
+    if (skinny_ok(w_u8, T, N, A, lda, W, ldw, ep)) {
+        SkinnyGroup g{};
+        g.A[0] = (const h16 *)A; g.W[0] = W; g.Y[0] = Y; g.lda = lda; g.ldw[0] = ldw; g.ldy[0] = ldy; g.M[0] = (int)M; g.ep[0] = ep;
+        return skinny_launch(w_u8, 1, T, N, g, st);
+    }
     const int cfg = pick_cfg(T, N, M, w_u8, !ep.small_tiles, dma_ok(w_u8, N, M, A, lda, W, ldw, Y, ldy, ep),
                              ep.splitk_ws ? ep.splitk_bytes : 0);
     return w_u8 ? launch_pick<true>(cfg, T, N, M, A, lda, W, ldw, Y, ldy, ep, st)
@@ -947,6 +1107,19 @@ int gemm_group_launch(bool w_u8, int n, int64_t T, int64_t N, const rwkv_half *c
         max_out = std::max<int64_t>(max_out, T * mats[i]->M);
         m4 = m4 && !(mats[i]->M & 3);
         dma = dma && dma_ok(w_u8, N, mats[i]->M, g.A[i], N, g.W[i], g.ldw[i], g.Y[i], mats[i]->M, g.ep[i]);
+    }
+    {
+        bool skinny = true;
+        for (int i = 0; i < n; ++i) skinny = skinny && skinny_ok(w_u8, T, N, g.A[i], N, g.W[i], g.ldw[i], g.ep[i]);
+        if (skinny) {
+            SkinnyGroup sg{};
+            sg.lda = N;
+            for (int i = 0; i < n; ++i) {
+                sg.A[i] = g.A[i]; sg.W[i] = g.W[i]; sg.Y[i] = g.Y[i]; sg.ldw[i] = g.ldw[i]; sg.ldy[i] = g.M[i]; sg.M[i] = g.M[i];
+                sg.ep[i] = g.ep[i];
+            }
+            return skinny_launch(w_u8, n, T, N, sg, st);
+        }
     }
     if (dma) {
         // tile size and K split of least cost, as for a single product

@@ -101,7 +101,10 @@ def test_mm8_one(N, M):
                                    # long calls: 256 x 256 tiles loaded straight into LDS; whole, ragged and split-K
                                    (4096, 8192, 1000), (16384, 4096, 520), (2560, 10240, 768),
                                    # ragged tiles of the direct-to-LDS kernel: widths and row counts that end inside a tile
-                                   (128, 200, 37), (192, 1000, 300), (64, 8, 2), (1024, 136, 129)])
+                                   (128, 200, 37), (192, 1000, 300), (64, 8, 2), (1024, 136, 129),
+                                   # 2 .. 16 rows: every weight row streamed once, K split over the 16 waves of a workgroup
+                                   (768, 768, 3), (768, 50277, 9), (4096, 4096, 2), (4096, 16384, 16), (16384, 4096, 7),
+                                   (2560, 2560, 13), (5120, 20480, 16), (128, 211, 4), (64, 24, 16), (2048, 512, 6)])
 def test_mm8_seq(N, M, B):
     ops = _ops()
     x, ref, (q, mx, rx, my, ry) = _mm8_case(N, M, B, N + M + B)
@@ -136,7 +139,9 @@ def test_mm8_linearity_full_size():
                                    (768, 768, 7), (3072, 768, 128), (4096, 4096, 300), (768, 50277, 4),
                                    # long calls (256 x 256 tiles loaded straight into LDS): split-K, ragged, shallow
                                    (4096, 4096, 1024), (4096, 8192, 520), (128, 4096, 1024),
-                                   (128, 200, 37), (192, 1000, 300), (64, 8, 2)])
+                                   (128, 200, 37), (192, 1000, 300), (64, 8, 2),
+                                   # 2 .. 16 rows: the streaming kernel
+                                   (768, 768, 3), (4096, 4096, 16), (16384, 4096, 5), (2560, 10240, 11), (128, 211, 2), (2048, 512, 6)])
 @pytest.mark.parametrize("out_dtype", [torch.float16, torch.float32])
 def test_gemm_f16(N, M, B, out_dtype):
     ops = _ops()
