@@ -519,7 +519,26 @@ DEV void gemm_dma_body(int T, int N, int M, const h16 *__restrict__ A, int64_t l
         sp = so;
         so = sn;
     }
-    __builtin_amdgcn_s_waitcnt(0x0070);   // vmcnt(0) lgkmcnt(0): nothing may land in LDS after the workgroup has gone
+    // vmcnt(0) lgkmcnt(0): nothing may land in LDS after the workgroup has gone -- and nothing in registers: the last
+    // iteration has read a fragment set that nobody multiplies.  The compiler does not know that an inline-asm
+    // ds_read writes its output later: to it those registers are dead from here on, and it reused them for the
+    // epilogue's column index and addresses ahead of this wait (a read that returned late then overwrote the
+    // index: an access far outside the buffers).  So the wait comes first, fenced against the scheduler, and every
+    // fragment register stays "in use" until it has passed.
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_waitcnt(0x0070);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int buf = 0; buf < 2; ++buf) {
+#pragma unroll
+        for (int a = 0; a < MI; ++a) asm volatile("" ::"v"(fa[buf][a]));
+#pragma unroll
+        for (int b = 0; b < NI; ++b) {
+            if constexpr (W_U8) asm volatile("" ::"v"(rawb[buf][b]));
+            else asm volatile("" ::"v"(fbh[buf][b]));
+        }
+    }
+    __builtin_amdgcn_sched_barrier(0);
 
     // Each thread finishes eight consecutive outputs of one row: 16-byte loads of the residual / gate rows, 16-byte
     // stores, and a body small enough to stay in the instruction cache (per-element code for 128 accumulators

@@ -155,13 +155,14 @@ def load():
     return lib
 
 
-class _StreamOrder:
-    """Model calls issued from different streams are put in one order on the device.
+class StreamOrder:
+    """Calls on ONE model object issued from different streams are put in one order on the device.
 
-    A forward call whose stream differs from the previous call's first makes its stream wait (on the device, no
-    host synchronisation) for the event recorded after that previous call.  Calls on one stream cost one event
-    record each and are not delayed.  Reason: a GPU memory fault was seen with sequence calls of two models in
-    flight on two streams at once and its cause has not been found; until it is, such calls do not overlap."""
+    A model object owns one workspace, one logits buffer and (streamed strategies) one staging buffer, so two of its
+    calls must not overlap.  A forward call whose stream differs from the object's previous call first makes its
+    stream wait (on the device, no host synchronisation) for the event recorded after that previous call.  Calls
+    on one stream cost one event record each and are not delayed; calls on different model objects are not ordered
+    against each other and may overlap."""
 
     def __init__(self):
         self.stream = None
@@ -180,9 +181,6 @@ class _StreamOrder:
             self.event = torch.cuda.Event()
         self.event.record(cur)
         self.stream = cur.cuda_stream
-
-
-stream_order = _StreamOrder()
 
 
 def check(rc, what):

@@ -45,6 +45,7 @@ def _ptr(t):
 class RWKV:
     def __init__(self, model, strategy, verbose=True, convert_and_save_and_exit=None):
         prxxx = (lambda *a, **k: print(*a, **k)) if verbose else (lambda *a, **k: None)
+        self._stream_order = _lib.StreamOrder()
         self.args = types.SimpleNamespace()
         args = self.args
         args.strategy_string = _strategy.normalize(strategy)          # ValueError on a bad string
@@ -576,11 +577,11 @@ class RWKV:
 
     def forward(self, tokens, state, full_output=False):
         """model.py:1443-1677.  Returns (logits fp32 [vocab] or [T, vocab], state)."""
-        cur = _lib.stream_order.before()
+        cur = self._stream_order.before()
         try:
             return self._forward(tokens, state, full_output)
         finally:
-            _lib.stream_order.after(cur)
+            self._stream_order.after(cur)
 
     def _forward(self, tokens, state, full_output):
         with torch.no_grad():

@@ -32,6 +32,7 @@ def _pad64(n):
 
 class RWKV_x070:
     def __init__(self, model, strategy):
+        self._stream_order = _lib.StreamOrder()
         self.args = types.SimpleNamespace()
         args = self.args
         ss = strategy.strip().split(' ')                              # model.py:234-243
@@ -250,11 +251,11 @@ class RWKV_x070:
 
     def forward(self, idx, state, full_output=False):
         """model.py:292-302."""
-        cur = _lib.stream_order.before()
+        cur = self._stream_order.before()
         try:
             return self._forward(idx, state, full_output)
         finally:
-            _lib.stream_order.after(cur)
+            self._stream_order.after(cur)
 
     def _forward(self, idx, state, full_output):
         with torch.no_grad():
