@@ -154,6 +154,24 @@ def cpu_baseline(shape, budget_s=25.0):
     }
 
 
+SPINUP_S = 1.0
+
+
+def spin_up(fn, seconds, sync_every=1):
+    """Runs fn() untimed for `seconds` (host clock), synchronising every `sync_every` calls so that the host does
+    not run ahead of the device; returns with the device idle for no longer than that last synchronisation."""
+    import torch
+    t0 = time.perf_counter()
+    i = 0
+    while time.perf_counter() - t0 < seconds:
+        fn()
+        i += 1
+        if i % sync_every == 0:
+            torch.cuda.synchronize()
+    torch.cuda.synchronize()
+    return i
+
+
 def gemm_roofline(T, N, M, u8, reps=10):
     """The prefill contraction alone on the model's largest matrix shape (channel-mix key, [T, N] x [N, M]),
     through the C ABI (rwkv_mm8_seq_f16 incl. its activation-scaling pass, or rwkv_gemm_f16), timed with two
@@ -188,8 +206,8 @@ def gemm_roofline(T, N, M, u8, reps=10):
         name = "gemm_dma_kernel<fp16 weights> (direct-to-LDS loads; 256x256 or 128x128 tile by the launch cost model)"
     for _ in range(3):
         run()
+    spin_up(run, min(SPINUP_S, 0.5), sync_every=32)
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    torch.cuda.synchronize()
     e0.record()
     for _ in range(reps):
         run()
@@ -239,8 +257,13 @@ def isolated_mm8(reps=40):
         for name, fn, n in (("mm8_one", one, reps), ("mm8_seq", seq, max(4, reps // 4))):
             for i in range(3):
                 fn(i)
+            k = [0]
+
+            def warm():
+                k[0] += 1
+                fn(k[0])
+            spin_up(warm, min(SPINUP_S, 0.3), sync_every=64)
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            torch.cuda.synchronize()
             e0.record()
             for i in range(n):
                 fn(i)
@@ -261,6 +284,10 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=256)
     ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--spinup", type=float, default=1.0,
+                    help="seconds of the same work run untimed right before every timed region, on top of --warmup: "
+                         "the shader clock takes tens of milliseconds of continuous load to rise from its idle level "
+                         "(1.4 GHz in a cold 4 ms burst, 1.8 GHz sustained, measured with the cycle counter)")
     ap.add_argument("--shape", default="v4-7b")
     ap.add_argument("--strategy", default="cuda fp16i8")
     ap.add_argument("--prefill", type=int, default=1024)
@@ -310,25 +337,31 @@ def main():
             out, state = model.forward(ptoks[i:i + chunk], state)
         return out, state
 
+    global SPINUP_S
+    SPINUP_S = args.spinup
     prefill()
-    torch.cuda.synchronize()
-    pt = []
-    for _ in range(3):
+    spin_up(prefill, args.spinup)
+    pt, evs = [], []
+    for _ in range(3):      # queued back to back: no idle gap between the calls
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
         out, state = prefill()
         e1.record()
-        torch.cuda.synchronize()
-        pt.append(e0.elapsed_time(e1) * 1e-3)
+        evs.append((e0, e1))
+    torch.cuda.synchronize()
+    pt = [e0.elapsed_time(e1) * 1e-3 for e0, e1 in evs]
     t_prefill = float(np.median(pt))
     prefill_flops = 2.0 * args.prefill * (wbytes / (1 if u8 else 2) - C * V) + 2.0 * C * V
 
     # ---- decode: W warm-up + K timed greedy steps, token stays on the device
     tok = out.argmax().reshape(1).to(torch.int32)
-    for _ in range(args.warmup):
+    def one_step():
+        nonlocal out, state, tok
         out, state = model.forward(tok, state)
         tok = out.argmax().reshape(1).to(torch.int32)
-    torch.cuda.synchronize()
+    for _ in range(args.warmup):
+        one_step()
+    n_spin = spin_up(one_step, args.spinup, sync_every=64)
     t0 = time.perf_counter()
     for _ in range(args.steps):
         out, state = model.forward(tok, state)
@@ -386,6 +419,7 @@ def main():
         "metric": "7B fp16i8 decode tok/s (% HBM peak) + prefill tok/s, 1 MI355X" if args.shape == "v4-7b" and u8 else
                   f"{args.shape} '{args.strategy}' decode tok/s (% HBM peak) + prefill tok/s, 1 MI355X",
         "value": tok_s, "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "spinup_s": args.spinup, "spinup_steps": n_spin,
         "ms_per_step": 1e3 * t_dev / args.steps, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "u8 weights, fp16 activations, fp32 accumulate" if u8 else "fp16",
         "data": "synthetic (random-init weights, random tokens)",
