@@ -293,6 +293,31 @@ def test_v56_forward_parity(ver, tag, strat):
     assert torch.equal(r_out, g_out)
 
 
+@pytest.mark.parametrize("ver", [4, 5.2, 6])
+@pytest.mark.parametrize("strat", ["cuda fp16i8", "cuda fp16"])
+def test_short_call_lengths(ver, strat):
+    """Calls of 2, 3, 9 and 16 tokens (a ragged last prompt chunk, rwkv/utils.py:98-101): every product of such a
+    call goes through the 2..16-row streaming kernel.  Each call against the oracle fed the same chunks, the final
+    state too, and the last logits against one 30-token call (the tile kernels)."""
+    cfg = dict(n_layer=2, n_embd=256, n_ffn=1024, vocab=211)      # K ranges of 4 and 16 chunks per wave, odd width head
+    ck = synth.make_checkpoint(version=ver, seed=41 + int(ver * 10), affine=True, **cfg)
+    m = _rwkv()(ck, strat, verbose=False)
+    o = OracleRWKV(ck, strat)
+    toks = synth.random_tokens(30, cfg["vocab"], seed=43)
+    s, so, out = None, None, None
+    for a, b in ((0, 2), (2, 5), (5, 14), (14, 30)):
+        out, s = m.forward(toks[a:b], s)
+        oout, so = o.forward(toks[a:b], so)
+        d = float(np.abs(_np(out) - oout).max())
+        assert d <= LOGIT_TOL, (a, b, d)
+    for i, (x, y) in enumerate(zip(s, so)):
+        np.testing.assert_allclose(_np(x), y.astype(np.float32), rtol=2e-2, atol=2e-2, err_msg=f"state {i}")
+    whole, sw = m.forward(toks, None)
+    assert float((whole - out).abs().max()) <= LOGIT_TOL
+    for i, (x, y) in enumerate(zip(s, sw)):
+        np.testing.assert_allclose(_np(x), _np(y), rtol=2e-2, atol=2e-2, err_msg=f"state {i} vs one call")
+
+
 @pytest.mark.parametrize("ver,tag", V56)
 @pytest.mark.parametrize("strat", ["cuda fp16i8", "cuda fp16"])
 def test_v56_long_prompt(ver, tag, strat):

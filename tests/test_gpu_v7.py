@@ -207,6 +207,24 @@ def test_v7_long_prompt_and_odd_lora_ranks():
         assert np.abs(_np(s) - ref.astype(np.float32)).max() <= 1e-2 * scale, i
 
 
+def test_v7_short_call_lengths():
+    """Calls of 2, 3, 9 and 16 tokens: every product of such a call goes through the 2..16-row streaming kernel
+    (fp16 weights, LoRA products of odd ranks included)."""
+    cfg = dict(n_layer=2, n_embd=256, n_ffn=1024, vocab=300, lora=(32, 96, 32, 160))
+    ck = synth.make_checkpoint_v7(seed=73, **cfg)
+    m, o = _x070()(ck, "cuda fp16"), OracleRWKV7(ck, "cuda fp16", kernel_form=True)
+    toks = synth.random_tokens(30, cfg["vocab"], seed=12)
+    st, ost = None, None
+    for a, b in ((0, 2), (2, 5), (5, 14), (14, 30)):
+        out, st = m.forward(toks[a:b], st)
+        oo, ost = o.forward(toks[a:b], ost)
+        d = float(np.abs(_np(out) - oo.astype(np.float32)).max())
+        assert d <= LOGIT_TOL, (a, b, d)
+    for i, (s, ref) in enumerate(zip(st, ost)):
+        scale = max(float(np.abs(ref.astype(np.float32)).max()), 1.0)
+        assert np.abs(_np(s) - ref.astype(np.float32)).max() <= 1e-2 * scale, i
+
+
 def test_v7_side_stream_path(tiny7):
     """A call of 256 tokens or more runs the independent products of a layer on three streams; its logits and
     states must match the oracle and the same prompt fed in shorter calls (which stay on one stream)."""
