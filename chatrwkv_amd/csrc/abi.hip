@@ -1,3 +1,3 @@
 #include "common.h"
 
-extern "C" int rwkv_abi_version(void) { return 2; }
+extern "C" int rwkv_abi_version(void) { return 3; }

@@ -428,9 +428,80 @@ __global__ __launch_bounds__(1024) void tmix7_kernel(Tmix7Args a) {
             *(u32x4 *)(a.commit_dst + 8 * j8) = *(const u32x4 *)(a.commit_src + 8 * j8);
 }
 
+// ---- DeepEmbed channel mix (model.py:578-594): keys of token t scaled by ((xx_t @ s1) @ E_t) @ s2 + s0 -----------
+// First stage, one workgroup per token: sv = xx_t @ s1 (32 sums over C, eight per wave), then ss = sv @ E_t with
+// E_t = row token_t of the merged table viewed 32 x 32.  Both rounded to fp16 as the reference's fp16 tensors are.
+__global__ __launch_bounds__(256) void de_ss_kernel(int T, int C, int vocab, const int32_t *__restrict__ tokens,
+                                                    const rwkv_half *__restrict__ xx, const rwkv_half *__restrict__ s1,
+                                                    const rwkv_half *__restrict__ emb, rwkv_half *__restrict__ ss) {
+    __shared__ float sv[32];
+    const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const rwkv_half *x = xx + (size_t)t * C;
+    float acc[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[j] = 0.f;
+    for (int c8 = lane; c8 < (C >> 3); c8 += 64) {
+        const h16x8 xv = *(const h16x8 *)(x + 8 * c8);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const h16x8 wv = *(const h16x8 *)(s1 + (size_t)(wave * 8 + j) * C + 8 * c8);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) acc[j] += (float)xv[e] * (float)wv[e];
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const float v = wave_sum(acc[j]);
+        if (lane == 0) sv[wave * 8 + j] = (float)(h16)v;
+    }
+    __syncthreads();
+    if (threadIdx.x < 32) {
+        const rwkv_half *E = emb + (size_t)min(max(tokens[t], 0), vocab - 1) * 1024;
+        float a = 0.f;
+        for (int i = 0; i < 32; ++i) a += sv[i] * (float)h2f(E[i * 32 + threadIdx.x]);
+        ss[(size_t)t * 32 + threadIdx.x] = f2h(a);
+    }
+}
+
+// Second stage: k[t][f] *= (ss_t @ s2)[f] + s0[f], every step rounded to fp16.  A workgroup takes 256 columns of
+// eight tokens, so a column of s2 is fetched once per eight tokens.
+__global__ __launch_bounds__(256) void de_gate_kernel(int T, int F, const rwkv_half *__restrict__ ss,
+                                                      const rwkv_half *__restrict__ s2, const rwkv_half *__restrict__ s0,
+                                                      rwkv_half *__restrict__ k) {
+    __shared__ float ssl[8][32];
+    const int t0 = blockIdx.x * 8, f = blockIdx.y * 256 + threadIdx.x;
+    {
+        const int tt = threadIdx.x >> 5, j = threadIdx.x & 31;
+        ssl[tt][j] = t0 + tt < T ? h2f(ss[(size_t)(t0 + tt) * 32 + j]) : 0.f;
+    }
+    __syncthreads();
+    if (f >= F) return;
+    float col[32];
+#pragma unroll
+    for (int j = 0; j < 32; ++j) col[j] = h2f(s2[(size_t)j * F + f]);
+    const float b = h2f(s0[f]);
+    for (int tt = 0; tt < 8 && t0 + tt < T; ++tt) {
+        float a = 0.f;
+#pragma unroll
+        for (int j = 0; j < 32; ++j) a += ssl[tt][j] * col[j];
+        const float g = (float)(h16)((float)(h16)a + b);
+        rwkv_half *kp = k + (size_t)(t0 + tt) * F + f;
+        *kp = f2h(h2f(*kp) * g);
+    }
+}
+
+int de_gate_launch(const rwkv_v7_layer &l, int64_t T, int C, int F, int vocab, const int32_t *tokens, const rwkv_half *xx,
+                   rwkv_half *ss, rwkv_half *k, hipStream_t st) {
+    hipLaunchKernelGGL(de_ss_kernel, dim3((unsigned)T), dim3(256), 0, st, (int)T, C, vocab, tokens, xx, l.de_s1, l.de_emb, ss);
+    hipLaunchKernelGGL(de_gate_kernel, dim3((unsigned)((T + 7) / 8), (unsigned)((F + 255) / 256)), dim3(256), 0, st, (int)T, F,
+                       ss, l.de_s2, l.de_s0, k);
+    RWKV_LAUNCH_CHECK();
+    return RWKV_OK;
+}
+
 struct Ws7 {
     rwkv_half *x, *mix[6], *l1, *lw, *la, *lv, *lg, *w_raw, *a_raw, *vg_raw, *g, *r, *k, *v, *v_first, *an, *b, *att, *vx,
-        *xx_att, *xx_ffn;
+        *xx_att, *xx_ffn, *de_ss;
     float *dec, *rk, *y32, *splitk;
     size_t total;
 };
@@ -451,6 +522,7 @@ Ws7 carve7(void *base, int64_t T, const rwkv_v7_model *m) {
     w.att = take(tc);
     w.vx = take((size_t)T * F * 2);
     w.xx_att = take(C * 2); w.xx_ffn = take(C * 2);
+    w.de_ss = take((size_t)T * 32 * 2);
     w.dec = (float *)take((size_t)T * C * 4);
     w.rk = (float *)take((size_t)T * m->n_head * 4);
     w.y32 = (float *)take((size_t)T * C * 4);
@@ -504,6 +576,10 @@ static int v7_check(const rwkv_v7_model *m) {
             return RWKV_E_NULL;
         if (i > 0 && !l.v0) return RWKV_E_NULL;
         if (!aligned16(l.lora1) || !aligned16(l.lora2)) return RWKV_E_LAYOUT;
+        if (l.de_emb || l.de_s1 || l.de_s2 || l.de_s0) {   // the DeepEmbed tensors come all four or not at all
+            if (!l.de_emb || !l.de_s1 || !l.de_s2 || !l.de_s0) return RWKV_E_NULL;
+            if (!aligned16(l.de_s1)) return RWKV_E_LAYOUT;
+        }
         for (int j = 0; j < 6; ++j)
             if (!l.x_mix[j]) return RWKV_E_NULL;
         if (!mat_ok7(l.att_receptance, C, C) || !mat_ok7(l.att_key, C, C) || !mat_ok7(l.att_value, C, C) ||
@@ -586,6 +662,7 @@ extern "C" int rwkv_v7_forward(const rwkv_v7_model *m, const rwkv_v56_layer_stat
                 a.out[0] = ws.vx; a.maa_form = 1;
                 lnmix1_launch(false, a, c.grid, st);
             }
+            if (l.de_emb && (rc = de_gate_launch(l, 1, C, m->n_ffn, m->vocab, tokens, ws.xx_ffn, ws.de_ss, ws.vx, st))) return rc;
             if ((rc = mm(c, l.ffn_value, false, ws.vx, ACT_RESIDUAL, ws.x, nullptr, 1.f, ws.x, ws.xx_ffn, s.ffn_xx, C))) return rc;
             RWKV_LAUNCH_CHECK();
             continue;
@@ -653,9 +730,11 @@ extern "C" int rwkv_v7_forward(const rwkv_v7_model *m, const rwkv_v56_layer_stat
             a.T = (int)T; a.C = C; a.x = ws.x; a.ln_w = l.ln2_w; a.ln_b = l.ln2_b; a.sx = s.ffn_xx;
             a.xx_last = nullptr; a.state_out = s.ffn_xx; a.maa_form = 1;
             a.mix[0] = l.ffn_x_k; a.xs[0] = ws.mix[0];
-            if ((rc = lnmix_seq_launch(a, 1, st))) return rc;
+            a.mix[1] = nullptr; a.xs[1] = ws.mix[1];   // DeepEmbed also reads the LayerNorm output itself
+            if ((rc = lnmix_seq_launch(a, l.de_emb ? 2 : 1, st))) return rc;
         }
         if ((rc = mm(c, l.ffn_key, false, ws.mix[0], ACT_RELU_SQ, nullptr, nullptr, 1.f, ws.vx))) return rc;
+        if (l.de_emb && (rc = de_gate_launch(l, T, C, m->n_ffn, m->vocab, tokens, ws.mix[1], ws.de_ss, ws.vx, st))) return rc;
         if ((rc = mm(c, l.ffn_value, false, ws.vx, ACT_RESIDUAL, ws.x, nullptr, 1.f, ws.x))) return rc;
         RWKV_LAUNCH_CHECK();
     }

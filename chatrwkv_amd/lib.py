@@ -101,7 +101,8 @@ class RwkvV7Layer(ctypes.Structure):
                 ("lora1", _vp), ("lora2", _vp),
                 ("k_k", _vp), ("k_a", _vp), ("r_k", _vp), ("lnx_w", _vp), ("lnx_b", _vp),
                 ("att_receptance", RwkvMat), ("att_key", RwkvMat), ("att_value", RwkvMat), ("att_output", RwkvMat),
-                ("ffn_x_k", _vp), ("ffn_key", RwkvMat), ("ffn_value", RwkvMat)]
+                ("ffn_x_k", _vp), ("ffn_key", RwkvMat), ("ffn_value", RwkvMat),
+                ("de_emb", _vp), ("de_s1", _vp), ("de_s2", _vp), ("de_s0", _vp)]
 
 
 class RwkvV7Model(ctypes.Structure):

@@ -10,7 +10,9 @@ fp16 [C]; model.py:284-290), ``idx`` an int, a one-element list (one-token mode)
 
 Differences a caller can observe: state tensors are updated in place; ``model`` may also be an
 in-memory ``{name: tensor}`` dict; a one-element integer tensor on the GPU is accepted as ``idx``.
-The DeepEmbed variant (RWKV_DE_VERSION=1) and the fp32 / bf16 strategies are not implemented.
+The DeepEmbed variant is selected as in the reference, by RWKV_DE_VERSION=1 in the environment when the object is
+built (model.py:274-277, 578-594); the checkpoint must then carry the ffn.s_* tensors.  The fp32 / bf16 strategies
+are not implemented.
 """
 import collections
 import ctypes
@@ -40,8 +42,7 @@ class RWKV_x070:
             raise AssertionError("currently rwkv7 strategy must be: cuda/cpu fp16/fp32/bf16")
         if not ss[0].startswith('cuda') or ss[0] not in ('cuda', 'cuda:0') or ss[1] != 'fp16':
             raise NotImplementedError("chatrwkv_amd runs RWKV-7 under 'cuda fp16' only")
-        if os.environ.get('RWKV_DE_VERSION') == '1':
-            raise NotImplementedError("the DeepEmbed variant of RWKV-7 is not implemented")
+        self.deep_embed = os.environ.get('RWKV_DE_VERSION') == '1'     # model.py:274, 304
         if isinstance(model, dict):
             args.MODEL_NAME = '<dict>'
             w = dict(model)
@@ -87,11 +88,32 @@ class RWKV_x070:
             torch.cuda.synchronize()
             z['emb.weight'] = emb16
             del emb32
+            if self.deep_embed:
+                self._merge_deep_embed()
             self._build_descriptors()
         self._graphs = collections.OrderedDict()
         self._seq_ws = None
         gc.collect()
         torch.cuda.empty_cache()
+
+    def _merge_deep_embed(self):
+        """model.py:274-277: ffn.s_emb += emb @ ffn.s_emb_x^T per layer (emb already carries ln0), the product
+        through the library's fp16 GEMM (fp32 accumulation, rounded to fp16, then the fp16 add)."""
+        z, a, L = self.z, self.args, _lib.load()
+        st = torch.cuda.current_stream().cuda_stream
+        V, C = z['emb.weight'].shape
+        for i in range(a.n_layer):
+            ff = f'blocks.{i}.ffn.'
+            sx = z[ff + 's_emb_x.weight']                              # [1024, C] row-major = [C][1024] input-contiguous
+            if tuple(z[ff + 's_emb.weight'].shape) != (V, 1024) or tuple(sx.shape) != (1024, C):
+                raise ValueError("DeepEmbed tensors must be ffn.s_emb.weight [vocab, 1024] and ffn.s_emb_x.weight [1024, n_embd]")
+            prod = torch.empty((V, 1024), dtype=torch.float16, device=self.device)
+            _lib.check(L.rwkv_gemm_f16(V, C, 1024, z['emb.weight'].data_ptr(), C, sx.data_ptr(), 1, C,
+                                       prod.data_ptr(), 1024, _lib.RWKV_DT_F16, st), "rwkv_gemm_f16")
+            z[ff + 's_emb.weight'] = (z[ff + 's_emb.weight'] + prod).contiguous()
+            z[ff + 's1t'] = z[ff + 's1'].t().contiguous()               # [32][C]
+            del z[ff + 's_emb_x.weight']
+        torch.cuda.synchronize()
 
     # ------------------------------------------------------------------ descriptors
     def _mat(self, name):
@@ -141,6 +163,12 @@ class RWKV_x070:
             l.att_value, l.att_output = self._mat(at + 'value.weight'), self._mat(at + 'output.weight')
             l.ffn_x_k = z[ff + 'x_k'].data_ptr()
             l.ffn_key, l.ffn_value = self._mat(ff + 'key.weight'), self._mat(ff + 'value.weight')
+            if self.deep_embed:
+                if tuple(z[ff + 's1t'].shape) != (32, C) or tuple(z[ff + 's2'].shape) != (32, a.n_ffn) or \
+                        z[ff + 's0'].numel() != a.n_ffn:
+                    raise ValueError("DeepEmbed tensors must be ffn.s1 [n_embd, 32], ffn.s2 [32, n_ffn], ffn.s0 [n_ffn]")
+                l.de_emb, l.de_s1 = z[ff + 's_emb.weight'].data_ptr(), z[ff + 's1t'].data_ptr()
+                l.de_s2, l.de_s0 = z[ff + 's2'].data_ptr(), z[ff + 's0'].data_ptr()
         m = _lib.RwkvV7Model()
         m.n_layer, m.n_embd, m.n_ffn, m.vocab, m.n_head = a.n_layer, C, a.n_ffn, a.vocab_size, self.n_head
         m.lora_w, m.lora_a, m.lora_v, m.lora_g = ranks

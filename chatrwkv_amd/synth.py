@@ -163,12 +163,16 @@ def v7_lora_dims(n_embd):
     return r32(1.8 * c ** 0.5), r32(1.8 * c ** 0.5), r32(1.3 * c ** 0.5), r32(0.6 * c ** 0.8)
 
 
-def make_checkpoint_v7(n_layer=2, n_embd=128, n_ffn=None, vocab=97, seed=0, head_size=64, lora=None, device=None):
+def make_checkpoint_v7(n_layer=2, n_embd=128, n_ffn=None, vocab=97, seed=0, head_size=64, lora=None, device=None,
+                       deep_embed=False):
     """RWKV-7 checkpoint with the keys ``RWKV_x070.__init__`` reads (model.py:245-282) and the forward
     passes use (model.py:349-358): per block ``att.x_{r,w,k,v,a,g}``, ``att.{w,a,v}{0,1,2}``,
     ``att.g{1,2}``, ``att.k_k``, ``att.k_a``, ``att.r_k`` [H, N], the four square matrices, ``att.ln_x``,
     ``ffn.x_k`` and the two channel-mix matrices.  LoRA matrices are stored [in, rank] / [rank, out]
-    and are not transposed by the loader.  ``lora`` = (decay, a, v, gate) ranks."""
+    and are not transposed by the loader.  ``lora`` = (decay, a, v, gate) ranks.
+    ``deep_embed``: also the tensors of the DeepEmbed variant (RWKV_DE_VERSION=1, model.py:274-277, 578-594): per
+    block ``ffn.s_emb.weight`` [V, 1024], ``ffn.s_emb_x.weight`` [1024, C], ``ffn.s1`` [C, 32], ``ffn.s2``
+    [32, F] and ``ffn.s0`` [1, 1, F]."""
     C = int(n_embd)
     F = int(n_ffn) if n_ffn is not None else 4 * C
     V = int(vocab)
@@ -208,6 +212,12 @@ def make_checkpoint_v7(n_layer=2, n_embd=128, n_ffn=None, vocab=97, seed=0, head
         w[f + "x_k"] = g.uniform(f + "x_k", (1, 1, C), 0.0, 1.0)
         w[f + "key.weight"] = g.normal(f + "key.weight", (F, C), 0.05)
         w[f + "value.weight"] = g.normal(f + "value.weight", (C, F), 0.05)
+        if deep_embed:
+            w[f + "s_emb.weight"] = g.normal(f + "s_emb.weight", (V, 1024), 0.3)
+            w[f + "s_emb_x.weight"] = g.normal(f + "s_emb_x.weight", (1024, C), 0.03)
+            w[f + "s1"] = g.normal(f + "s1", (C, 32), 0.1)
+            w[f + "s2"] = g.normal(f + "s2", (32, F), 0.2)
+            w[f + "s0"] = g.uniform(f + "s0", (1, 1, F), 0.5, 1.5)
     w["ln_out.weight"] = g.uniform("ln_out.weight", (C,), 0.8, 1.2)
     w["ln_out.bias"] = g.normal("ln_out.bias", (C,), 0.05)
     w["head.weight"] = g.normal("head.weight", (V, C), 0.05)

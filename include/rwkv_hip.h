@@ -44,7 +44,7 @@ typedef uint16_t rwkv_half;
 #define RWKV_DT_F16 0
 #define RWKV_DT_F32 1
 
-/* Library / device identification.  Returns the ABI version (currently 2). */
+/* Library / device identification.  Returns the ABI version (currently 3). */
 int rwkv_abi_version(void);
 
 /* ---------------------------------------------------------------------------------------
@@ -293,7 +293,8 @@ int rwkv_wkv7_forward(int64_t B, int64_t T, int64_t C, int64_t H, float *state, 
 /* =======================================================================================
  * RWKV-7 ("x070"): one entry point for both modes of RWKV_x070.forward (model.py:292-302), replacing
  * forward_one / forward_seq (model.py:336-363, 457-487), RWKV_x070_TMix_one / _seq (model.py:492-572),
- * RWKV_x070_CMix_one / _seq (model.py:597-608) and RWKV7_OP (model.py:198-219).  The reference runs RWKV-7
+ * RWKV_x070_CMix_one / _seq (model.py:597-608; the DeepEmbed forms model.py:578-594 when a layer carries the de_*
+ * tensors) and RWKV7_OP (model.py:198-219).  The reference runs RWKV-7
  * in fp16, bf16 or fp32 without quantisation (model.py:236-243); this entry point is the fp16 one.  Head
  * size must be 64.  The four LoRA pairs (decay w, in-context rate a, value residual v, gate g) are fp16
  * and input-contiguous like the model matrices, every rank padded with zeros to a multiple of 64 and the
@@ -312,6 +313,14 @@ typedef struct {
     rwkv_mat att_receptance, att_key, att_value, att_output;
     const rwkv_half *ffn_x_k;                             /* [C] */
     rwkv_mat ffn_key, ffn_value;
+    /* DeepEmbed variant (RWKV_DE_VERSION=1: model.py:274-277, 578-594); all four NULL = the plain channel mix.
+     * The squared-relu keys of token t are scaled by ((xx_t @ s1) @ E_t) @ s2 + s0, xx_t the LayerNorm output,
+     * E_t = row token_t of de_emb viewed 32 x 32.
+     *   de_emb [vocab][1024]  ffn.s_emb.weight with the embedding residual merged in (model.py:276-277)
+     *   de_s1  [32][C]        ffn.s1 ([C, 32]) transposed, input-contiguous like the model matrices
+     *   de_s2  [32][F]        ffn.s2 as stored
+     *   de_s0  [F]            ffn.s0 */
+    const rwkv_half *de_emb, *de_s1, *de_s2, *de_s0;
 } rwkv_v7_layer;
 
 typedef struct {

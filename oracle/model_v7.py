@@ -5,8 +5,9 @@ Test infrastructure only (see oracle/__init__.py).
 ``OracleRWKV7(checkpoint, strategy)`` restates ``RWKV_x070.__init__`` (model.py:224-282),
 ``forward_one`` / ``forward_seq`` (model.py:336-363, 457-487), the time mix
 ``RWKV_x070_TMix_one`` / ``_seq`` (model.py:492-572) and the channel mix
-``RWKV_x070_CMix_one`` / ``_seq`` (model.py:597-608).  The DeepEmbed variants
-(``RWKV_DE_VERSION=1``) are not covered.
+``RWKV_x070_CMix_one`` / ``_seq`` (model.py:597-608), and with ``deep_embed=True`` the DeepEmbed variant the
+reference selects with ``RWKV_DE_VERSION=1``: the merge of the embedding residual into ``ffn.s_emb``
+(model.py:274-277) and the gated channel mix (model.py:578-594).
 
 Strategies: '<device> fp32' runs every operation in fp32; '<device> fp16' keeps activations and
 weights in numpy float16, which rounds after every elementwise operation as torch does on fp16
@@ -95,7 +96,7 @@ def wkv7_kernel(S, r, w_log, k, v, a, b):
 
 
 class OracleRWKV7:
-    def __init__(self, checkpoint, strategy, kernel_form=False):
+    def __init__(self, checkpoint, strategy, kernel_form=False, deep_embed=False):
         dev, dt = strategy.split(' ')                                 # model.py:234-243
         if dt not in ('fp16', 'fp32'):
             raise ValueError("oracle supports '<device> fp16' and '<device> fp32' for RWKV-7")
@@ -117,6 +118,11 @@ class OracleRWKV7:
             z[k] = np.ascontiguousarray(t).astype(A)
         # model.py:272: the embedding absorbs ln0, computed on the already-converted table
         z['emb.weight'] = ops.layer_norm(z['emb.weight'], z['blocks.0.ln0.weight'], z['blocks.0.ln0.bias'])
+        self.deep_embed = bool(deep_embed)
+        if self.deep_embed:                                            # model.py:274-277
+            for i in range(self.n_layer):
+                p = f'blocks.{i}.ffn.'
+                z[p + 's_emb.weight'] = z[p + 's_emb.weight'] + _mm(z['emb.weight'], z[p + 's_emb_x.weight'].T)
         self.z = z
 
     def generate_zero_state(self):
@@ -163,12 +169,19 @@ class OracleRWKV7:
         y = y + (rk * v.reshape(T, H, -1)).reshape(T, C)
         return _mm(y * g, z[p + 'output.weight']), x[-1], S, v_first
 
-    def _cmix(self, i, x, x_prev):
-        """model.py:597-608."""
+    def _cmix(self, i, x, x_prev, toks=None):
+        """model.py:597-608; with DeepEmbed model.py:578-594: the squared-relu keys of token t are scaled by
+        ((x_t @ s1) @ E_t) @ s2 + s0, E_t the 32 x 32 matrix stored in row token_t of ffn.s_emb."""
         z, p = self.z, f'blocks.{i}.ffn.'
         xx = np.concatenate([x_prev[None, :], x[:-1]], axis=0) - x
         k = x + xx * z[p + 'x_k']
         k = ops.relu_sq(_mm(k, z[p + 'key.weight']))
+        if self.deep_embed:
+            T = x.shape[0]
+            E = z[p + 's_emb.weight'][np.asarray(toks, dtype=np.int64)].reshape(T, 32, 32)
+            sv = _mm(x, z[p + 's1'])                                                     # [T, 32]
+            ss = np.einsum('ti,tij->tj', sv.astype(f32), E.astype(f32)).astype(x.dtype)  # [T, 32]
+            k = k * (_mm(ss, z[p + 's2']) + z[p + 's0'])
         return _mm(k, z[p + 'value.weight']), x[-1]
 
     # ------------------------------------------------------------------ forward
@@ -188,7 +201,7 @@ class OracleRWKV7:
                                                                     state[3 * i + 1], not one)
             x = x + xx
             xx = ops.layer_norm(x, z[b + 'ln2.weight'], z[b + 'ln2.bias'])
-            xx, state[3 * i + 2] = self._cmix(i, xx, state[3 * i + 2])
+            xx, state[3 * i + 2] = self._cmix(i, xx, state[3 * i + 2], toks)
             x = x + xx
         if one or not full_output:
             x = x[-1:]

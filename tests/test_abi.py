@@ -37,7 +37,7 @@ def test_header_symbols_exported_and_bound():
         assert n in lib.SIGNATURES, f"{n} has no ctypes signature in chatrwkv_amd/lib.py"
     for n in lib.SIGNATURES:
         assert n in names, f"{n} bound in lib.py but not declared in the header"
-    assert L.rwkv_abi_version() == 2
+    assert L.rwkv_abi_version() == 3
 
 
 def test_argument_validation_without_gpu():

@@ -225,6 +225,49 @@ def test_v7_short_call_lengths():
         assert np.abs(_np(s) - ref.astype(np.float32)).max() <= 1e-2 * scale, i
 
 
+def test_v7_deep_embed(monkeypatch):
+    """The DeepEmbed variant (RWKV_DE_VERSION=1, model.py:274-277, 578-594): merged embedding table, gated channel
+    mix in sequence and one-token calls (graph replay included), against the oracle and the reference's own
+    'cpu fp16' run of the same checkpoint; a wider model in calls of 70, 9 and 1 tokens against the oracle."""
+    monkeypatch.setenv("RWKV_DE_VERSION", "1")
+    ck = synth.make_checkpoint_v7(seed=CKPT_SEED + 1, deep_embed=True, **TINY7)
+    m, o = _x070()(ck, "cuda fp16"), OracleRWKV7(ck, "cuda fp16", deep_embed=True)
+    assert m.deep_embed
+    g = dict(np.load(os.path.join(G, "e2e_v7_de_cpu_fp16.npz")))
+    toks = [int(t) for t in g["tokens"]]
+    full, st = m.forward(toks, None, full_output=True)
+    ofull, ost = o.forward(toks, None, full_output=True)
+    d = float(np.abs(_np(full) - ofull.astype(np.float32)).max())
+    assert d <= LOGIT_TOL, d
+    assert float(np.abs(_np(full) - g["full_logits"]).max()) <= LOGIT_TOL
+    for i, (s, ref) in enumerate(zip(st, ost)):
+        scale = max(float(np.abs(ref.astype(np.float32)).max()), 1.0)
+        assert np.abs(_np(s) - ref.astype(np.float32)).max() <= 1e-2 * scale, i
+        assert np.abs(_np(s) - g[f"full_state_{i}"]).max() <= 1e-2 * scale, i
+    st, ost = None, None
+    for j, (a, b) in enumerate(CHUNKS):
+        out, st = m.forward(toks[a:b] if b - a > 1 else toks[a], st)
+        oo, ost = o.forward(toks[a:b], ost)
+        assert float(np.abs(_np(out) - oo.astype(np.float32)).max()) <= LOGIT_TOL, j
+        assert float(np.abs(_np(out) - g["chunk_logits"][j]).max()) <= LOGIT_TOL, j
+    # the plain model on the same checkpoint gives other logits: the gate is in the path
+    monkeypatch.delenv("RWKV_DE_VERSION")
+    plain = _x070()(ck, "cuda fp16")
+    pfull, _ = plain.forward(toks, None, full_output=True)
+    assert float((pfull.float() - full.float()).abs().max()) > 10 * LOGIT_TOL
+    monkeypatch.setenv("RWKV_DE_VERSION", "1")
+    cfg = dict(n_layer=2, n_embd=256, n_ffn=1024, vocab=300, lora=(32, 96, 32, 160))
+    ck = synth.make_checkpoint_v7(seed=75, deep_embed=True, **cfg)
+    m, o = _x070()(ck, "cuda fp16"), OracleRWKV7(ck, "cuda fp16", kernel_form=True, deep_embed=True)
+    toks = synth.random_tokens(84, cfg["vocab"], seed=13)
+    st, ost = None, None
+    for a, b in ((0, 70), (70, 79), (79, 80), (80, 81), (81, 84)):
+        out, st = m.forward(toks[a:b], st)
+        oo, ost = o.forward(toks[a:b], ost)
+        d = float(np.abs(_np(out) - oo.astype(np.float32)).max())
+        assert d <= LOGIT_TOL, (a, b, d)
+
+
 def test_v7_side_stream_path(tiny7):
     """A call of 256 tokens or more runs the independent products of a layer on three streams; its logits and
     states must match the oracle and the same prompt fed in shorter calls (which stay on one stream)."""

@@ -21,11 +21,13 @@ TOL = {"cpu fp32": 2e-5, "cpu fp16": 1.2e-2}
 
 @pytest.mark.parametrize("strat", ["cpu fp32", "cpu fp16"])
 @pytest.mark.parametrize("kernel_form", [False, True])
-def test_v7_forward_matches_reference(strat, kernel_form):
-    g = dict(np.load(os.path.join(G, f"e2e_v7_{strat.replace(' ', '_')}.npz")))
-    ck = synth.make_checkpoint_v7(seed=CKPT_SEED, **TINY7)
+@pytest.mark.parametrize("de", [False, True])
+def test_v7_forward_matches_reference(strat, kernel_form, de):
+    """de: the DeepEmbed variant (reference run with RWKV_DE_VERSION=1 on a checkpoint with the ffn.s_* tensors)."""
+    g = dict(np.load(os.path.join(G, f"e2e_v7_{'de_' if de else ''}{strat.replace(' ', '_')}.npz")))
+    ck = synth.make_checkpoint_v7(seed=CKPT_SEED + (1 if de else 0), deep_embed=de, **TINY7)
     toks = [int(t) for t in g["tokens"]]
-    m = OracleRWKV7(ck, strat, kernel_form=kernel_form)
+    m = OracleRWKV7(ck, strat, kernel_form=kernel_form, deep_embed=de)
     full, st = m.forward(toks, None, full_output=True)
     assert full.shape == g["full_logits"].shape
     assert np.abs(full.astype(np.float32) - g["full_logits"]).max() <= TOL[strat]
@@ -43,6 +45,21 @@ def test_v7_forward_matches_reference(strat, kernel_form):
     # chunked evaluation equals the one-shot evaluation at the chunk ends
     for j, (a, b) in enumerate(CHUNKS):
         assert np.abs(outs[j] - g["full_logits"][b - 1]).max() <= 4 * TOL[strat]
+
+
+def test_deep_embed_with_a_unit_gate_is_the_plain_model():
+    """s2 = 0 and s0 = 1 make the DeepEmbed gate 1 for every token: the logits must equal the plain model's."""
+    ck = synth.make_checkpoint_v7(seed=5, deep_embed=True, **TINY7)
+    for i in range(TINY7["n_layer"]):
+        ck[f"blocks.{i}.ffn.s2"] = np.zeros_like(ck[f"blocks.{i}.ffn.s2"])
+        ck[f"blocks.{i}.ffn.s0"] = np.ones_like(ck[f"blocks.{i}.ffn.s0"])
+    toks = synth.random_tokens(7, TINY7["vocab"], seed=6)
+    a, _ = OracleRWKV7(ck, "cpu fp32", deep_embed=True).forward(toks, None, full_output=True)
+    b, _ = OracleRWKV7(ck, "cpu fp32").forward(toks, None, full_output=True)
+    assert np.array_equal(a, b)
+    ck2 = synth.make_checkpoint_v7(seed=5, deep_embed=True, **TINY7)
+    c, _ = OracleRWKV7(ck2, "cpu fp32", deep_embed=True).forward(toks, None, full_output=True)
+    assert np.abs(c - b).max() > 0.1
 
 
 def _scalar_wkv7(S, r, w_log, k, v, a, b):
