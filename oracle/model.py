@@ -327,6 +327,10 @@ class OracleRWKV:
             kx, vx, rx = mix('time_mix_k'), mix('time_mix_v'), mix('time_mix_r')
             if gated:
                 gx = mix('time_mix_g')
+        # output_dtype fp32 (model.py:1283-1285, 1369-1371).  With fp16 weights the reference's native GEMM writes the
+        # fp32 sums unrounded (gemm_fp16_cublas.cpp:31-33) and so does this emulation; the reference's pure-torch
+        # 'cpu fp16' run (the goldens) and the HIP path round r, k, v to fp16 once before widening them: one extra
+        # fp16 rounding, inside the 2e-2 logit tolerance of the tests that compare the three.
         r = self._mm(rx, a + 'receptance.weight', output_dtype=f32).reshape(T, H, N)
         k = self._mm(kx, a + 'key.weight', output_dtype=f32).reshape(T, H, N)
         v = self._mm(vx, a + 'value.weight', output_dtype=f32).reshape(T, H, N)
