@@ -293,6 +293,40 @@ def test_v56_forward_parity(ver, tag, strat):
     assert torch.equal(r_out, g_out)
 
 
+@pytest.mark.parametrize("ver", [4, 6])
+def test_long_greedy_run_graph_equals_direct(ver):
+    """400 greedy steps after a 64-token prompt at n_embd 1024, once by HIP-graph replay with the token kept on the
+    device and once by direct launches with the token fetched every step: the same token sequence, bit-equal final
+    logits and states.  A race between replays, a stale graph argument or a lost state update shows here."""
+    cfg = dict(n_layer=4, n_embd=1024, n_ffn=4096, vocab=4099)
+    ck = synth.make_checkpoint(version=ver, seed=51 + int(ver), affine=True, **cfg)
+    m = _rwkv()(ck, "cuda fp16i8", verbose=False)
+    prompt = synth.random_tokens(64, cfg["vocab"], seed=52)
+
+    def run(graph):
+        os.environ["RWKV_HIP_GRAPH"] = "1" if graph else "0"
+        try:
+            out, st = m.forward(prompt, None)
+            seq = []
+            tok = out.argmax().reshape(1).to(torch.int32)
+            for _ in range(400):
+                out, st = m.forward(tok if graph else [int(tok)], st)
+                tok = out.argmax().reshape(1).to(torch.int32)
+                seq.append(tok)
+            torch.cuda.synchronize()
+            return torch.cat(seq).cpu(), out.clone(), [t.clone() for t in st]
+        finally:
+            os.environ["RWKV_HIP_GRAPH"] = "1"
+
+    seq_g, out_g, st_g = run(True)
+    seq_d, out_d, st_d = run(False)
+    assert torch.equal(seq_g, seq_d)
+    assert torch.equal(out_g, out_d)
+    for a, b in zip(st_g, st_d):
+        assert torch.equal(a, b)
+    assert len(set(seq_g.tolist())) > 3        # not a degenerate run
+
+
 @pytest.mark.parametrize("ver", [4, 5.2, 6])
 @pytest.mark.parametrize("strat", ["cuda fp16i8", "cuda fp16"])
 def test_short_call_lengths(ver, strat):
