@@ -38,10 +38,12 @@ HBM_PEAK = 8.0e12      # bytes/s, MI355X HBM3E
 # kernel: x2.0 / x1.0).  Counter figures, not read in this run: TRAFFIC_SOURCE has the commands and the table, and
 # every roofline object names it next to the number so that a stale value can be told from a fresh one.
 TRAFFIC_SOURCE = "profiles/decode_7b_fp16i8_hbm_traffic.md"
-MEASURED_TRAFFIC = {("v4-7b", "cuda fp16i8", 32, "ffn_rk"): 85082112 + 49254,
-                    ("v4-7b", "cuda fp16i8", 32, "att_kvr_wkv"): 52142694 + 65536,
-                    # the prefill contraction [1024 x 4096] x [4096 x 16384], uint8 weights, 256 x 256 tiles
-                    ("gemm", 1024, 4096, 16384, True): 134557082 + 33554432}
+# (bytes read, bytes written) per launch as that profile lists them
+TRAFFIC_READ_WRITTEN = {("v4-7b", "cuda fp16i8", 32, "ffn_rk"): (85082112, 49254),
+                        ("v4-7b", "cuda fp16i8", 32, "att_kvr_wkv"): (52142694, 65536),
+                        # the prefill contraction [1024 x 4096] x [4096 x 16384], uint8 weights, 256 x 256 tiles
+                        ("gemm", 1024, 4096, 16384, True): (134557082, 33554432)}
+MEASURED_TRAFFIC = {k: r + w for k, (r, w) in TRAFFIC_READ_WRITTEN.items()}
 MFMA_F16_PEAK = 2.5e15  # flop/s dense fp16
 
 
