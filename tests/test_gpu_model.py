@@ -622,9 +622,10 @@ def test_7b_shape_properties_v6_v7(kind):
 
 
 # ------------------------------------------------------------------------------ full width, statistics, initial state
-@pytest.mark.parametrize("shape,V", [("v4-7b", 50277), ("v4-14b", 5003)])
+@pytest.mark.parametrize("shape,V", [("v4-7b", 50277), ("v4-14b", 5003), ("v6-7b", 5003)])
 def test_full_width_oracle_parity(shape, V, capsys):
-    """Two layers of the 7B / 14B RWKV-4 shapes (the 14B one with a short vocabulary: its head is the same
+    """Two layers of the 7B / 14B RWKV-4 shapes and of the 7B RWKV-6 shape (n_embd 4096, n_ffn 14336, 64 heads, LoRA
+    ranks 32 / 64; the 14B and RWKV-6 ones with a short vocabulary: their head is the same
     kernel as the 7B one's) under 'cuda fp16i8' against the oracle on the same checkpoint: a sequence call of
     320 tokens (large and small MFMA tiles, K split, ragged last row tile, chunked WKV scan), then four
     one-token steps (streaming kernels at full width).  Logits within 2e-2 of the oracle's emulation, same
@@ -632,8 +633,8 @@ def test_full_width_oracle_parity(shape, V, capsys):
     def beat(msg):                                       # a line a minute: the oracle's conversion is slow
         with capsys.disabled():
             print(f"[full width {shape}] {msg}", flush=True)
-    _, _, C, F, _ = synth.SHAPES[shape]
-    ck = synth.make_checkpoint(version=4, n_layer=2, n_embd=C, n_ffn=F, vocab=V, seed=17, affine=True, device="cuda:0")
+    version, _, C, F, _ = synth.SHAPES[shape]
+    ck = synth.make_checkpoint(version=version, n_layer=2, n_embd=C, n_ffn=F, vocab=V, seed=17, affine=True, device="cuda:0")
     m = _rwkv()(ck, "cuda fp16i8", verbose=False)
     beat("model converted on the GPU")
     ck = {k: v.cpu() for k, v in ck.items()}
