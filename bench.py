@@ -174,7 +174,7 @@ def spin_up(fn, seconds, sync_every=1):
     return i
 
 
-def gemm_roofline(T, N, M, u8, reps=10):
+def gemm_roofline(T, N, M, u8, reps=20):
     """The prefill contraction alone on the model's largest matrix shape (channel-mix key, [T, N] x [N, M]),
     through the C ABI (rwkv_mm8_seq_f16 incl. its activation-scaling pass, or rwkv_gemm_f16), timed with two
     events on the stream it is launched on: algorithmic flops 2 T N M over the mean launch time against the
@@ -256,7 +256,7 @@ def isolated_mm8(reps=40):
             lib.check(L.rwkv_mm8_seq_f16(T, N, M, xs.data_ptr(), N, w[i % ncopy].data_ptr(), 1, N, mx.data_ptr(), rx.data_ptr(),
                                          my.data_ptr(), ry.data_ptr(), ys.data_ptr(), M, ws.data_ptr(), nbytes, st),
                       "rwkv_mm8_seq_f16")
-        for name, fn, n in (("mm8_one", one, reps), ("mm8_seq", seq, max(4, reps // 4))):
+        for name, fn, n in (("mm8_one", one, reps), ("mm8_seq", seq, max(4, reps // 2))):
             for i in range(3):
                 fn(i)
             k = [0]
@@ -329,7 +329,7 @@ def main():
     del ck
     torch.cuda.empty_cache()
 
-    # ---- prefill: one call over `prefill` tokens (median of 3, after one warm-up call)
+    # ---- prefill: one call over `prefill` tokens (median of 5 calls queued back to back, after the spin-up)
     ptoks = synth.random_tokens(args.prefill, V, seed=2)
     chunk = args.chunk if args.chunk > 0 else args.prefill
 
@@ -344,7 +344,7 @@ def main():
     prefill()
     spin_up(prefill, args.spinup)
     pt, evs = [], []
-    for _ in range(3):      # queued back to back: no idle gap between the calls
+    for _ in range(5):      # queued back to back: no idle gap between the calls
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
         out, state = prefill()
