@@ -17,8 +17,9 @@ One JSON line is printed:
   decode_hbm            whole-step figure: uint8 weight bytes per token x tokens/s / 8 TB/s
   prefill               prefill tokens/s and the MFMA fraction of the whole prefill
   isolated_mm8_op       the dequant-matmul operator alone at the 7B shapes: mm8_one GB/s, mm8_seq TFLOP/s
-  prefill_roofline      the prefill contraction alone on the model's largest matrix shape: 2 T N M flops /
-                        mean launch duration (HIP events), against the 2.5 PFLOP/s dense fp16 MFMA peak
+  prefill_roofline      the prefill contraction kernel alone on the model's largest matrix shape: 2 T N M flops /
+                        mean launch duration (HIP events around 20 launches, rwkv_mm8_seq_time_kernel), against
+                        the 2.5 PFLOP/s dense fp16 MFMA peak; "with_scaling_pass" = the whole rwkv_mm8_seq_f16
   cpu_baseline          the oracle's 'cpu fp32i8' path (numpy port of the reference's CPU arithmetic) timed on this
                         host on configs[0] (169M shape, 128-token prefill + 32 greedy steps, all BLAS threads)
   cpu_baseline_layer_sample   the same path on one layer + head of the benchmarked shape, extrapolated per token
@@ -175,10 +176,13 @@ def spin_up(fn, seconds, sync_every=1):
 
 
 def gemm_roofline(T, N, M, u8, reps=20):
-    """The prefill contraction alone on the model's largest matrix shape (channel-mix key, [T, N] x [N, M]),
-    through the C ABI (rwkv_mm8_seq_f16 incl. its activation-scaling pass, or rwkv_gemm_f16), timed with two
-    events on the stream it is launched on: algorithmic flops 2 T N M over the mean launch time against the
-    dense fp16 MFMA peak."""
+    """The prefill contraction kernel alone on the model's largest matrix shape (channel-mix key,
+    [T, N] x [N, M]), launched through the C ABI and timed with two events on the stream it is launched on:
+    algorithmic flops 2 T N M over the mean launch time against the dense fp16 MFMA peak.  With uint8 weights the
+    kernel is timed on rows that rwkv_mm8_seq_f16's activation-scaling pass has already scaled
+    (rwkv_mm8_seq_time_kernel), which is the duration a kernel trace reports for it; the whole operator, scaling
+    pass included, is timed beside it ("with_scaling_pass")."""
+    import ctypes
     import torch
     from chatrwkv_amd import lib
     L = lib.load()
@@ -186,19 +190,40 @@ def gemm_roofline(T, N, M, u8, reps=20):
     x = torch.randn(T, N, device=dev).half()
     y = torch.empty(T, M, device=dev, dtype=torch.float16)
     st = torch.cuda.current_stream().cuda_stream
+    flops = 2.0 * T * N * M
+
+    def timed(run):
+        for _ in range(3):
+            run()
+        spin_up(run, min(SPINUP_S, 0.5), sync_every=32)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            run()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e-3 / reps
+
+    extra = {}
     if u8:
         w = torch.randint(0, 256, (M, N), dtype=torch.uint8, device=dev)
         mx = torch.randn(M, device=dev).half(); rx = (torch.rand(M, device=dev) * 0.01).half()
         my = torch.randn(N, device=dev).half(); ry = (torch.rand(N, device=dev) * 0.06).half()
         nbytes = L.rwkv_mm8_seq_workspace(T, N)
         ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+        args = (T, N, M, x.data_ptr(), N, w.data_ptr(), 1, N, mx.data_ptr(), rx.data_ptr(), my.data_ptr(),
+                ry.data_ptr(), y.data_ptr(), M, ws.data_ptr(), nbytes, st)
 
         def run():
-            lib.check(L.rwkv_mm8_seq_f16(T, N, M, x.data_ptr(), N, w.data_ptr(), 1, N, mx.data_ptr(), rx.data_ptr(),
-                                         my.data_ptr(), ry.data_ptr(), y.data_ptr(), M, ws.data_ptr(), nbytes, st),
-                      "rwkv_mm8_seq_f16")
-        name = ("gemm_dma_kernel<uint8 weights> (direct-to-LDS loads; 256x256 or 128x128 tile by the launch cost model)"
-                + " + mm8_prepare_kernel")
+            lib.check(L.rwkv_mm8_seq_f16(*args), "rwkv_mm8_seq_f16")
+        t_op = timed(run)
+        ms = ctypes.c_float(0.0)
+        lib.check(L.rwkv_mm8_seq_time_kernel(*args, reps, ctypes.byref(ms)), "rwkv_mm8_seq_time_kernel")
+        t = ms.value * 1e-3
+        name = "gemm_dma_kernel<uint8 weights> (direct-to-LDS loads; 256x256 or 128x128 tile by the launch cost model)"
+        extra = {"with_scaling_pass": {"kernel": "mm8_prepare_kernel + " + name.split(" (")[0],
+                                       "ms_per_call": t_op * 1e3, "achieved": flops / t_op / 1e12,
+                                       "frac": flops / t_op / MFMA_F16_PEAK}}
     else:
         w = torch.randn(M, N, device=dev).half()
 
@@ -206,22 +231,12 @@ def gemm_roofline(T, N, M, u8, reps=20):
             lib.check(L.rwkv_gemm_f16(T, N, M, x.data_ptr(), N, w.data_ptr(), 1, N, y.data_ptr(), M, lib.RWKV_DT_F16, st),
                       "rwkv_gemm_f16")
         name = "gemm_dma_kernel<fp16 weights> (direct-to-LDS loads; 256x256 or 128x128 tile by the launch cost model)"
-    for _ in range(3):
-        run()
-    spin_up(run, min(SPINUP_S, 0.5), sync_every=32)
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
-    for _ in range(reps):
-        run()
-    e1.record()
-    torch.cuda.synchronize()
-    t = e0.elapsed_time(e1) * 1e-3 / reps
-    flops = 2.0 * T * N * M
+        t = timed(run)
     return {"bound": "mfma", "kernel": f"{name}, [{T} x {N}] x [{N} x {M}]", "achieved": flops / t / 1e12,
             "peak": MFMA_F16_PEAK / 1e12, "unit": "TFLOP/s", "frac": flops / t / MFMA_F16_PEAK,
             "traffic": MEASURED_TRAFFIC.get(("gemm", T, N, M, bool(u8))),
             "traffic_source": TRAFFIC_SOURCE if ("gemm", T, N, M, bool(u8)) in MEASURED_TRAFFIC else None,
-            "flops_per_launch": flops, "ms_per_launch": t * 1e3}
+            "flops_per_launch": flops, "ms_per_launch": t * 1e3, **extra}
 
 
 def isolated_mm8(reps=40):

@@ -19,6 +19,7 @@
 // different t0) run on the same XCD and the tile is fetched into that XCD's L2 once.
 #include <algorithm>
 #include "kernels.h"
+#include "../../include/rwkv_hip_bench.h"
 #include <cstdlib>
 #include <mutex>
 
@@ -1254,28 +1255,70 @@ extern "C" size_t rwkv_mm8_seq_workspace(int64_t B, int64_t N) {
     return (((size_t)B * N * 2 + 255) & ~(size_t)255) + (((size_t)B * 8 + 255) & ~(size_t)255) + RWKV_SPLITK_WS_BYTES;
 }
 
-extern "C" int rwkv_mm8_seq_f16(int64_t B, int64_t N, int64_t M, const rwkv_half *x, int64_t x_stride,
-                                const uint8_t *w, int64_t w_stride_n, int64_t w_stride_m, const rwkv_half *mx,
-                                const rwkv_half *rx, const rwkv_half *my, const rwkv_half *ry, rwkv_half *y,
-                                int64_t y_stride, void *workspace, size_t workspace_bytes, void *stream) {
+// rwkv_mm8_seq_f16 in its two launches: the activation-scaling pass (`reps` < 0), the contraction alone `reps`
+// times on the already scaled rows (`reps` > 0), or one of each (`reps` == 0: the product)
+static int mm8_seq_parts(int64_t B, int64_t N, int64_t M, const rwkv_half *x, int64_t x_stride, const uint8_t *w,
+                         int64_t w_stride_n, int64_t w_stride_m, const rwkv_half *mx, const rwkv_half *rx,
+                         const rwkv_half *my, const rwkv_half *ry, rwkv_half *y, int64_t y_stride, void *workspace,
+                         size_t workspace_bytes, hipStream_t st, int reps) {
     if (!x || !w || !mx || !rx || !my || !ry || !y || !workspace) return RWKV_E_NULL;
     if (B <= 0 || N <= 0 || M <= 0 || (N % BK) != 0 || B > (1 << 24) || M > (1 << 24)) return RWKV_E_SHAPE;
     if (w_stride_n != 1 || w_stride_m < N || (w_stride_m & 15) || !aligned16(w)) return RWKV_E_LAYOUT;
     if (x_stride < N || (x_stride & 7) || !aligned16(x) || y_stride < M || !aligned16(my) || !aligned16(ry))
         return RWKV_E_LAYOUT;
     if (workspace_bytes < rwkv_mm8_seq_workspace(B, N) || !aligned16(workspace)) return RWKV_E_WORKSPACE;
-    hipStream_t st = (hipStream_t)stream;
     rwkv_half *xs = (rwkv_half *)workspace;
     const size_t xs_bytes = ((size_t)B * N * 2 + 255) & ~(size_t)255;
     float *s0 = (float *)((unsigned char *)workspace + xs_bytes);
     float *s2 = s0 + B;
-    int rc = mm8_prepare_launch(B, N, x, x_stride, ry, my, xs, s0, s2, st);
-    if (rc) return rc;
+    if (reps <= 0) {
+        int rc = mm8_prepare_launch(B, N, x, x_stride, ry, my, xs, s0, s2, st);
+        if (rc || reps < 0) return rc;
+    }
     GemmEpi ep{};
     ep.mx = mx; ep.rx = rx; ep.s0 = s0; ep.s2 = s2; ep.act = ACT_NONE; ep.out_scale = 1.f; ep.out_dtype = RWKV_DT_F16;
     ep.splitk_ws = (float *)((unsigned char *)workspace + xs_bytes + (((size_t)B * 8 + 255) & ~(size_t)255));
     ep.splitk_bytes = RWKV_SPLITK_WS_BYTES;
-    return gemm_launch(true, B, N, M, xs, N, w, w_stride_m, y, y_stride, ep, st);
+    int rc = RWKV_OK;
+    for (int r = 0; r < (reps > 0 ? reps : 1) && rc == RWKV_OK; ++r)
+        rc = gemm_launch(true, B, N, M, xs, N, w, w_stride_m, y, y_stride, ep, st);
+    return rc;
+}
+
+extern "C" int rwkv_mm8_seq_f16(int64_t B, int64_t N, int64_t M, const rwkv_half *x, int64_t x_stride,
+                                const uint8_t *w, int64_t w_stride_n, int64_t w_stride_m, const rwkv_half *mx,
+                                const rwkv_half *rx, const rwkv_half *my, const rwkv_half *ry, rwkv_half *y,
+                                int64_t y_stride, void *workspace, size_t workspace_bytes, void *stream) {
+    return mm8_seq_parts(B, N, M, x, x_stride, w, w_stride_n, w_stride_m, mx, rx, my, ry, y, y_stride, workspace,
+                         workspace_bytes, (hipStream_t)stream, 0);
+}
+
+extern "C" int rwkv_mm8_seq_time_kernel(int64_t B, int64_t N, int64_t M, const rwkv_half *x, int64_t x_stride,
+                                        const uint8_t *w, int64_t w_stride_n, int64_t w_stride_m,
+                                        const rwkv_half *mx, const rwkv_half *rx, const rwkv_half *my,
+                                        const rwkv_half *ry, rwkv_half *y, int64_t y_stride, void *workspace,
+                                        size_t workspace_bytes, void *stream, int reps, float *ms_per_launch) {
+    if (!ms_per_launch) return RWKV_E_NULL;
+    if (reps <= 0) return RWKV_E_SHAPE;
+    hipStream_t st = (hipStream_t)stream;
+    int rc = mm8_seq_parts(B, N, M, x, x_stride, w, w_stride_n, w_stride_m, mx, rx, my, ry, y, y_stride, workspace,
+                           workspace_bytes, st, -1);
+    if (rc) return rc;
+    hipEvent_t e0, e1;
+    if (hipEventCreate(&e0) != hipSuccess) return (int)hipErrorOutOfMemory;
+    if (hipEventCreate(&e1) != hipSuccess) { (void)hipEventDestroy(e0); return (int)hipErrorOutOfMemory; }
+    (void)hipEventRecord(e0, st);
+    rc = mm8_seq_parts(B, N, M, x, x_stride, w, w_stride_n, w_stride_m, mx, rx, my, ry, y, y_stride, workspace,
+                       workspace_bytes, st, reps);
+    (void)hipEventRecord(e1, st);
+    hipError_t e = hipEventSynchronize(e1);
+    float ms = 0.f;
+    if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
+    if (e != hipSuccess && rc == RWKV_OK) rc = (int)e;
+    *ms_per_launch = ms / reps;
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    return rc;
 }
 
 // ---- rwkv_mm8_seq_f16 without a caller workspace ------------------------------------------------------------

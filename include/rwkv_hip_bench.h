@@ -1,6 +1,7 @@
 /*
  * Measurement aids of librwkv_hip.so: blocking entry points that time the one-token step of
- * rwkv_v4_forward_one (include/rwkv_hip.h) with HIP events on the stream the kernels run on.  They replace
+ * rwkv_v4_forward_one and the contraction kernel of rwkv_mm8_seq_f16 (include/rwkv_hip.h) with HIP events on
+ * the stream the kernels run on.  They replace
  * nothing in the reference and are not part of the product interface: bench.py is their only caller.
  */
 #ifndef RWKV_HIP_BENCH_H
@@ -29,6 +30,16 @@ int rwkv_v4_profile_one(const rwkv_v4_model *m, const rwkv_v4_layer_state *state
 int rwkv_v4_time_phase(const rwkv_v4_model *m, const rwkv_v4_layer_state *states, const int32_t *token,
                        float *logits, void *workspace, size_t workspace_bytes, void *stream, int phase,
                        int reps, float *ms_per_launch);
+
+/* Measurement aid: the arguments of rwkv_mm8_seq_f16.  Runs its activation-scaling pass once, then the
+ * contraction kernel alone `reps` times back to back on the scaled rows between two HIP events on `stream`,
+ * blocks, and returns the mean duration of one contraction launch in milliseconds (both launches of a product
+ * whose K is split).  y holds the product afterwards. */
+int rwkv_mm8_seq_time_kernel(int64_t B, int64_t N, int64_t M, const rwkv_half *x, int64_t x_stride,
+                             const uint8_t *w, int64_t w_stride_n, int64_t w_stride_m, const rwkv_half *mx,
+                             const rwkv_half *rx, const rwkv_half *my, const rwkv_half *ry, rwkv_half *y,
+                             int64_t y_stride, void *workspace, size_t workspace_bytes, void *stream, int reps,
+                             float *ms_per_launch);
 
 #ifdef __cplusplus
 }

@@ -119,6 +119,32 @@ def test_mm8_seq(N, M, B):
     assert np.abs(y1.cpu().numpy().astype(np.float64) - y[B - 1].cpu().numpy()).max() <= np.abs(ref).max() * 2 ** -9
 
 
+def test_mm8_seq_timing_aid_leaves_the_product():
+    """rwkv_mm8_seq_time_kernel (the kernel-only timer of the bench) runs the same two launches as
+    rwkv_mm8_seq_f16: the output is bit-equal and the mean launch time is positive; whole, ragged and split-K."""
+    import ctypes
+    from chatrwkv_amd import lib
+    ops = _ops()
+    L = lib.load()
+    for N, M, B in ((4096, 4096, 256), (1024, 136, 129), (16384, 4096, 520)):
+        x, ref, (q, mx, rx, my, ry) = _mm8_case(N, M, B, N + M + B)
+        xt = torch.from_numpy(x).to(DEV)
+        want = ops.cuda_mm8_seq(B, N, M, xt, q, mx, rx, my, ry)
+        y = torch.zeros((B, M), device=DEV, dtype=torch.float16)
+        nbytes = L.rwkv_mm8_seq_workspace(B, N)
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=DEV)
+        ms = ctypes.c_float(-1.0)
+        rc = L.rwkv_mm8_seq_time_kernel(B, N, M, xt.data_ptr(), N, q.data_ptr(), q.stride(0), q.stride(1),
+                                        mx.data_ptr(), rx.data_ptr(), my.data_ptr(), ry.data_ptr(), y.data_ptr(), M,
+                                        ws.data_ptr(), nbytes, torch.cuda.current_stream().cuda_stream, 3,
+                                        ctypes.byref(ms))
+        lib.check(rc, "rwkv_mm8_seq_time_kernel")
+        assert torch.equal(y, want) and 0.0 < ms.value < 100.0
+        assert L.rwkv_mm8_seq_time_kernel(B, N, M, xt.data_ptr(), N, q.data_ptr(), q.stride(0), q.stride(1),
+                                          mx.data_ptr(), rx.data_ptr(), my.data_ptr(), ry.data_ptr(), y.data_ptr(),
+                                          M, ws.data_ptr(), nbytes, None, 0, ctypes.byref(ms)) == -1  # RWKV_E_SHAPE
+
+
 def test_mm8_linearity_full_size():
     """Size-independent property at the 7B shape: mm8(a + b) == mm8(a) + mm8(b) in fp32 up to rounding."""
     ops = _ops()
