@@ -145,6 +145,58 @@ __global__ __launch_bounds__(256) void v6_mix2_kernel(Mix2Args a) {
     }
 }
 
+// The same sums for sequence calls with four adjacent channels per thread: grid (ceil(T / TT), ceil(C / 1024), 5), TT
+// tokens per workgroup (16, or 4 in short calls, which would otherwise have too few workgroups for the chip).  The
+// coefficient, xx, sxd and output accesses are 8 bytes per lane instead of 2, and one LDS read of four tokens' t1
+// serves four channels; every channel's sum still runs in index order, so the results equal v6_mix2_kernel's.
+template <int TT>
+__global__ __launch_bounds__(256) void v6_mix2x4_kernel(Mix2Args a) {
+    __shared__ __align__(16) float st1[64][TT];
+    const int t0 = blockIdx.x * TT, c = (blockIdx.y * 256 + threadIdx.x) * 4, j = blockIdx.z, R = a.R, C = a.C;
+    const int nt = min(TT, a.T - t0);
+    for (int i = threadIdx.x; i < TT * R; i += 256) {
+        const int tt = i / R, r = i - tt * R;
+        st1[r][tt] = tt < nt ? h2f(a.t1[(size_t)(t0 + tt) * 5 * R + j * R + r]) : 0.f;
+    }
+    __syncthreads();
+    if (c >= C) return;
+    const h16x4 maa = *(const h16x4 *)(a.maa[j] + c);
+    const rwkv_half *w = a.w2 + (size_t)j * R * C + c;
+    f32x4 m[TT];
+#pragma unroll
+    for (int tt = 0; tt < TT; ++tt) m[tt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int i0 = 0; i0 < R; i0 += 8) {
+        h16x4 wv[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) wv[i] = *(const h16x4 *)(w + (size_t)(i0 + i) * C);   // R is a multiple of 8
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const f32x4 wf = {(float)wv[i][0], (float)wv[i][1], (float)wv[i][2], (float)wv[i][3]};
+#pragma unroll
+            for (int q = 0; q < TT / 4; ++q) {
+                const f32x4 s4 = *(const f32x4 *)&st1[i0 + i][4 * q];
+                m[4 * q + 0] += s4[0] * wf;
+                m[4 * q + 1] += s4[1] * wf;
+                m[4 * q + 2] += s4[2] * wf;
+                m[4 * q + 3] += s4[3] * wf;
+            }
+        }
+    }
+#pragma unroll
+    for (int tt = 0; tt < TT; ++tt) {
+        const size_t o = (size_t)(t0 + min(tt, nt - 1)) * C + c;
+        const h16x4 xx4 = *(const h16x4 *)(a.xx + o), sd4 = *(const h16x4 *)(a.sxd + o);
+        h16x4 out4;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const float xx = (float)xx4[e];
+            const float mm = round_h((float)maa[e] + round_h(m[tt][e]));
+            out4[e] = (h16)(xx + round_h((float)sd4[e] * mm));
+        }
+        if (tt < nt) *(h16x4 *)(a.out[j] + o) = out4;
+    }
+}
+
 struct Ws56 {
     rwkv_half *x, *xx, *sxd, *xxx, *t1, *mix[5], *d1, *d2, *r, *k, *v, *g, *att, *vx, *xs, *xx_att, *xx_ffn;
     float *sums, *splitk, *y32;
@@ -287,6 +339,10 @@ extern "C" int rwkv_v56_forward(const rwkv_v56_model *m, const rwkv_v56_layer_st
             b.T = (int)T; b.C = C; b.R = lm; b.t1 = ws.t1; b.w2 = l.tm_w2;
             for (int j = 0; j < 5; ++j) { b.maa[j] = l.att_mix[1 + j]; b.out[j] = ws.mix[j]; }
             if (T == 1) hipLaunchKernelGGL(v6_mix2_kernel<1>, dim3(1, (unsigned)((C + 255) / 256), 5), dim3(256), 0, st, b);
+            else if (!(C & 3) && lm <= 64) {
+                if (T <= 512) hipLaunchKernelGGL(v6_mix2x4_kernel<4>, dim3((unsigned)((T + 3) / 4), (unsigned)((C + 1023) / 1024), 5), dim3(256), 0, st, b);
+                else hipLaunchKernelGGL(v6_mix2x4_kernel<16>, dim3((unsigned)((T + 15) / 16), (unsigned)((C + 1023) / 1024), 5), dim3(256), 0, st, b);
+            }
             else hipLaunchKernelGGL(v6_mix2_kernel<16>, dim3((unsigned)((T + 15) / 16), (unsigned)((C + 255) / 256), 5), dim3(256), 0, st, b);
             wx = ws.mix[0]; kx = ws.mix[1]; vx = ws.mix[2]; rx = ws.mix[3]; gx = ws.mix[4];
             // one token: the first decay-LoRA stage rides at the end of the receptance / key / value / gate launch
