@@ -455,120 +455,6 @@ __global__ __launch_bounds__(256) void wkv56_split_kernel(Wkv56Args a) {
     for (int e = 0; e < 4; ++e) S[(4 * g + e) * HS + i] = s[e];
 }
 
-// wkv56_split_kernel with eight waves per workgroup: thread (value i, key group g of 32) owns keys 2g, 2g + 1 of
-// column i, so a SIMD holds two waves whose token loops overlap each other's latencies.  lane & 31 = g, lane >> 5 and
-// the wave index give i; the sum over the 32 key groups is a DPP row sum plus a row broadcast (lanes 16..31 and
-// 48..63 hold it).  Slabs of 64 tokens, staged by all 512 threads.  Each state entry and each y goes through the same
-// operations as in wkv56_split_kernel, but y sums its 64 products in a different order.
-constexpr int TS3 = 64;  // tokens per slab
-
-DEV float row32_sum_hi(float v) {   // valid in the upper 16 lanes of each half-wave
-    v = row16_sum(v);
-    // row_bcast:15 -- lane 15 of rows 0 and 2 is added into every lane of rows 1 and 3
-    return v + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x142, 0xa, 0xf, false));
-}
-
-template <int WMODE>
-__global__ __launch_bounds__(512) void wkv56_split8_kernel(Wkv56Args a) {
-    __shared__ __align__(16) float sr[TS3][HS], sk[TS3][HS], sw[TS3][HS];
-    __shared__ float sv[TS3][16];
-    const int T = a.T, C = a.C;
-    const int h = blockIdx.x >> 2, vb = blockIdx.x & 3;
-    const int lane = threadIdx.x & 63, g = lane & 31;
-    const int il = (threadIdx.x >> 6) * 2 + (lane >> 5);   // value column within the block of 16
-    const int i = vb * 16 + il;
-    // staging role: token threadIdx.x / 8 of the slab, channels 8 (threadIdx.x % 8) .. + 7 of the head
-    const int stt = threadIdx.x >> 3, sp = threadIdx.x & 7, sc = sp * 8;
-    float *S = a.state + (size_t)h * HS * HS;               // [key][value]
-    float s[2], u2[2], wc[2];
-#pragma unroll
-    for (int e = 0; e < 2; ++e) {
-        const int j = 2 * g + e;
-        s[e] = S[j * HS + i];
-        u2[e] = a.u[h * HS + j];
-        wc[e] = WMODE == 0 ? ((const float *)a.w)[h * HS + j] : 0.f;
-    }
-    float tdec[8];
-#pragma unroll
-    for (int e = 0; e < 8; ++e) tdec[e] = WMODE == 2 ? a.t_decay[h * HS + sc + e] : 0.f;
-    h16x8 pr, pk, pw = {};
-    h16x2 pv;
-    auto fetch = [&](int t0) {
-        const size_t o = (size_t)min(t0 + stt, T - 1) * C + h * HS;   // rows past the end re-read the last one
-        pr = *(const h16x8 *)((const rwkv_half *)a.r + o + sc);
-        pk = *(const h16x8 *)((const rwkv_half *)a.k + o + sc);
-        if (WMODE == 2) pw = *(const h16x8 *)((const rwkv_half *)a.w + o + sc);
-        pv = *(const h16x2 *)((const rwkv_half *)a.v + o + vb * 16 + 2 * sp);
-    };
-    fetch(0);
-    for (int t0 = 0; t0 < T; t0 += TS3) {
-        const int nt = min(TS3, T - t0);
-        __syncthreads();  // previous slab fully consumed
-#pragma unroll
-        for (int u = 0; u < 2; ++u) {
-            f32x4 r4, k4, w4;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                r4[e] = (float)pr[4 * u + e];
-                k4[e] = (float)pk[4 * u + e];
-                w4[e] = WMODE == 2 ? expf(-expf(tdec[4 * u + e] + (float)pw[4 * u + e])) : 0.f;
-            }
-            *(f32x4 *)&sr[stt][sc + 4 * u] = r4;
-            *(f32x4 *)&sk[stt][sc + 4 * u] = k4;
-            if (WMODE == 2) *(f32x4 *)&sw[stt][sc + 4 * u] = w4;
-        }
-        sv[stt][2 * sp] = (float)pv[0];
-        sv[stt][2 * sp + 1] = (float)pv[1];
-        __syncthreads();
-        fetch(t0 + TS3);
-        struct Tok { float vi; f32x2 r2, k2, w2; };
-        auto ldtok = [&](int tt) {
-            Tok q;
-            q.vi = sv[tt][il];
-            q.r2 = *(const f32x2 *)&sr[tt][2 * g];
-            q.k2 = *(const f32x2 *)&sk[tt][2 * g];
-            q.w2 = WMODE == 2 ? *(const f32x2 *)&sw[tt][2 * g] : f32x2{};
-            return q;
-        };
-        auto partial = [&](const Tok &q) {
-            float y = 0.f;
-#pragma unroll
-            for (int e = 0; e < 2; ++e) {
-                const float x = q.k2[e] * q.vi;
-                y += q.r2[e] * (u2[e] * x + s[e]);
-                s[e] = s[e] * (WMODE == 2 ? q.w2[e] : wc[e]) + x;
-            }
-            return y;
-        };
-        for (int tt = 0; tt < nt; tt += 8) {
-            Tok q[8];
-#pragma unroll
-            for (int p = 0; p < 8; ++p) q[p] = ldtok(min(tt + p, TS3 - 1));
-            float y[8];
-            if (tt + 7 < nt) {
-#pragma unroll
-                for (int p = 0; p < 8; ++p) y[p] = partial(q[p]);
-#pragma unroll
-                for (int p = 0; p < 8; ++p) y[p] = row32_sum_hi(y[p]);
-                if (g == 31) {
-                    float *yo = a.y + (size_t)(t0 + tt) * C + h * HS + i;
-#pragma unroll
-                    for (int p = 0; p < 8; ++p) yo[p * (size_t)C] = y[p];
-                }
-            } else {
-#pragma unroll
-                for (int p = 0; p < 7; ++p)
-                    if (tt + p < nt) {
-                        const float yy = row32_sum_hi(partial(q[p]));
-                        if (g == 31) a.y[(size_t)(t0 + tt + p) * C + h * HS + i] = yy;
-                    }
-            }
-        }
-    }
-#pragma unroll
-    for (int e = 0; e < 2; ++e) S[(2 * g + e) * HS + i] = s[e];
-}
-
 // GroupNorm over each head's 64 outputs (eps 64e-5), affine, fp16 rounding, gate: one wave per (token, head).
 __global__ __launch_bounds__(256) void wkv56_gn_kernel(int T, int C, const float *__restrict__ y,
                                                        const float *__restrict__ lnx_w, const float *__restrict__ lnx_b,
@@ -654,10 +540,7 @@ int wkv56_fused_launch(bool v6, int T, int C, int H, float *state, const rwkv_ha
     if (T >= 32 && y32) {
         // long call: four workgroups per head, raw y to the fp32 scratch, GroupNorm + gate in a second launch
         a.y = y32;
-        if (T >= TS3) {   // eight waves per workgroup (measured at 1024 tokens, 64 heads: +1.3 % on the whole prefill)
-            if (v6) hipLaunchKernelGGL((wkv56_split8_kernel<2>), dim3((unsigned)(4 * H)), dim3(512), 0, st, a);
-            else hipLaunchKernelGGL((wkv56_split8_kernel<0>), dim3((unsigned)(4 * H)), dim3(512), 0, st, a);
-        } else if (v6) hipLaunchKernelGGL((wkv56_split_kernel<2>), dim3((unsigned)(4 * H)), dim3(256), 0, st, a);
+        if (v6) hipLaunchKernelGGL((wkv56_split_kernel<2>), dim3((unsigned)(4 * H)), dim3(256), 0, st, a);
         else hipLaunchKernelGGL((wkv56_split_kernel<0>), dim3((unsigned)(4 * H)), dim3(256), 0, st, a);
         const int64_t waves = (int64_t)T * H;
         hipLaunchKernelGGL(wkv56_gn_kernel, dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, st, T, C, y32, lnx_w, lnx_b,
