@@ -1,4 +1,4 @@
-"""The reference-side binding printed in INTEGRATION.md, executed as it stands: the python block that replaces the
+"""The reference-side binding printed in the integration guide at the repository root, executed as it stands: the python block that replaces the
 reference's JIT-loaded ops (model.py:29-86) is taken out of the document, pointed at the built library, and its
 three wrappers are checked against the fp64 / oracle results the operator tests use.  A signature in the document
 that drifts from include/rwkv_hip.h fails here."""
@@ -26,7 +26,7 @@ def _binding():
     assert "ctypes.CDLL('librwkv_hip.so')" in src
     src = src.replace("ctypes.CDLL('librwkv_hip.so')", f"ctypes.CDLL({_lib.LIB_PATH!r})")
     ns = {}
-    exec(compile(src, "INTEGRATION.md", "exec"), ns)
+    exec(compile(src, "<documented binding>", "exec"), ns)
     return ns
 
 
