@@ -531,7 +531,9 @@ extern "C" int rwkv_v4_forward_seq(const rwkv_v4_model *m, const rwkv_v4_layer_s
         e = GemmEpi{};
         e.out_scale = 1.f; e.out_dtype = RWKV_DT_F16;
         e.act = ACT_SIGMOID;
-        ForkScope par2(ss, st, 1, !dma_seq && (T / 128) * (C / 128) > 128);
+        // the receptance product beside the key product: where neither would split K, and in calls of three row tiles
+        // (257 .. 384 tokens: +4 % at n_embd 4096; slower at 256 and from 385 on)
+        ForkScope par2(ss, st, 1, !dma_seq && ((T / 128) * (C / 128) > 128 || ((T + 127) / 128 == 3 && C >= 2048)));
         float *sk2 = par2 ? nullptr : ws.splitk;
         if (T <= 128 && !(C & 127) && !(F & 127)) {
             // short calls: receptance and key in one grouped launch
