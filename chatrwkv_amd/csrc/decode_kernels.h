@@ -36,22 +36,57 @@ struct MatDev {
     const rwkv_half *mx, *rx, *my, *ry;
 };
 
-// Workgroup sums of K values with ONE barrier: `red` (K * DWAVES floats) must not be in use by
-// an earlier reduction that other waves may still be reading (callers pass disjoint regions).
-// Stage 2 reads one wave's partial per lane (lane l takes wave l % 16: DWAVES == 16 == one DPP
-// row) and finishes with a 16-lane row sum.
+// Sum over the wave that only the last lane needs: the row butterfly, then the row totals travel up through
+// two DPP row broadcasts, (r3 + r2) + (r1 + r0) -- the value wave_sum forms, in 6 instructions instead of 11.
+DEV float wave_sum_lane63(float v) {
+    v = row16_sum(v);
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x142, 0xa, 0xf, false));  // row_bcast:15
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x143, 0xc, 0xf, false));  // row_bcast:31
+    return v;
+}
+// Sums of K values over the first `npw` waves of the workgroup (the waves that run a prologue), in two
+// halves with a synchronisation between them, which the caller places: `put` by each of those waves
+// before it, `get` by any wave after it.  `red` (K * DWAVES floats) must not be in use by an
+// earlier reduction that other waves may still be reading (callers pass disjoint regions).  `get` reads
+// one wave's partial per lane (lane l takes wave l % 16: DWAVES == 16 == one DPP row; waves >= npw count
+// as zero) and finishes with a 16-lane row sum.
 template <int K>
-DEV void block_sum_1b(float (&v)[K], float *red) {
-    static_assert(DWAVES == 16, "stage 2 assumes 16 waves");
+DEV void wave_sums_put(float (&v)[K], float *red) {
     const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
 #pragma unroll
-    for (int k = 0; k < K; ++k) v[k] = wave_sum(v[k]);
-    if (lane == 0)
+    for (int k = 0; k < K; ++k) v[k] = wave_sum_lane63(v[k]);
+    if (lane == 63)
 #pragma unroll
         for (int k = 0; k < K; ++k) red[k * DWAVES + wid] = v[k];
-    __syncthreads();
+}
+template <int K>
+DEV void wave_sums_get(float (&v)[K], const float *red, int npw) {
+    static_assert(DWAVES == 16, "one partial per lane of a DPP row");
+    const int l = threadIdx.x & 15;
 #pragma unroll
-    for (int k = 0; k < K; ++k) v[k] = row16_sum(red[k * DWAVES + (lane & 15)]);
+    for (int k = 0; k < K; ++k) v[k] = row16_sum(l < npw ? red[k * DWAVES + l] : 0.f);
+}
+
+// Hand-shake among the prologue waves of a workgroup, and from them to the other waves, through two counters
+// in LDS instead of s_barrier.  A workgroup barrier completes when its LAST wave arrives, and the waves that
+// stream weights arrive late: the issue of a tile load blocks while the CU's request queue is full.  With
+// counters the prologue waves wait for each other only, and a streaming wave looks at the second counter
+// when it needs the activation vector, after it has put its first tile in flight.
+// The counters are cleared before the workgroup's first barrier.  LDS operations of one wave are performed
+// in order, so a wave's partial sums and vector items are in LDS before its increment.  The spin is bounded
+// so that a mistake elsewhere ends in wrong numbers, not in a wave that never exits.
+constexpr int PRO_SPIN_MAX = 1 << 22;
+DEV void pro_arrive(unsigned *cnt) {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    if ((threadIdx.x & 63) == 0) __hip_atomic_fetch_add(cnt, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+}
+DEV void pro_wait(unsigned *cnt, unsigned n) {
+    for (int i = 0; i < PRO_SPIN_MAX; ++i) {
+        const unsigned c = __hip_atomic_load(cnt, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        if ((unsigned)__builtin_amdgcn_readfirstlane((int)c) >= n) break;
+        __builtin_amdgcn_s_sleep(1);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
 }
 
 // fp16 element-wise helpers, one rounding per operation (no contraction into fma): what the
@@ -61,7 +96,11 @@ DEV h16x8 mul_h(h16x8 a, h16x8 b) { return a * b; }
 // xx * m + prev * (1 - m)
 DEV h16x8 mix_lerp(h16x8 xx, h16x8 prev, h16x8 m) {
     const h16x8 one = {(h16)1.f, (h16)1.f, (h16)1.f, (h16)1.f, (h16)1.f, (h16)1.f, (h16)1.f, (h16)1.f};
-    const h16x8 a = xx * m, t = one - m, b = prev * t;
+    // 1 - m as (-m) + 1 with the sign flipped on the bit pattern: the compiler turns a vector "1 - m" into scalar
+    // half subtractions and re-packing (9 instructions per 2 elements instead of 2)
+    const u32x4 sign = {0x80008000u, 0x80008000u, 0x80008000u, 0x80008000u};
+    const h16x8 negm = __builtin_bit_cast(h16x8, __builtin_bit_cast(u32x4, m) ^ sign);
+    const h16x8 a = xx * m, t = negm + one, b = prev * t;
     return a + b;
 }
 // xx + (prev - xx) * m
@@ -103,15 +142,20 @@ struct LnMixPro {
         }
     }
 
+    // Run by the prologue waves only (the waves with owning threads): the waits for the operand loads sit
+    // in here, so a wave that skips it never waits for the weight tile it has in flight.  The prologue
+    // waves meet once in the middle (sync[0]) and report on sync[1] when their part of the vectors and
+    // sums is in LDS; every wave calls finish() once sync[1] has reached the number of prologue waves.
     // red: 2 * DWAVES + 3 * NJ * DWAVES floats
     // maa_form: the RWKV-6 mixing kx = xx + (prev - xx) * m instead of kx = xx * m + prev * (1 - m)
-    DEV void compute(int C, bool has_sx, const rwkv_half *const (&mixp)[NJ], h16 *const (&xs)[NJ], VecSums (&S)[NJ],
-                     rwkv_half *xx_out, float *red, bool maa_form = false) {
-        // All threads run the arithmetic (threads that own no elements work on zeros and are masked out
-        // of the LDS writes): the waits on the operand loads then sit on every path.  The prologue is
-        // bound by VALU issue (its ~10 operand vectors live in two waves per SIMD), so the element-wise
-        // chain uses packed fp16 instructions, which round after every operation exactly as the
-        // reference's fp16 tensor arithmetic does, and v_dot2_f32_f16 for the fp32 sums.
+    DEV void compute(int C, bool has_sx, const rwkv_half *const (&mixp)[NJ], h16 *const (&xs)[NJ],
+                     rwkv_half *xx_out, float *red, unsigned *sync, bool maa_form = false) {
+        // All threads of these waves run the arithmetic (threads that own no elements work on zeros and are
+        // masked out of the LDS writes).  The prologue is bound by VALU issue (its ~10 operand vectors live
+        // in two waves per SIMD), so the element-wise chain uses packed fp16 instructions, which round
+        // after every operation exactly as the reference's fp16 tensor arithmetic does, and v_dot2_f32_f16
+        // for the fp32 sums.
+        const int npw = ((C >> 3) + 63) >> 6;
         const h16x2 ones = {(h16)1.f, (h16)1.f};
         float m[2] = {0.f, 0.f};
 #pragma unroll
@@ -120,7 +164,10 @@ struct LnMixPro {
             m[0] = __builtin_amdgcn_fdot2(xp, ones, m[0], false);
             m[1] = __builtin_amdgcn_fdot2(xp, xp, m[1], false);
         }
-        block_sum_1b<2>(m, red);
+        wave_sums_put<2>(m, red);
+        pro_arrive(&sync[0]);
+        pro_wait(&sync[0], npw);
+        wave_sums_get<2>(m, red, npw);
         const float mean = m[0] / C;
         const float rstd = rsqrtf(fmaxf(m[1] / C - mean * mean, 0.f) + LN_EPS);
         const int nseg = C >> 4, j8 = threadIdx.x;
@@ -130,7 +177,6 @@ struct LnMixPro {
         h16x8 xx;
 #pragma unroll
         for (int e = 0; e < 8; ++e) xx[e] = (h16)(((float)x[e] - mean) * rstd * (float)lw[e] + (float)lb[e]);
-        if (own && xx_out && blockIdx.x == 0) *(h16x8 *)(xx_out + 8 * j8) = xx;
         const h16x8 pv = has_sx ? sx : xx;
 #pragma unroll
         for (int j = 0; j < NJ; ++j) {
@@ -149,16 +195,24 @@ struct LnMixPro {
             }
             if (own) ((h16x8 *)xs[j])[xs_item<U8>(j8, nseg)] = o;
         }
-        // one barrier publishes both the LDS activation vectors and the partial sums
-        block_sum_1b<3 * NJ>(acc, red + 2 * DWAVES);
-        if (U8)
+        if (U8) wave_sums_put<3 * NJ>(acc, red + 2 * DWAVES);
+        pro_arrive(&sync[1]);   // this wave's part of the activation vectors and of the partial sums is in LDS
+        // the new token-shift state, by workgroup 0 -- after the hand-shake, whose release would wait for the store
+        if (own && xx_out && blockIdx.x == 0) *(h16x8 *)(xx_out + 8 * j8) = xx;
+    }
+
+    // every wave, once all prologue waves have reported
+    static DEV void finish(int C, VecSums (&S)[NJ], const float *red) {
+        if (!U8) return;
+        float acc[3 * NJ];
+        wave_sums_get<3 * NJ>(acc, red + 2 * DWAVES, ((C >> 3) + 63) >> 6);
 #pragma unroll
-            for (int j = 0; j < NJ; ++j) { S[j].s0 = acc[3 * j]; S[j].s1 = acc[3 * j + 1]; S[j].s2 = acc[3 * j + 2]; }
+        for (int j = 0; j < NJ; ++j) { S[j].s0 = acc[3 * j]; S[j].s1 = acc[3 * j + 1]; S[j].s2 = acc[3 * j + 2]; }
     }
 };
 
-// wave-uniform: does this wave hold any of the `groups` 8-element groups that threads 0..groups-1 own?
-DEV bool pro_owner_wave(int groups) { return __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)) * 64 < groups; }
+// number of waves that hold any of the `groups` 8-element groups that threads 0..groups-1 own
+DEV int pro_waves(int groups) { return (groups + 63) >> 6; }
 
 template <bool U8>
 DEV const uint8_t *row_ptr(const MatDev &m, int64_t row) {
@@ -175,9 +229,11 @@ DEV float finish(float dot, const VecSums &S, float rx, float mx) {
 // otherwise).  Every wave owns a contiguous range of groups and walks it as a flat sequence of
 // batches (G groups x U segments per lane), ping-ponging between two register tiles: the loads
 // of batch q+1 are in flight while batch q is multiplied.
-//   pro_wave:             wave-uniform: this wave's threads hold prologue operands
-//   pro_load():           issue the loads of the prologue operands (called first)
-//   pro_compute():        build the LDS activation vectors (contains the workgroup barriers)
+//   npw:                  number of prologue waves: the first npw waves' threads hold prologue operands (PRO)
+//   sync:                 two counters in LDS (PRO)
+//   pro_load():           prologue waves: issue the loads of the prologue operands (called first)
+//   pro_compute():        prologue waves: build the LDS activation vectors, then pro_arrive(&sync[1])
+//   pro_finish():         every wave, once sync[1] == npw (reads the sums the prologue left in LDS)
 //   rowf(g, k, row, xs):  weight row pointer and LDS activation vector of row k of group g
 //   epi_load(g) -> E:     loads of the operands the epilogue of group g needs, as loaded (no
 //                         arithmetic on them: that would wait for the loads where they are issued)
@@ -195,9 +251,10 @@ DEV float finish(float dot, const VecSums &S, float rx, float mx) {
 // Epilogue operands travel with the tile buffers: the operands of a group batch are loaded into
 // the slot of the tile that carries its second segment batch (its only one when there is one
 // per group batch), and read back when its last segment batch has been reduced.
-template <bool U8, int G, int K, int U, class E, class ProLoad, class ProCompute, class RowFn, class EpiLoad, class EpiFn>
-DEV void stream_rows(int ngroups, int nseg, bool pro_wave, ProLoad pro_load, ProCompute pro_compute, RowFn rowf,
-                     EpiLoad epi_load, EpiFn epi) {
+template <bool U8, int G, int K, int U, class E, bool PRO, class ProLoad, class ProCompute, class ProFinish, class RowFn,
+          class EpiLoad, class EpiFn>
+DEV void stream_rows(int ngroups, int nseg, int npw, unsigned *sync, ProLoad pro_load, ProCompute pro_compute,
+                     ProFinish pro_finish, RowFn rowf, EpiLoad epi_load, EpiFn epi) {
     constexpr int R = G * K;
     const int lane = threadIdx.x & 63;
     // the wave index through readfirstlane: the compiler then knows that everything derived from it (row
@@ -252,19 +309,39 @@ DEV void stream_rows(int ngroups, int nseg, bool pro_wave, ProLoad pro_load, Pro
             for (int r = 0; r < R; ++r) acc[r] = 0.f;
         }
     };
-    pro_load();
+    // Waves whose threads hold prologue operands request them, run the prologue and fetch their first tile
+    // after it.  The other waves request their first tile at once, which keeps HBM busy meanwhile, and then
+    // wait for the prologue's result.
     // The vector memory path of a CU returns data in request order across its waves: a prologue operand
-    // (an L2 hit) requested after another wave's weight tile (HBM) comes back after that tile.  The barrier
-    // puts the prologue requests of all 16 waves in front of every tile request, so the prologue can run
-    // while the first tiles are in flight instead of after them.
-    __builtin_amdgcn_s_barrier();
-    // Waves whose threads hold prologue operands start the prologue at once and fetch their first tile after
-    // it: issuing a tile blocks while the CU's request queue is full, and the prologue's workgroup barriers
-    // would wait for that.  The other waves have nothing to do in the prologue but to pass its barriers, and
-    // their first tiles keep HBM busy meanwhile.
-    if (!pro_wave) load(t0, e0, 0);
-    pro_compute();
-    if (pro_wave) load(t0, e0, 0);
+    // requested after another wave's weight tile comes back after that tile.  The barrier puts the prologue
+    // requests in front of every tile request, so the prologue can run while the first tiles are in flight
+    // instead of after them (it also orders the clearing of the counters before their first use).
+    // The two paths are separate code from the first instruction on (one scalar branch): the compiler's
+    // waits for the prologue operands count every load of the wave down to zero, and it places them on
+    // every path on which those loads may have been issued.  On a common path a wave with a tile in flight
+    // waited for that tile inside the prologue, and at a workgroup barrier so did everyone else: 2 - 4 us of
+    // a 6 - 18 us launch during which nothing was requested from HBM.
+    // What was measured around this (7B shape, us per token): a second tile in flight before the wait
+    // 1875 against 1792 (requests that cannot be issued while the CU's queue is full hold up the prologue
+    // waves on the same SIMD); workgroup barriers instead of the counters 1812 against 1786; the streaming
+    // waves not waiting for the operand requests at all (no first barrier) 1798 against 1784.
+    if (PRO) {
+        const bool pro_wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)) < npw;
+        if (threadIdx.x == 0) { sync[0] = 0; sync[1] = 0; }
+        if (pro_wave) {
+            pro_load();
+            __syncthreads();
+            pro_compute();
+            load(t0, e0, 0);
+        } else {
+            __syncthreads();
+            load(t0, e0, 0);
+        }
+        pro_wait(&sync[1], (unsigned)npw);
+        pro_finish();
+    } else {
+        load(t0, e0, 0);
+    }
     for (int q = 0; q < nb; q += 2) {
         load(t1, e1, q + 1);
         process(t0, q);
@@ -296,6 +373,7 @@ template <bool U8, int G>
 __global__ __launch_bounds__(DTHREADS) void att_kernel(AttArgs a) {
     extern __shared__ __align__(16) unsigned char smem[];
     __shared__ float red[(2 + 9) * DWAVES];
+    __shared__ unsigned sync[2];
     const int C = a.C;
     h16 *xs[3] = {(h16 *)smem, (h16 *)smem + C, (h16 *)smem + 2 * C};
     VecSums S[3];
@@ -303,7 +381,8 @@ __global__ __launch_bounds__(DTHREADS) void att_kernel(AttArgs a) {
     auto pro_load = [&]() {
         pro.load(resolve_x(a.x, a.emb, a.token, C, a.vocab), C, a.ln_w, a.ln_b, a.sx, a.mix, a.mat);
     };
-    auto pro_compute = [&]() { pro.compute(C, a.sx != nullptr, a.mix, xs, S, a.xx_tmp, red); };
+    auto pro_compute = [&]() { pro.compute(C, a.sx != nullptr, a.mix, xs, a.xx_tmp, red, sync); };
+    auto pro_finish = [&]() { LnMixPro<U8, 3>::finish(C, S, red); };
     auto rowf = [&](int c, int k, const uint8_t *&row, const h16 *&xv) {
         row = row_ptr<U8>(a.mat[k], c);
         xv = xs[k];
@@ -336,7 +415,8 @@ __global__ __launch_bounds__(DTHREADS) void att_kernel(AttArgs a) {
         a.pp[c] = p;
         a.rwkv[c] = f2h(r * round_h(wkv));
     };
-    stream_rows<U8, G, 3, 2, AttEpi>(C, (C * (U8 ? 1 : 2)) >> 4, pro_owner_wave(C >> 3), pro_load, pro_compute, rowf, epi_load, epi);
+    stream_rows<U8, G, 3, 2, AttEpi, true>(C, (C * (U8 ? 1 : 2)) >> 4, pro_waves(C >> 3), sync, pro_load, pro_compute, pro_finish,
+                                           rowf, epi_load, epi);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -363,6 +443,7 @@ template <bool U8, int NJ, int G>
 __global__ __launch_bounds__(DTHREADS) void lnmix_kernel(LnMixArgs a) {
     extern __shared__ __align__(16) unsigned char smem[];
     __shared__ float red[(2 + 3 * NJ) * DWAVES];
+    __shared__ unsigned sync[2];
     const int C = a.C;
     h16 *xs[NJ];
     const rwkv_half *mix[NJ];
@@ -373,7 +454,8 @@ __global__ __launch_bounds__(DTHREADS) void lnmix_kernel(LnMixArgs a) {
     const int M0 = a.M[0];
     LnMixPro<U8, NJ> pro;
     auto pro_load = [&]() { pro.load(a.x, C, a.ln_w, a.ln_b, a.sx, mix, mat); };
-    auto pro_compute = [&]() { pro.compute(C, a.sx != nullptr, mix, xs, S, a.xx_tmp, red, a.maa_form != 0); };
+    auto pro_compute = [&]() { pro.compute(C, a.sx != nullptr, mix, xs, a.xx_tmp, red, sync, a.maa_form != 0); };
+    auto pro_finish = [&]() { LnMixPro<U8, NJ>::finish(C, S, red); };
     auto rowf = [&](int g, int, const uint8_t *&row, const h16 *&xv) {
         const int j = (NJ > 1 && g >= M0) ? 1 : 0;
         row = row_ptr<U8>(mat[j], j ? g - M0 : g);
@@ -402,9 +484,9 @@ __global__ __launch_bounds__(DTHREADS) void lnmix_kernel(LnMixArgs a) {
             ((rwkv_half *)a.out[j])[m] = f2h(t * t);
         }
     };
-    stream_rows<U8, G, 1, (G >= 4 ? 1 : 2), ScaleEpi>(M0 + (NJ > 1 ? a.M[1] : 0), (C * (U8 ? 1 : 2)) >> 4,
-                                                      pro_owner_wave(C >> 3), pro_load,
-                                                      pro_compute, rowf, epi_load, epi);
+    stream_rows<U8, G, 1, (G >= 4 ? 1 : 2), ScaleEpi, true>(M0 + (NJ > 1 ? a.M[1] : 0), (C * (U8 ? 1 : 2)) >> 4,
+                                                            pro_waves(C >> 3), sync, pro_load, pro_compute, pro_finish, rowf,
+                                                            epi_load, epi);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -439,6 +521,7 @@ template <bool U8, int U, int VPN, int OW>
 __global__ __launch_bounds__(DTHREADS) void vec_kernel(VecArgs a) {
     extern __shared__ __align__(16) unsigned char smem[];
     __shared__ float red[3 * DWAVES];
+    __shared__ unsigned sync[2];
     const int N = a.N;
     h16 *xs = (h16 *)smem;
     VecSums S;
@@ -478,8 +561,15 @@ __global__ __launch_bounds__(DTHREADS) void vec_kernel(VecArgs a) {
                 ((h16x8 *)xs)[xs_item<U8>(j8, nseg)] = o;
             }
         }
-        block_sum_1b<3>(acc, red);  // the barrier also publishes xs
-        if (U8) { S.s0 = acc[0]; S.s1 = acc[1]; S.s2 = acc[2]; }
+        if (U8) wave_sums_put<3>(acc, red);
+        pro_arrive(&sync[1]);
+    };
+    const int npw = pro_waves(min(N >> 3, 64 * OW));
+    auto pro_finish = [&]() {
+        if (!U8) return;
+        float acc[3];
+        wave_sums_get<3>(acc, red, npw);
+        S.s0 = acc[0]; S.s1 = acc[1]; S.s2 = acc[2];
     };
     auto rowf = [&](int m, int, const uint8_t *&row, const h16 *&xv) {
         row = row_ptr<U8>(a.mat, m);
@@ -511,7 +601,8 @@ __global__ __launch_bounds__(DTHREADS) void vec_kernel(VecArgs a) {
         }
         ((rwkv_half *)a.out)[m] = f2h(o);
     };
-    stream_rows<U8, 1, 1, U, VecEpi>(a.M, (N * (U8 ? 1 : 2)) >> 4, pro_owner_wave(min(N >> 3, 64 * OW)), pro_load, pro_compute, rowf, epi_load, epi);
+    stream_rows<U8, 1, 1, U, VecEpi, true>(a.M, (N * (U8 ? 1 : 2)) >> 4, npw, sync, pro_load, pro_compute, pro_finish, rowf, epi_load,
+                                           epi);
     // the token-shift state every workgroup of the previous launch read: committed after this workgroup's
     // rows, so that the copy's load -> store dependency does not sit in front of the weight stream
     if (blockIdx.x == 0 && a.commit_dst)
@@ -545,6 +636,7 @@ template <bool U8, int NM>
 __global__ __launch_bounds__(DTHREADS) void multi_vec_kernel(MultiVecArgs a) {
     extern __shared__ __align__(16) unsigned char smem[];
     __shared__ float red[3 * NM * DWAVES];
+    __shared__ unsigned sync[2];
     const int N = a.N, M = a.M;
     h16 *xs[NM];
 #pragma unroll
@@ -589,10 +681,15 @@ __global__ __launch_bounds__(DTHREADS) void multi_vec_kernel(MultiVecArgs a) {
             if (own) ((h16x8 *)xs[j])[xs_item<U8>(threadIdx.x, nseg)] = o;
         }
         if (own) ((h16x8 *)xs_x)[threadIdx.x] = px;
-        block_sum_1b<3 * NM>(acc, red);  // the barrier also publishes xs
-        if (U8)
+        if (U8) wave_sums_put<3 * NM>(acc, red);
+        pro_arrive(&sync[1]);
+    };
+    auto pro_finish = [&]() {
+        if (!U8) return;
+        float acc[3 * NM];
+        wave_sums_get<3 * NM>(acc, red, pro_waves(N >> 3));
 #pragma unroll
-            for (int j = 0; j < NM; ++j) { S[j].s0 = acc[3 * j]; S[j].s1 = acc[3 * j + 1]; S[j].s2 = acc[3 * j + 2]; }
+        for (int j = 0; j < NM; ++j) { S[j].s0 = acc[3 * j]; S[j].s1 = acc[3 * j + 1]; S[j].s2 = acc[3 * j + 2]; }
     };
     // a group is one output index m with its NM rows (row m of every matrix), so the matrix number is a
     // compile-time constant everywhere (an array of per-matrix fields indexed at run time would go to scratch)
@@ -622,7 +719,8 @@ __global__ __launch_bounds__(DTHREADS) void multi_vec_kernel(MultiVecArgs a) {
             a.out[k][m] = f2h(o);
         }
     };
-    stream_rows<U8, 1, NM, 2, Epi>(M, (N * (U8 ? 1 : 2)) >> 4, pro_owner_wave(N >> 3), pro_load, pro_compute, rowf, epi_load, epi);
+    stream_rows<U8, 1, NM, 2, Epi, true>(M, (N * (U8 ? 1 : 2)) >> 4, pro_waves(N >> 3), sync, pro_load, pro_compute, pro_finish, rowf,
+                                         epi_load, epi);
     if (a.xmat) {
         auto rowf2 = [&](int g, int, const uint8_t *&row, const h16 *&xv) {
             row = (const uint8_t *)(a.xmat + (size_t)g * N);
@@ -630,7 +728,7 @@ __global__ __launch_bounds__(DTHREADS) void multi_vec_kernel(MultiVecArgs a) {
         };
         auto epi_load2 = [&](int) { return NoEpi{}; };
         auto epi2 = [&](int g, const float (&d)[1], const NoEpi &) { a.xout[g] = f2h(tanhf(round_h(d[0]))); };
-        stream_rows<false, 1, 1, 2, NoEpi>(a.xm, (N * 2) >> 4, false, [] {}, [] {}, rowf2, epi_load2, epi2);
+        stream_rows<false, 1, 1, 2, NoEpi, false>(a.xm, (N * 2) >> 4, 0, nullptr, [] {}, [] {}, [] {}, rowf2, epi_load2, epi2);
     }
     if (blockIdx.x == 0 && a.commit_dst)
         for (int j8 = threadIdx.x; j8 < (a.commit_n >> 3); j8 += blockDim.x)

@@ -11,6 +11,9 @@
 // Bytes are widened two at a time to the fp16 values (1024 + b) with one v_perm_b32 and fed to
 // v_dot2_f32_f16 (fp32 accumulate); the 1024 offset is removed afterwards with S1 = sum xs[j]:
 //   sum xs[j] * (w + 0.5) = dot - 1023.5 * S1.
+// (Turning the pairs into (b + 0.5) with a packed fp16 subtraction, which is exact and saves the third sum
+// of every prologue, costs one more vector instruction per two weights in the streaming loop and was
+// measured 2.7 % slower per token.)
 #pragma once
 #include "common.h"
 
@@ -47,78 +50,6 @@ DEV float dot8_f16(u32x4 w, h16x8 x, float acc) {
     acc = __builtin_amdgcn_fdot2(__builtin_shufflevector(wh, wh, 4, 5), __builtin_shufflevector(x, x, 4, 5), acc, false);
     acc = __builtin_amdgcn_fdot2(__builtin_shufflevector(wh, wh, 6, 7), __builtin_shufflevector(x, x, 6, 7), acc, false);
     return acc;
-}
-
-// One wave: acc[r] += <row r, xs[r]> for R rows, every lane ends with the full sums.
-// u8: rows are N bytes, xs[r] in the split LDS layout above (nseg = N/16); rows may share one
-// activation vector (pass the same pointer: the LDS reads are then common) or have one each.
-// U = number of 16-byte segments per lane loaded before any is consumed (loads in flight = R*U).
-template <int R, int U>
-DEV void wave_rows_dot_u8(const uint8_t *const (&rows)[R], const h16 *const (&xs)[R], int nseg, float (&acc)[R]) {
-    const int lane = threadIdx.x & 63;
-    int s = lane;
-    // full batches: all 64 lanes have U segments
-    for (; s + 64 * (U - 1) < nseg; s += 64 * U) {
-        u32x4 wv[U][R];
-#pragma unroll
-        for (int u = 0; u < U; ++u)
-#pragma unroll
-            for (int r = 0; r < R; ++r)
-                wv[u][r] = __builtin_nontemporal_load((const u32x4 *)(rows[r] + 16 * (size_t)(s + 64 * u)));
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-#pragma unroll
-            for (int r = 0; r < R; ++r) {
-                const h16x8 *xlo = (const h16x8 *)xs[r];
-                const h16x8 x0 = xlo[s + 64 * u], x1 = xlo[nseg + s + 64 * u];
-                acc[r] = dot16_u8(wv[u][r], x0, x1, acc[r]);
-            }
-        }
-    }
-    for (; s < nseg; s += 64) {
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-            const h16x8 *xlo = (const h16x8 *)xs[r];
-            const h16x8 x0 = xlo[s], x1 = xlo[nseg + s];
-            u32x4 wv = __builtin_nontemporal_load((const u32x4 *)(rows[r] + 16 * (size_t)s));
-            acc[r] = dot16_u8(wv, x0, x1, acc[r]);
-        }
-    }
-#pragma unroll
-    for (int r = 0; r < R; ++r) acc[r] = wave_sum(acc[r]);
-}
-
-// fp16 rows: N halves per row, xs[r] stored linearly in LDS; segments are 8 values (16 bytes).
-template <int R, int U>
-DEV void wave_rows_dot_f16(const h16 *const (&rows)[R], const h16 *const (&xs)[R], int nseg8, float (&acc)[R]) {
-    const int lane = threadIdx.x & 63;
-    int s = lane;
-    for (; s + 64 * (U - 1) < nseg8; s += 64 * U) {
-        u32x4 wv[U][R];
-#pragma unroll
-        for (int u = 0; u < U; ++u)
-#pragma unroll
-            for (int r = 0; r < R; ++r)
-                wv[u][r] = __builtin_nontemporal_load((const u32x4 *)(rows[r] + 8 * (size_t)(s + 64 * u)));
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-#pragma unroll
-            for (int r = 0; r < R; ++r) {
-                const h16x8 x = ((const h16x8 *)xs[r])[s + 64 * u];
-                acc[r] = dot8_f16(wv[u][r], x, acc[r]);
-            }
-        }
-    }
-    for (; s < nseg8; s += 64) {
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-            const h16x8 x = ((const h16x8 *)xs[r])[s];
-            u32x4 wv = __builtin_nontemporal_load((const u32x4 *)(rows[r] + 8 * (size_t)s));
-            acc[r] = dot8_f16(wv, x, acc[r]);
-        }
-    }
-#pragma unroll
-    for (int r = 0; r < R; ++r) acc[r] = wave_sum(acc[r]);
 }
 
 // A register tile of weights: U 16-byte segments of R rows per lane.  Loading and consuming are

@@ -278,16 +278,16 @@ struct Att7Args {
 __global__ __launch_bounds__(DTHREADS) void att7_kernel(Att7Args a) {
     extern __shared__ __align__(16) unsigned char smem[];
     __shared__ float red[(2 + 3 * 6) * DWAVES];
+    __shared__ unsigned sync[2];
     const int C = a.C;
     h16 *xs[6];
     const rwkv_half *mix[6];
     MatDev nomat[6] = {};
 #pragma unroll
     for (int j = 0; j < 6; ++j) { xs[j] = (h16 *)smem + j * C; mix[j] = a.mix[j]; }
-    VecSums S[6];
     LnMixPro<false, 6> pro;
     auto pro_load = [&]() { pro.load(a.x, C, a.ln_w, a.ln_b, a.sx, mix, nomat); };
-    auto pro_compute = [&]() { pro.compute(C, true, mix, xs, S, a.xx_tmp, red, true); };
+    auto pro_compute = [&]() { pro.compute(C, true, mix, xs, a.xx_tmp, red, sync, true); };
     auto rowf = [&](int c, int k, const uint8_t *&row, const h16 *&xv) {
         row = row_ptr<false>(a.mat[k], c);
         xv = xs[k == 0 ? 0 : (k == 1 ? 2 : 3)];
@@ -298,7 +298,7 @@ __global__ __launch_bounds__(DTHREADS) void att7_kernel(Att7Args a) {
         for (int k = 0; k < 3; ++k) a.out[k][c] = f2h(d[k]);
     };
     const int nseg = (C * 2) >> 4;
-    stream_rows<false, 1, 3, 2, NoEpi>(C, nseg, pro_owner_wave(C >> 3), pro_load, pro_compute, rowf, epi_load, epi);
+    stream_rows<false, 1, 3, 2, NoEpi, true>(C, nseg, pro_waves(C >> 3), sync, pro_load, pro_compute, [] {}, rowf, epi_load, epi);
     // first LoRA stages: row g of the stacked matrix belongs to block j = w, a, v, g
     auto block_of = [&](int g) { return (g >= a.o_a ? 1 : 0) + (g >= a.o_v ? 1 : 0) + (g >= a.o_g ? 1 : 0); };
     auto rowf2 = [&](int g, int, const uint8_t *&row, const h16 *&xv) {
@@ -313,7 +313,7 @@ __global__ __launch_bounds__(DTHREADS) void att7_kernel(Att7Args a) {
         v = j == 0 ? tanhf(v) : (j == 3 ? sigmoidf_(v) : v);
         a.l1[g] = f2h(v);
     };
-    stream_rows<false, 1, 1, 2, NoEpi>(a.rtot, nseg, false, [] {}, [] {}, rowf2, epi_load, epi2);
+    stream_rows<false, 1, 1, 2, NoEpi, false>(a.rtot, nseg, 0, nullptr, [] {}, [] {}, [] {}, rowf2, epi_load, epi2);
 }
 
 struct Tmix7Args {
