@@ -33,9 +33,16 @@ def _np(t):
     return t.detach().cpu().numpy() if hasattr(t, 'detach') else np.asarray(t)
 
 
+def _acc(dtype):
+    """Accumulation / state type beside an activation type: fp32, or fp64 in the exact evaluation."""
+    return f64 if dtype == f64 else f32
+
+
 def _mm(a, b):
-    """``a @ b`` on tensors of one dtype: fp32 accumulation, result in that dtype."""
-    return (a.astype(f32) @ b.astype(f32)).astype(a.dtype)
+    """``a @ b`` on tensors of one dtype: fp32 accumulation, result in that dtype (fp64 throughout in the
+    exact evaluation)."""
+    F = _acc(a.dtype)
+    return (a.astype(F) @ b.astype(F)).astype(a.dtype)
 
 
 def _sigmoid(x):
@@ -65,15 +72,16 @@ def wkv7_matrix(S, r, w, k, v, kk, a):
     H = S.shape[0]
     N = C // H
     A = r.dtype
-    S = S.astype(f32).copy()
+    F = _acc(A)
+    S = S.astype(F).copy()
     y = np.empty((T, C), dtype=A)
     for t in range(T):
         vk = (v[t].reshape(H, N, 1) * k[t].reshape(H, 1, N)).astype(A)
         ab = ((-kk[t]).reshape(H, N, 1) * (kk[t] * a[t]).astype(A).reshape(H, 1, N)).astype(A)
-        S = (S * w[t].reshape(H, 1, N) + np.einsum('him,hmj->hij', S, ab.astype(f32), dtype=f32)
-             + vk.astype(f32)).astype(f32)
-        y[t] = np.einsum('hij,hj->hi', S.astype(A).astype(f32), r[t].reshape(H, N).astype(f32),
-                         dtype=f32).astype(A).reshape(C)
+        S = (S * w[t].reshape(H, 1, N) + np.einsum('him,hmj->hij', S, ab.astype(F), dtype=F)
+             + vk.astype(F)).astype(F)
+        y[t] = np.einsum('hij,hj->hi', S.astype(A).astype(F), r[t].reshape(H, N).astype(F),
+                         dtype=F).astype(A).reshape(C)
     return y, S
 
 
@@ -84,24 +92,30 @@ def wkv7_kernel(S, r, w_log, k, v, a, b):
     T, C = r.shape
     H = S.shape[0]
     N = C // H
-    S = S.astype(f32).copy()
+    F = _acc(r.dtype)
+    S = S.astype(F).copy()
     y = np.empty((T, C), dtype=r.dtype)
     for t in range(T):
-        r_, k_, v_, a_, b_ = (x[t].astype(f32).reshape(H, N) for x in (r, k, v, a, b))
-        dec = np.exp(-np.exp(w_log[t].astype(f32))).reshape(H, 1, N)
-        sa = np.einsum('hij,hj->hi', S, a_, dtype=f32)
-        S = (S * dec + v_[:, :, None] * k_[:, None, :] + sa[:, :, None] * b_[:, None, :]).astype(f32)
-        y[t] = np.einsum('hij,hj->hi', S, r_, dtype=f32).reshape(C).astype(r.dtype)
+        r_, k_, v_, a_, b_ = (x[t].astype(F).reshape(H, N) for x in (r, k, v, a, b))
+        dec = np.exp(-np.exp(w_log[t].astype(F))).reshape(H, 1, N)
+        sa = np.einsum('hij,hj->hi', S, a_, dtype=F)
+        S = (S * dec + v_[:, :, None] * k_[:, None, :] + sa[:, :, None] * b_[:, None, :]).astype(F)
+        y[t] = np.einsum('hij,hj->hi', S, r_, dtype=F).reshape(C).astype(r.dtype)
     return y, S
 
 
 class OracleRWKV7:
-    def __init__(self, checkpoint, strategy, kernel_form=False, deep_embed=False):
+    def __init__(self, checkpoint, strategy, kernel_form=False, deep_embed=False, exact=False):
+        """exact=True: the weights are converted as ``strategy`` says (the same stored fp16 / fp32 values,
+        the embedding table normalised and rounded as the loader does), then every operation of the
+        forward pass runs in fp64 with no rounding: the value that both half-precision evaluations
+        approximate."""
         dev, dt = strategy.split(' ')                                 # model.py:234-243
         if dt not in ('fp16', 'fp32'):
             raise ValueError("oracle supports '<device> fp16' and '<device> fp32' for RWKV-7")
         A = self.atype = f16 if dt == 'fp16' else f32
         self.kernel_form = kernel_form
+        self.exact = bool(exact)
         z = {}
         src = {k: _np(v) for k, v in checkpoint.items()}
         self.n_head, self.head_size = src['blocks.0.att.r_k'].shape    # model.py:247
@@ -123,6 +137,9 @@ class OracleRWKV7:
             for i in range(self.n_layer):
                 p = f'blocks.{i}.ffn.'
                 z[p + 's_emb.weight'] = z[p + 's_emb.weight'] + _mm(z['emb.weight'], z[p + 's_emb_x.weight'].T)
+        if self.exact:
+            z = {k: t.astype(f64) for k, t in z.items()}
+            self.atype = f64
         self.z = z
 
     def generate_zero_state(self):
@@ -130,7 +147,7 @@ class OracleRWKV7:
         C, H, N = self.n_embd, self.n_head, self.head_size
         st = []
         for _ in range(self.n_layer):
-            st += [np.zeros(C, self.atype), np.zeros((H, N, N), f32), np.zeros(C, self.atype)]
+            st += [np.zeros(C, self.atype), np.zeros((H, N, N), _acc(self.atype)), np.zeros(C, self.atype)]
         return st
 
     # ------------------------------------------------------------------ blocks
@@ -161,11 +178,12 @@ class OracleRWKV7:
             y, S = wkv7_kernel(S, r, w_log, k, v, -kk, (kk * a).astype(A))
         else:
             # model.py:507, 562
-            dec = np.exp(f32(-0.606531) * _sigmoid(zw.astype(f32))).astype(f32)
+            F = _acc(A)
+            dec = np.exp(F(-0.606531) * _sigmoid(zw.astype(F))).astype(F)
             y, S = wkv7_matrix(S, r, dec, k, v, kk, a)
         y = ops.group_norm(y, H, z[p + 'ln_x.weight'], z[p + 'ln_x.bias'])  # eps 64e-5 (model.py:514)
         T, C = y.shape
-        rk = (r * k * z[p + 'r_k']).reshape(T, H, -1).astype(f32).sum(axis=-1, keepdims=True).astype(A)
+        rk = (r * k * z[p + 'r_k']).reshape(T, H, -1).astype(_acc(A)).sum(axis=-1, keepdims=True).astype(A)
         y = y + (rk * v.reshape(T, H, -1)).reshape(T, C)
         return _mm(y * g, z[p + 'output.weight']), x[-1], S, v_first
 
@@ -180,7 +198,8 @@ class OracleRWKV7:
             T = x.shape[0]
             E = z[p + 's_emb.weight'][np.asarray(toks, dtype=np.int64)].reshape(T, 32, 32)
             sv = _mm(x, z[p + 's1'])                                                     # [T, 32]
-            ss = np.einsum('ti,tij->tj', sv.astype(f32), E.astype(f32)).astype(x.dtype)  # [T, 32]
+            F = _acc(x.dtype)
+            ss = np.einsum('ti,tij->tj', sv.astype(F), E.astype(F)).astype(x.dtype)        # [T, 32]
             k = k * (_mm(ss, z[p + 's2']) + z[p + 's0'])
         return _mm(k, z[p + 'value.weight']), x[-1]
 

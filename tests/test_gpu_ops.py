@@ -67,7 +67,7 @@ def test_repack_round_trip():
 
 # ------------------------------------------------------------------------------ mm8_one / mm8_seq
 MM8_SHAPES = [(768, 768), (768, 3072), (3072, 768), (768, 50277), (2560, 2560), (4096, 4096), (4096, 16384),
-              (16384, 4096), (5120, 20480)]
+              (16384, 4096), (5120, 20480), (4096, 65536)]
 
 
 def _mm8_case(N, M, B, seed):
@@ -117,6 +117,26 @@ def test_mm8_seq(N, M, B):
     # one-token mode and sequence mode agree on the same row (up to fp16 rounding)
     y1 = ops.cuda_mm8_one(N, M, xt[B - 1].contiguous(), q, mx, rx, my, ry)
     assert np.abs(y1.cpu().numpy().astype(np.float64) - y[B - 1].cpu().numpy()).max() <= np.abs(ref).max() * 2 ** -9
+
+
+@pytest.mark.parametrize("N,M", [(5120, 20480), (20480, 5120), (5120, 5120)])
+def test_mm8_seq_14b_call_length(N, M):
+    """The launches of the 14B configuration at its own call length (1024 rows; BASELINE.json configs[4]): 320 large
+    tiles = 1.25 rounds over the chip for the wide product, K split for the deep one.  Checked against the fp64
+    evaluation on 40 rows that include both ends of every 128- and 256-row tile boundary, all columns."""
+    ops = _ops()
+    B = 1024
+    w, (q, mx, rx, my, ry) = _quantized(N, M, N + M + B)
+    x = _rng(N + M + B + 1).standard_normal((B, N)).astype(np.float16)
+    rows = sorted({0, 1, 63, 64, 127, 128, 129, 255, 256, 257, 383, 384, 511, 512, 513, 639, 640, 767, 768, 769, 895,
+                   896, 1000, 1022, 1023} | {int(r) for r in _rng(7).integers(0, B, 15)})
+    ref = x[rows].astype(np.float64) @ oquant.dequant_f64(q, mx, rx, my, ry)
+    dev = [_to_dev_ic(q)] + [torch.from_numpy(a).to(DEV) for a in (mx, rx, my, ry)]
+    y = ops.cuda_mm8_seq(B, N, M, torch.from_numpy(x).to(DEV), *dev)
+    assert y.dtype == torch.float16 and y.shape == (B, M)
+    scale = np.sqrt(np.mean(ref ** 2))
+    d = np.abs(y[rows].cpu().numpy().astype(np.float64) - ref)
+    assert d.max() <= 1e-3 * scale + np.abs(ref).max() * 2 ** -10, (d.max(), scale)
 
 
 def test_mm8_seq_timing_aid_leaves_the_product():

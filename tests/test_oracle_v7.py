@@ -47,6 +47,27 @@ def test_v7_forward_matches_reference(strat, kernel_form, de):
         assert np.abs(outs[j] - g["full_logits"][b - 1]).max() <= 4 * TOL[strat]
 
 
+@pytest.mark.parametrize("kernel_form", [False, True])
+def test_v7_exact_mode_is_the_fp32_model_without_rounding(kernel_form):
+    """exact=True evaluates the converted model in fp64.  Under 'cpu fp32' the stored weights are the checkpoint's own,
+    so the fp64 evaluation must agree with the fp32 one (pinned above by the reference's run) to fp32 rounding; under
+    'cpu fp16' (weights rounded to fp16, arithmetic exact) it must lie within the fp16 tolerance of the reference's
+    half-precision logits and closer to the fp32 logits than that all-half run is."""
+    g32 = dict(np.load(os.path.join(G, "e2e_v7_cpu_fp32.npz")))
+    g16 = dict(np.load(os.path.join(G, "e2e_v7_cpu_fp16.npz")))
+    ck = synth.make_checkpoint_v7(seed=CKPT_SEED, **TINY7)
+    toks = [int(t) for t in g32["tokens"]]
+    e32, st = OracleRWKV7(ck, "cpu fp32", kernel_form=kernel_form, exact=True).forward(toks, None, full_output=True)
+    assert e32.dtype == np.float64 and st[1].dtype == np.float64
+    assert np.abs(e32 - g32["full_logits"]).max() <= TOL["cpu fp32"]
+    for i, s in enumerate(st):
+        assert np.abs(s - g32[f"full_state_{i}"]).max() <= TOL["cpu fp32"], i
+    e16, _ = OracleRWKV7(ck, "cpu fp16", kernel_form=kernel_form, exact=True).forward(toks, None, full_output=True)
+    assert np.abs(e16 - g16["full_logits"]).max() <= TOL["cpu fp16"]
+    # only the weights are rounded to fp16 in e16: it is closer to the fp32 model than the all-fp16 run
+    assert np.abs(e16 - g32["full_logits"]).mean() < np.abs(g16["full_logits"] - g32["full_logits"]).mean()
+
+
 def test_deep_embed_with_a_unit_gate_is_the_plain_model():
     """s2 = 0 and s0 = 1 make the DeepEmbed gate 1 for every token: the logits must equal the plain model's."""
     ck = synth.make_checkpoint_v7(seed=5, deep_embed=True, **TINY7)
