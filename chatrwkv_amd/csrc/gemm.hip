@@ -23,6 +23,17 @@
 #include <cstdlib>
 #include <mutex>
 
+// Set-up that must run once per device (function attributes belong to the current device's copy of a kernel).
+struct PerDeviceOnce {
+    bool done[64] = {};
+    // the slot of the current device, or nullptr when the device cannot be read (the caller then repeats the set-up)
+    bool *slot() {
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return nullptr;
+        return &done[dev];
+    }
+};
+
 namespace {
 
 constexpr int BK = 64;  // halves per LDS row
@@ -740,15 +751,16 @@ __global__ __launch_bounds__(512) void gemm_dma_group_kernel(int T, int N, GemmG
 template <bool W_U8, int TM, int TN>
 int launch_dma_group(const GemmGroup &g, int n, int64_t T, int64_t N, int64_t grid_x, int ks, hipStream_t st) {
     constexpr size_t lds = DmaCfg<W_U8, TM, TN>::LDS;
-    static bool attr_done = false;
-    if (!attr_done) {
+    static PerDeviceOnce once;
+    bool *attr_done = once.slot();
+    if (!attr_done || !*attr_done) {
         hipError_t e = hipFuncSetAttribute((const void *)gemm_dma_group_kernel<W_U8, false, TM, TN>,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e == hipSuccess)
             e = hipFuncSetAttribute((const void *)gemm_dma_group_kernel<W_U8, true, TM, TN>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                     (int)lds);
         if (e != hipSuccess) return (int)e;
-        attr_done = true;
+        if (attr_done) *attr_done = true;
     }
     const dim3 grid((unsigned)grid_x, (unsigned)n, (unsigned)ks);
     if (ks > 1) hipLaunchKernelGGL((gemm_dma_group_kernel<W_U8, true, TM, TN>), grid, dim3(512), lds, st, (int)T, (int)N, g);
@@ -993,12 +1005,13 @@ template <bool W_U8, int BT, int BM, int WT, int WM, int PF>
 int launch_cfg(int64_t T, int64_t N, int64_t M, const rwkv_half *A, int64_t lda, const void *W, int64_t ldw, void *Y,
                int64_t ldy, const GemmEpi &ep, hipStream_t st) {
     constexpr size_t lds = 2 * (size_t)(BT + BM) * BK * sizeof(h16);
-    static bool attr_done = false;
-    if (lds > 64 * 1024 && !attr_done) {
+    static PerDeviceOnce once;
+    bool *attr_done = once.slot();
+    if (lds > 64 * 1024 && (!attr_done || !*attr_done)) {
         hipError_t e = hipFuncSetAttribute((const void *)gemm_kernel<W_U8, BT, BM, WT, WM, PF, false>,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return (int)e;
-        attr_done = true;
+        if (attr_done) *attr_done = true;
     }
     const int64_t tiles = ((T + BT - 1) / BT) * ((M + BM - 1) / BM);
     // Too few tiles to fill the chip (short prompts, narrow matrices): split the contraction over KS
@@ -1079,13 +1092,14 @@ template <bool W_U8, int TM, int TN>
 int launch_dma(int64_t T, int64_t N, int64_t M, const rwkv_half *A, int64_t lda, const void *W, int64_t ldw, void *Y,
                int64_t ldy, const GemmEpi &ep, hipStream_t st) {
     constexpr size_t lds = DmaCfg<W_U8, TM, TN>::LDS;
-    static bool attr_done = false;
-    if (!attr_done) {
+    static PerDeviceOnce once;
+    bool *attr_done = once.slot();
+    if (!attr_done || !*attr_done) {
         hipError_t e = hipFuncSetAttribute((const void *)gemm_dma_kernel<W_U8, false, TM, TN>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e == hipSuccess)
             e = hipFuncSetAttribute((const void *)gemm_dma_kernel<W_U8, true, TM, TN>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return (int)e;
-        attr_done = true;
+        if (attr_done) *attr_done = true;
     }
     if (!dma_ok(W_U8, N, M, A, lda, W, ldw, Y, ldy, ep)) return RWKV_E_LAYOUT;
     const int64_t tiles = ((T + TM - 1) / TM) * ((M + TN - 1) / TN);
@@ -1401,4 +1415,23 @@ extern "C" int rwkv_gemm_f16(int64_t B, int64_t N, int64_t M, const rwkv_half *a
     GemmEpi ep{};
     ep.act = ACT_NONE; ep.out_scale = 1.f; ep.out_dtype = c_dtype; ep.raw_f32 = (c_dtype == RWKV_DT_F32);
     return gemm_launch(false, B, N, M, a, a_stride, b, b_stride_m, c, c_stride, ep, st);
+}
+
+extern "C" int rwkv_gemm_f16_batched(int64_t batch, int64_t B, int64_t N, int64_t M, const rwkv_half *a, int64_t a_stride,
+                                     int64_t a_batch_stride, const rwkv_half *b, int64_t b_stride_n, int64_t b_stride_m,
+                                     int64_t b_batch_stride, void *c, int64_t c_stride, int64_t c_batch_stride, int c_dtype,
+                                     void *stream) {
+    if (batch <= 0 || batch > (1 << 20)) return RWKV_E_SHAPE;
+    if (!a || !b || !c) return RWKV_E_NULL;
+    if (c_dtype != RWKV_DT_F16 && c_dtype != RWKV_DT_F32) return RWKV_E_DTYPE;
+    // every product of the batch must itself be acceptable: 16-byte aligned operands
+    if ((a_batch_stride & 7) || (b_batch_stride & 7) || a_batch_stride < 0 || b_batch_stride < 0 || c_batch_stride < 0)
+        return RWKV_E_LAYOUT;
+    const size_t csz = c_dtype == RWKV_DT_F16 ? 2 : 4;
+    for (int64_t i = 0; i < batch; ++i) {
+        const int rc = rwkv_gemm_f16(B, N, M, a + i * a_batch_stride, a_stride, b + i * b_batch_stride, b_stride_n, b_stride_m,
+                                     (char *)c + (size_t)(i * c_batch_stride) * csz, c_stride, c_dtype, stream);
+        if (rc) return rc;
+    }
+    return RWKV_OK;
 }

@@ -376,21 +376,38 @@ int run_gemm(const rwkv_mat &m, bool u8, int64_t T, const rwkv_half *A, const fl
 // to fill the chip alone: k / v / r of the time mix and r / k of the channel mix run side by side.
 }  // namespace
 
+namespace {
+// The table of side-stream sets: one per (device, caller stream) pair, at most 32 at a time.  A set whose caller
+// stream has been given back (rwkv_release_stream) is taken over, with its streams and events, by the next new pair
+// on the same device.
+struct SideSlot { int dev; hipStream_t caller; bool bound; SideStreams ss; };
+constexpr int MAX_SIDE_SLOTS = 32;
+SideSlot g_side_slots[MAX_SIDE_SLOTS];
+int g_n_side_slots = 0;
+std::mutex g_side_mu;
+}  // namespace
+
 SideStreams *side_streams(hipStream_t caller) {
-    struct Slot { int dev; hipStream_t caller; SideStreams ss; };
-    constexpr int MAX_SLOTS = 32;
-    static Slot slots[MAX_SLOTS];
-    static int n_slots = 0;
-    static std::mutex mu;
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess) return nullptr;
-    std::lock_guard<std::mutex> lock(mu);
-    for (int i = 0; i < n_slots; ++i)
-        if (slots[i].dev == dev && slots[i].caller == caller) return slots[i].ss.ok ? &slots[i].ss : nullptr;
-    if (n_slots == MAX_SLOTS) return nullptr;      // more caller streams than slots: those run without side streams
-    Slot &sl = slots[n_slots++];
+    std::lock_guard<std::mutex> lock(g_side_mu);
+    SideSlot *spare = nullptr;
+    for (int i = 0; i < g_n_side_slots; ++i) {
+        SideSlot &sl = g_side_slots[i];
+        if (sl.dev != dev) continue;
+        if (sl.bound && sl.caller == caller) return sl.ss.ok ? &sl.ss : nullptr;
+        if (!sl.bound && sl.ss.ok && !spare) spare = &sl;
+    }
+    if (spare) {
+        spare->caller = caller;
+        spare->bound = true;
+        return &spare->ss;
+    }
+    if (g_n_side_slots == MAX_SIDE_SLOTS) return nullptr;   // more caller streams than slots: those run without side streams
+    SideSlot &sl = g_side_slots[g_n_side_slots++];
     sl.dev = dev;
     sl.caller = caller;
+    sl.bound = true;
     SideStreams &ss = sl.ss;
     ss.ok = hipStreamCreateWithFlags(&ss.s[0], hipStreamNonBlocking) == hipSuccess &&
             hipStreamCreateWithFlags(&ss.s[1], hipStreamNonBlocking) == hipSuccess &&
@@ -398,6 +415,21 @@ SideStreams *side_streams(hipStream_t caller) {
             hipEventCreateWithFlags(&ss.join[0], hipEventDisableTiming) == hipSuccess &&
             hipEventCreateWithFlags(&ss.join[1], hipEventDisableTiming) == hipSuccess;
     return ss.ok ? &ss : nullptr;
+}
+
+extern "C" int rwkv_release_stream(void *stream) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    std::lock_guard<std::mutex> lock(g_side_mu);
+    for (int i = 0; i < g_n_side_slots; ++i) {
+        SideSlot &sl = g_side_slots[i];
+        if (sl.dev == dev && sl.bound && sl.caller == (hipStream_t)stream) {
+            sl.bound = false;
+            sl.caller = nullptr;
+        }
+    }
+    return RWKV_OK;
 }
 
 // after fork, work launched on side stream j sees everything queued on `st` so far
@@ -533,7 +565,7 @@ extern "C" int rwkv_v4_forward_seq(const rwkv_v4_model *m, const rwkv_v4_layer_s
         e.act = ACT_SIGMOID;
         // the receptance product beside the key product: where neither would split K, and in calls of three row tiles
         // (257 .. 384 tokens: +4 % at n_embd 4096; slower at 256 and from 385 on)
-        ForkScope par2(ss, st, 1, !dma_seq && ((T / 128) * (C / 128) > 128 || ((T + 127) / 128 == 3 && C >= 2048)));
+        ForkScope par2(ss, st, 1, !dma_seq && ((T / 128) * (C / 128) > 128 || ((T + 127) / 128 == 3 && C == 4096)));
         float *sk2 = par2 ? nullptr : ws.splitk;
         if (T <= 128 && !(C & 127) && !(F & 127)) {
             // short calls: receptance and key in one grouped launch

@@ -38,6 +38,8 @@ SIGNATURES = {
     "rwkv_mm8_seq_time_kernel": (_int, [_i64, _i64, _i64, _vp, _i64, _vp, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _i64, _vp, _sz, _vp, _int, _vp]),
     "rwkv_mm8_seq_f16_static": (_int, [_i64, _i64, _i64, _vp, _i64, _vp, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _i64, _vp]),
     "rwkv_gemm_f16": (_int, [_i64, _i64, _i64, _vp, _i64, _vp, _i64, _i64, _vp, _i64, _int, _vp]),
+    "rwkv_gemm_f16_batched": (_int, [_i64, _i64, _i64, _i64, _vp, _i64, _i64, _vp, _i64, _i64, _i64, _vp, _i64, _i64, _int, _vp]),
+    "rwkv_release_stream": (_int, [_vp]),
     "rwkv_wkv4_forward": (_int, [_i64, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _int, _vp, _vp, _vp, _vp]),
     "rwkv_wkv5_forward": (_int, [_i64, _i64, _i64, _i64, _vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "rwkv_wkv6_forward": (_int, [_i64, _i64, _i64, _i64, _vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),

@@ -42,6 +42,19 @@ def _ptr(t):
     return ctypes.c_void_p(t.data_ptr())
 
 
+def _load_checkpoint(path):
+    """The checkpoint dict of ``path`` on the CPU, read without executing anything from the file
+    (``weights_only=True``).  Memory-mapped where the file allows it; files in torch's older, non-zip
+    serialization, which the reference's plain ``torch.load`` (model.py:641) accepts, cannot be mapped and are
+    read whole."""
+    try:
+        return torch.load(path, map_location='cpu', weights_only=True, mmap=True)
+    except RuntimeError as e:
+        if 'mmap' not in str(e):
+            raise
+        return torch.load(path, map_location='cpu', weights_only=True)
+
+
 class RWKV:
     def __init__(self, model, strategy, verbose=True, convert_and_save_and_exit=None):
         prxxx = (lambda *a, **k: print(*a, **k)) if verbose else (lambda *a, **k: None)
@@ -62,7 +75,7 @@ class RWKV:
             if not args.MODEL_NAME.endswith('.pth'):
                 args.MODEL_NAME += '.pth'
             prxxx(f'Loading {args.MODEL_NAME} ...')
-            w = torch.load(args.MODEL_NAME, map_location='cpu', weights_only=True, mmap=True)
+            w = _load_checkpoint(args.MODEL_NAME)
 
         converted = '_strategy' in w                                  # model.py:646-656
         if converted:

@@ -10,6 +10,8 @@ reference's device layout (strides (M, 1)) once, with the repack kernel.
 Every function requires tensors on a ROCm device and raises if the native library is
 missing or rejects the call; nothing here computes with PyTorch.
 """
+import weakref
+
 import torch
 
 from . import lib as _lib
@@ -44,6 +46,27 @@ def to_input_contiguous(w):
         w = w.contiguous()
     _lib.check(fn(N, M, _ptr(w), w.stride(0), w.stride(1), _ptr(store), 1, N, _stream()), "repack")
     return store.t()
+
+
+# Weight matrices that arrive in the reference's own device layout (output index contiguous: what
+# ``w[x].contiguous()`` of model.py:860 leaves, asserted at cuda/wrapper.cpp:56) are repacked once per tensor and the
+# copy is kept for as long as the tensor lives, so that a binding written against the reference's converted checkpoint
+# works unchanged; an in-place change of the tensor (its version counter) repacks it again.
+_repacked = {}
+
+
+def _kernel_layout(w):
+    """``w`` [N, M] as the kernels read it (strides (1, ld)): itself, or its cached repacked copy."""
+    N = w.shape[0]
+    if w.stride(0) == 1 and w.stride(1) >= N:
+        return w
+    key = id(w)
+    hit = _repacked.get(key)
+    if hit is not None and hit[0]() is w and hit[1] == w._version and hit[2] == w.data_ptr():
+        return hit[3]
+    ic = to_input_contiguous(w)
+    _repacked[key] = (weakref.ref(w, lambda _, k=key: _repacked.pop(k, None)), w._version, w.data_ptr(), ic)
+    return ic
 
 
 def quantize_u8(w, scale_dtype=torch.float16, input_contiguous=True):
@@ -82,6 +105,7 @@ def cuda_mm8_one(N, M, x, w, mx, rx, my, ry):
     assert w.dtype == torch.uint8
     assert x.shape == (N,) and w.shape == (N, M)
     assert rx.shape == mx.shape == (M,) and ry.shape == my.shape == (N, 1)
+    w = _kernel_layout(w)
     y = torch.empty((M,), device=w.device, dtype=torch.float16)
     rc = _lib.load().rwkv_mm8_one_f16(N, M, _ptr(x.contiguous()), _ptr(w), w.stride(0), w.stride(1), _ptr(mx), _ptr(rx),
                                       _ptr(my), _ptr(ry), _ptr(y), F16, _stream())
@@ -92,6 +116,7 @@ def cuda_mm8_one(N, M, x, w, mx, rx, my, ry):
 def mm8_one_f32(N, M, x, w, mx, rx, my, ry):
     """The raw fp32 sums of torch.ops.rwkv.mm8_one (cuda/wrapper.cpp:84) before model.py:86 rounds them."""
     _need_cuda(x, w)
+    w = _kernel_layout(w)
     y = torch.empty((M,), device=w.device, dtype=torch.float32)
     rc = _lib.load().rwkv_mm8_one_f16(N, M, _ptr(x.contiguous()), _ptr(w), w.stride(0), w.stride(1), _ptr(mx), _ptr(rx),
                                       _ptr(my), _ptr(ry), _ptr(y), F32, _stream())
@@ -108,6 +133,7 @@ def cuda_mm8_seq(B, N, M, x, w, mx, rx, my, ry):
     assert rx.shape == mx.shape == (M,) and ry.shape == my.shape == (N, 1)
     if x.stride(1) != 1:
         x = x.contiguous()
+    w = _kernel_layout(w)
     L = _lib.load()
     y = torch.empty((B, M), device=w.device, dtype=torch.float16)
     nbytes = L.rwkv_mm8_seq_workspace(B, N)
@@ -126,26 +152,39 @@ def mm8(x, w, mx, rx, my, ry):
 
 
 def _input_contiguous_f16(b):
-    """A 2-D fp16 matrix [N, M] in the layout the kernels stream (strides (1, N)); copies only if it is not."""
-    if b.stride(0) == 1 and b.stride(1) >= b.shape[0] and b.stride(1) % 8 == 0:
+    """A fp16 matrix [N, M], or a batch of them [batch, N, M], in the layout the kernels stream (strides (1, N) within a
+    matrix); copies only if it is not."""
+    if b.stride(-2) == 1 and b.stride(-1) >= b.shape[-2] and b.stride(-1) % 8 == 0 and (b.dim() == 2 or b.stride(0) % 8 == 0):
         return b
-    return b.t().contiguous().t()
+    return b.transpose(-1, -2).contiguous().transpose(-1, -2)
 
 
 def matmul_float(a, b, output_dtype=None):
     """model.py:144-161 (gemm_fp16_cublas): fp16 x fp16, fp32 accumulation, output written
     directly in ``output_dtype`` (fp16 or fp32).  1-D ``a`` gives a 1-D result; 3-D ``a`` and ``b`` are a
-    batch of products (cuda/gemm_fp16_cublas.cpp:61-75), run one after the other."""
+    batch of products (cuda/gemm_fp16_cublas.cpp:61-75): one call of rwkv_gemm_f16_batched."""
     _need_cuda(a, b)
     if output_dtype is None:
         output_dtype = a.dtype
     assert a.dtype == b.dtype == torch.float16
     assert output_dtype in (torch.float16, torch.float32)
     if a.dim() == 3:
-        assert b.dim() == 3 and a.shape[0] == b.shape[0]
-        c = torch.empty((a.shape[0], a.shape[1], b.shape[-1]), dtype=output_dtype, device=a.device)
-        for i in range(a.shape[0]):
-            c[i] = matmul_float(a[i], b[i], output_dtype=output_dtype)
+        assert b.dim() == 3 and a.shape[0] == b.shape[0] and a.shape[2] == b.shape[1]
+        step = 8 if a.shape[1] == 1 else 64          # the contraction kernel's K step (8 for one-row products)
+        if a.shape[2] % step:
+            pad = step - a.shape[2] % step
+            a = torch.nn.functional.pad(a, (0, pad))
+            b = torch.nn.functional.pad(b, (0, 0, 0, pad))
+        if a.stride(2) != 1 or a.stride(1) % 8 or a.stride(0) % 8:
+            a = a.contiguous()
+        b = _input_contiguous_f16(b)
+        nb, B, N = a.shape
+        M = b.shape[2]
+        c = torch.empty((nb, B, M), dtype=output_dtype, device=a.device)
+        rc = _lib.load().rwkv_gemm_f16_batched(nb, B, N, M, _ptr(a), a.stride(1), a.stride(0), _ptr(b), b.stride(1),
+                                               b.stride(2), b.stride(0), _ptr(c), c.stride(1), c.stride(0),
+                                               F16 if output_dtype == torch.float16 else F32, _stream())
+        _lib.check(rc, "rwkv_gemm_f16_batched")
         return c
     one = a.dim() == 1
     a2 = a.unsqueeze(0) if one else a

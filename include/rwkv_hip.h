@@ -98,13 +98,26 @@ int rwkv_mm8_seq_f16(int64_t B, int64_t N, int64_t M, const rwkv_half *x, int64_
  * otherwise RWKV_E_SCRATCH and nothing is enqueued.  Same kernels and arguments as rwkv_mm8_seq_f16; the K split
  * is chosen within 16 MiB of slabs instead of 64, so a result can differ from rwkv_mm8_seq_f16's in the order of
  * its fp32 sums (at most one fp16 rounding step).  All calls on one GPU share that GPU's array: calls that may
- * overlap there (different streams, different host threads) race; calls on one stream are safe. */
+ * overlap there (different streams, different host threads) race; calls on one stream are safe.
+ * The first call on a device does host-side set-up (the address of the built-in array, kernel attributes) that
+ * must not happen while a stream is capturing: make one call outside capture first (any valid size); every later
+ * call only enqueues kernels and may be captured into a graph and replayed. */
 size_t rwkv_mm8_seq_static_max_elems(void);
 size_t rwkv_mm8_seq_static_max_rows(void);
 int rwkv_mm8_seq_f16_static(int64_t B, int64_t N, int64_t M, const rwkv_half *x, int64_t x_stride,
                             const uint8_t *w, int64_t w_stride_n, int64_t w_stride_m,
                             const rwkv_half *mx, const rwkv_half *rx, const rwkv_half *my, const rwkv_half *ry,
                             rwkv_half *y, int64_t y_stride, void *stream);
+
+/* Side streams.  Sequence calls of 256 tokens or more may run independent products of a layer on two extra streams
+ * (default priority) beside the caller's; the library creates one such pair, with three events, for each (device,
+ * caller stream) pair on its first use and keeps it until the process ends.  At most 32 pairs exist at a time: calls
+ * on a further stream run every product on the caller's stream (same results, a few per cent slower).  A caller that
+ * is about to destroy a stream hands its pair back with rwkv_release_stream(stream) (current device), after the
+ * stream's work has completed; the next new stream takes the pair over.  Without that call a destroyed stream's pair
+ * stays bound to its handle value.  No counterpart in the reference, whose launches use the legacy default stream
+ * only (cuda/operators.cu:57, 111, 151). */
+int rwkv_release_stream(void *stream);
 
 /* gemm_fp16: c[B, M] = a[B, N] @ b[N, M], fp16 operands, fp32 accumulation, c written
  * directly as fp16 or fp32 (c_dtype) with no intermediate fp16 rounding.  Replaces
@@ -113,6 +126,15 @@ int rwkv_mm8_seq_f16_static(int64_t B, int64_t N, int64_t M, const rwkv_half *x,
 int rwkv_gemm_f16(int64_t B, int64_t N, int64_t M, const rwkv_half *a, int64_t a_stride,
                   const rwkv_half *b, int64_t b_stride_n, int64_t b_stride_m,
                   void *c, int64_t c_stride, int c_dtype, void *stream);
+
+/* The batched form of gemm_fp16: c[i] = a[i] @ b[i] for i < batch, operand i at a + i * a_batch_stride (elements;
+ * likewise b, c).  Replaces the 3-D case of torch.ops.rwkv.gemm_fp16_cublas (cublasGemmStridedBatchedEx,
+ * cuda/gemm_fp16_cublas.cpp:61-75; the caller is the RWKV-6 mixing LoRA `bmm` of model.py:1269, 1310).  Every product
+ * must satisfy rwkv_gemm_f16's layout rules; the products are queued on `stream` one after the other. */
+int rwkv_gemm_f16_batched(int64_t batch, int64_t B, int64_t N, int64_t M, const rwkv_half *a, int64_t a_stride,
+                          int64_t a_batch_stride, const rwkv_half *b, int64_t b_stride_n, int64_t b_stride_m,
+                          int64_t b_batch_stride, void *c, int64_t c_stride, int64_t c_batch_stride, int c_dtype,
+                          void *stream);
 
 /* ---------------------------------------------------------------------------------------
  * wkv_forward: RWKV-4 WKV recurrence over T tokens with running-maximum tracking.

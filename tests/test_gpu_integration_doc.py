@@ -51,6 +51,12 @@ def test_documented_binding_runs_and_agrees():
     ys = ns["cuda_mm8_seq"](B, N, M, xt, qd, dmx, drx, dmy, dry)
     assert ys.dtype == torch.float16 and tuple(ys.shape) == (B, M)
     assert np.abs(ys.cpu().numpy().astype(np.float64) - ref).max() <= tol
+    # the reference's own device layout (model.py:860: contiguous [in, out]): the binding repacks it once per tensor
+    q_ref = torch.from_numpy(q).to(DEV)
+    assert q_ref.stride() == (M, 1)
+    assert torch.equal(ns["cuda_mm8_seq"](B, N, M, xt, q_ref, dmx, drx, dmy, dry), ys)
+    assert torch.equal(ns["cuda_mm8_one"](N, M, xt[0].contiguous(), q_ref, dmx, drx, dmy, dry), y1)
+    assert len(ns["_kept"]) == 1
     T, C = 19, 256
     k = rng.standard_normal((T, C)).astype(np.float32)
     v = rng.standard_normal((T, C)).astype(np.float32)

@@ -904,6 +904,33 @@ def test_two_caller_streams(ver):
         assert torch.equal(x, y)
 
 
+def test_more_caller_streams_than_side_stream_sets():
+    """The library keeps at most 32 sets of side streams.  Sequence calls of 300 tokens (long enough to use them) from
+    40 streams that are all alive: the ones beyond the 32nd run on the caller's stream alone and every result equals
+    the first one bit for bit; a stream that is handed back with rwkv_release_stream frees its set for the next."""
+    from chatrwkv_amd import lib
+    L = lib.load()
+    ck = synth.make_checkpoint(version=4, seed=95, n_layer=2, n_embd=1024, n_ffn=4096, vocab=500, affine=True)
+    m = _rwkv()(ck, "cuda fp16i8", verbose=False)
+    toks = synth.random_tokens(300, 500, seed=96)
+    ref, ref_st = m.forward(toks, None)
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream() for _ in range(40)]
+    for s in streams:
+        with torch.cuda.stream(s):
+            out, st = m.forward(toks, None)
+        s.synchronize()
+        assert torch.equal(out, ref)
+        for a, b in zip(st, ref_st):
+            assert torch.equal(a, b)
+    for s in streams:
+        assert L.rwkv_release_stream(s.cuda_stream) == 0
+    with torch.cuda.stream(streams[39]):
+        out, _ = m.forward(toks, None)
+    torch.cuda.synchronize()
+    assert torch.equal(out, ref)
+
+
 def test_calls_from_two_streams_are_ordered(tiny_models):
     """forward() issued from two torch streams alternately, on ONE model object (one workspace, one logits
     buffer): the calls are put in one order on the device, so every result equals the single-stream one."""

@@ -219,6 +219,58 @@ def test_gemm_f16_batched_and_row_major():
     assert np.abs(y32.cpu().numpy().astype(np.float64) - ref[0]).max() <= 1e-4 * max(np.abs(ref[0]).max(), 1.0)
 
 
+def test_gemm_f16_batched_entry_strides():
+    """rwkv_gemm_f16_batched through the C ABI with batch strides that are not the dense ones: operands and results
+    of the five products lie in larger buffers; long enough (300 rows, K = 64) for the MFMA kernel, and one-row
+    products for the streaming one."""
+    from chatrwkv_amd import lib
+    L = lib.load()
+    r = _rng(17)
+    nb, N, M = 5, 64, 136
+    for B in (300, 1):
+        a = torch.from_numpy(r.standard_normal((nb, B + 3, N)).astype(np.float16)).to(DEV)      # 3 unused rows per item
+        bt = torch.from_numpy((r.standard_normal((nb, M + 2, N)) * 0.1).astype(np.float16)).to(DEV)  # [batch, M + 2, N]
+        c = torch.full((nb, B + 1, M), float("nan"), dtype=torch.float32, device=DEV)
+        rc = L.rwkv_gemm_f16_batched(nb, B, N, M, a.data_ptr(), a.stride(1), a.stride(0), bt.data_ptr(), 1, bt.stride(1),
+                                     bt.stride(0), c.data_ptr(), c.stride(1), c.stride(0), lib.RWKV_DT_F32,
+                                     torch.cuda.current_stream().cuda_stream)
+        assert rc == 0, rc
+        torch.cuda.synchronize()
+        ref = np.einsum("bij,bkj->bik", a[:, :B].cpu().numpy().astype(np.float64), bt[:, :M].cpu().numpy().astype(np.float64))
+        got = c[:, :B].cpu().numpy().astype(np.float64)
+        assert np.abs(got - ref).max() <= 1e-4 * max(np.abs(ref).max(), 1.0)
+        assert bool(torch.isnan(c[:, B]).all())                                               # the spare row is untouched
+    assert L.rwkv_gemm_f16_batched(0, 4, 64, 8, a.data_ptr(), 64, 0, bt.data_ptr(), 1, 64, 0, c.data_ptr(), 8, 0, 0, None) == -1
+    assert L.rwkv_gemm_f16_batched(2, 4, 64, 8, a.data_ptr(), 64, 4, bt.data_ptr(), 1, 64, 0, c.data_ptr(), 8, 0, 0, None) == -2
+
+
+def test_mm8_accepts_the_reference_device_layout():
+    """A uint8 matrix as the reference's loader leaves it on the GPU (``.contiguous()`` [N, M], output index
+    contiguous; model.py:860): the operator functions repack it once per tensor and reuse the copy; results equal the
+    ones from the kernel layout bit for bit, and an in-place change of the tensor is seen."""
+    ops = _ops()
+    N, M, B = 768, 3072, 37
+    x, ref, (q_ic, mx, rx, my, ry) = _mm8_case(N, M, B, 4321)
+    q_ref = q_ic.contiguous()                                  # strides (M, 1): the reference's layout
+    assert q_ref.stride() == (M, 1) and q_ic.stride() == (1, N)
+    xt = torch.from_numpy(x).to(DEV)
+    y_ic = ops.cuda_mm8_seq(B, N, M, xt, q_ic, mx, rx, my, ry)
+    y_ref = ops.cuda_mm8_seq(B, N, M, xt, q_ref, mx, rx, my, ry)
+    assert torch.equal(y_ic, y_ref)
+    n_cached = len(ops._repacked)
+    y1 = ops.cuda_mm8_one(N, M, xt[0].contiguous(), q_ref, mx, rx, my, ry)
+    assert len(ops._repacked) == n_cached                      # the second call reused the repacked copy
+    assert torch.equal(y1, ops.cuda_mm8_one(N, M, xt[0].contiguous(), q_ic, mx, rx, my, ry))
+    q_ref[5].add_(1)                                           # in place: the version counter moves, the copy is redone
+    q_ic2 = q_ic.clone()
+    q_ic2[5].add_(1)
+    assert torch.equal(ops.cuda_mm8_seq(B, N, M, xt, q_ref, mx, rx, my, ry), ops.cuda_mm8_seq(B, N, M, xt, q_ic2, mx, rx, my, ry))
+    del q_ref
+    import gc
+    gc.collect()
+    assert len(ops._repacked) == n_cached - 1                  # the copy goes with the tensor
+
+
 # ------------------------------------------------------------------------------ WKV
 @pytest.mark.parametrize("T,C", [(1, 768), (7, 768), (64, 1000), (300, 768), (1024, 4096)])
 def test_wkv4(T, C):

@@ -112,3 +112,43 @@ def test_static_scratch_entry_rejects_oversize():
         lib.check(-6, "rwkv_mm8_seq_f16_static")
     torch.cuda.synchronize()
     assert float(y.abs().max()) == 0.0
+
+
+def test_static_scratch_entry_under_graph_capture():
+    """The entry point is meant for callers under HIP graph capture: after one call outside capture (the first call on
+    a device does host-side set-up), the call is captured into a graph; three replays, with eager work and
+    synchronisations between them and the input changed before the last one, each equal to rwkv_mm8_seq_f16 on the
+    same input bit for bit."""
+    from chatrwkv_amd import lib
+    L = lib.load()
+    x, q, vec, ref = _case(4096, 4096, 300, 11)
+    B, N, M = 300, 4096, 4096
+    mx, rx, my, ry = vec
+    ws = torch.empty(L.rwkv_mm8_seq_workspace(B, N), dtype=torch.uint8, device=DEV)
+    y_static = torch.empty((B, M), dtype=torch.float16, device=DEV)
+    y_ws = torch.empty((B, M), dtype=torch.float16, device=DEV)
+    _both(L, x, q, vec, y_static, y_ws, ws)                     # warm call outside capture
+    assert torch.equal(y_static, y_ws)
+    g = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(g, stream=side):
+            rc = L.rwkv_mm8_seq_f16_static(B, N, M, x.data_ptr(), x.stride(0), q.data_ptr(), q.stride(0), q.stride(1),
+                                           mx.data_ptr(), rx.data_ptr(), my.data_ptr(), ry.data_ptr(), y_static.data_ptr(),
+                                           y_static.stride(0), torch.cuda.current_stream().cuda_stream)
+            assert rc == 0, rc
+    torch.cuda.current_stream().wait_stream(side)
+    for rep in range(3):
+        if rep == 2:
+            x.mul_(0.5)                                        # new input in the same buffer
+        y_static.fill_(float("nan"))
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        rc = L.rwkv_mm8_seq_f16(B, N, M, x.data_ptr(), x.stride(0), q.data_ptr(), q.stride(0), q.stride(1), mx.data_ptr(),
+                                rx.data_ptr(), my.data_ptr(), ry.data_ptr(), y_ws.data_ptr(), y_ws.stride(0), ws.data_ptr(),
+                                ws.numel(), torch.cuda.current_stream().cuda_stream)
+        assert rc == 0, rc
+        torch.cuda.synchronize()
+        assert torch.equal(y_static, y_ws), rep
