@@ -269,8 +269,10 @@ class RWKV:
 
     def _plan_staging(self):
         """Streamed layers (model.py:854-858, 1526-1530, 1617-1620): their key / value / receptance / output matrices
-        live in pinned host memory and are copied into ONE device staging buffer, sized for the largest such layer,
-        right before the layer runs; every streamed layer's descriptors point into that buffer."""
+        live in pinned host memory and are copied into one of TWO device staging buffers, each sized for the largest
+        such layer; streamed layers alternate between the two, so that the next streamed layer's copy (on a copy
+        stream of its own) runs under the current layer's kernels.  Every streamed layer's descriptors point into
+        its buffer."""
         self._stage_ptr, self._stage_plan, sizes = {}, {}, {}
         for name, t in self.w.items():
             if isinstance(t, torch.Tensor) and not t.is_cuda and t.dim() == 2 and name.endswith(_STREAMED_KEYS):
@@ -281,10 +283,15 @@ class RWKV:
                 sizes[layer] = off + ((nbytes + 255) & ~255)
         self._staging = None
         if sizes:
-            self._staging = torch.empty(max(sizes.values()), dtype=torch.uint8, device=self.device)
+            nslot = 2 if len(sizes) > 1 else 1
+            self._staging = [torch.empty(max(sizes.values()), dtype=torch.uint8, device=self.device) for _ in range(nslot)]
+            self._stage_slot = {layer: k % nslot for k, layer in enumerate(sorted(self._stage_plan))}
             for layer, items in self._stage_plan.items():
                 for name, _, off, _ in items:
-                    self._stage_ptr[name] = self._staging.data_ptr() + off
+                    self._stage_ptr[name] = self._staging[self._stage_slot[layer]].data_ptr() + off
+            self._copy_stream = torch.cuda.Stream(device=self.device)        # default priority
+            self._slot_free = [None] * nslot       # recorded on the compute stream after the kernels that read the slot
+            self._streamed_order = sorted(self._stage_plan)
         # the calls one forward pass is made of: runs of resident layers, and every streamed layer alone
         self._segments, i, L = [], 0, self.args.n_layer
         while i < L:
@@ -298,15 +305,48 @@ class RWKV:
                 self._segments.append((i, j))
                 i = j
 
+    def _enqueue_stage_copy(self, layer):
+        """The host-to-device copies of one streamed layer on the copy stream, once the kernels that last read its
+        staging buffer have finished; returns the event its kernels must wait for."""
+        slot = self._stage_slot[layer]
+        cs = self._copy_stream
+        if self._slot_free[slot] is not None:
+            cs.wait_event(self._slot_free[slot])
+        buf = self._staging[slot]
+        with torch.cuda.stream(cs):
+            for _, host, off, nbytes in self._stage_plan[layer]:
+                buf[off:off + nbytes].copy_(host, non_blocking=True)
+            filled = torch.cuda.Event()
+            filled.record(cs)
+        return filled
+
     def _run_segments(self, call):
-        """call() once per segment with the model's layer range set, the streamed layer's matrices copied first
-        (same stream: the copy follows the previous layer's kernels and precedes this layer's)."""
+        """call() once per segment with the model's layer range set.  A streamed layer's matrices are copied into
+        its staging buffer on the copy stream, one streamed layer ahead of the kernels: the copy of the next
+        streamed layer is queued before this segment's kernels, waits only for the kernels that last read that
+        buffer (two streamed layers back), and this layer's kernels wait for their own copy."""
         m = self._model
+        if not self._stage_plan:
+            for lb, le in self._segments:
+                m.layer_begin, m.layer_end = lb, le
+                call()
+            m.layer_begin = m.layer_end = 0
+            return
+        cur = torch.cuda.current_stream()
+        order = self._streamed_order
+        filled = {order[0]: self._enqueue_stage_copy(order[0])}
         for lb, le in self._segments:
-            for _, host, off, nbytes in self._stage_plan.get(lb, ()):
-                self._staging[off:off + nbytes].copy_(host, non_blocking=True)
+            if lb in self._stage_plan:
+                k = order.index(lb)
+                if k + 1 < len(order):         # two buffers whenever there are two streamed layers
+                    filled[order[k + 1]] = self._enqueue_stage_copy(order[k + 1])
+                cur.wait_event(filled.pop(lb))
             m.layer_begin, m.layer_end = lb, le
             call()
+            if lb in self._stage_plan:
+                ev = torch.cuda.Event()
+                ev.record(cur)
+                self._slot_free[self._stage_slot[lb]] = ev
         m.layer_begin = m.layer_end = 0
 
     def _build_descriptors(self):
