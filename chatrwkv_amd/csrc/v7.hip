@@ -85,20 +85,35 @@ struct Wkv7Args {
 //     y_i = sum_j S'_ij r_j = sum_j S_ij (w_j r_j) + v_i (k . r) + sa_i (b . r)
 // so that both row sums of a token run on the OLD state side by side; k . r and b . r are per-token
 // scalars computed while staging.
-//   IN_F16: element type of r, k, v, a, b (and of w, y in the operator form)
+//   DT:     element type of r, k, v, a, b (and of w, y in the operator form): RWKV_DT_F16, RWKV_DT_F32 or RWKV_DT_BF16
 //   MODEL:  w is the fp32 decay itself and y an fp32 scratch; otherwise w is the log-decay
 //           (decay = exp(-exp(w))) and y has the input type
 // Staging: thread (token tid / 8, channels 8 (tid % 8) ..+7) loads its share of the NEXT slab into
 // registers before the token loop of the current one, so the loads' latency is hidden behind the loop.
-template <bool IN_F16>
+// bf16 <-> fp32: the upper half of the fp32 pattern; stores round to nearest even (NaN stays NaN)
+DEV float bf2f(uint16_t v) { return __builtin_bit_cast(float, (uint32_t)v << 16); }
+DEV uint16_t f2bf(float f) {
+    const uint32_t u = __builtin_bit_cast(uint32_t, f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);
+    return (uint16_t)((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
+}
+
+template <int DT>
 struct Stage7 {
     float r[8], k[8], a[8], b[8], w[8], v[2];
 
     DEV void load8(const void *p, size_t o, float (&d)[8]) {
-        if (IN_F16) {
+        if (DT == RWKV_DT_F16) {
             const h16x8 x = *(const h16x8 *)((const rwkv_half *)p + o);
 #pragma unroll
             for (int e = 0; e < 8; ++e) d[e] = (float)x[e];
+        } else if (DT == RWKV_DT_BF16) {
+            const u32x4 x = *(const u32x4 *)((const uint16_t *)p + o);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                d[2 * e] = __builtin_bit_cast(float, x[e] << 16);
+                d[2 * e + 1] = __builtin_bit_cast(float, x[e] & 0xffff0000u);
+            }
         } else {
             const f32x4 x0 = *(const f32x4 *)((const float *)p + o), x1 = *(const f32x4 *)((const float *)p + o + 4);
 #pragma unroll
@@ -107,7 +122,7 @@ struct Stage7 {
     }
 };
 
-template <bool IN_F16, bool MODEL>
+template <int DT, bool MODEL>
 __global__ __launch_bounds__(256) void wkv7_kernel(Wkv7Args a) {
     __shared__ __align__(16) float swr[TS7][HS7], sk[TS7][HS7], sw[TS7][HS7], sa[TS7][HS7], sb[TS7][HS7];
     __shared__ float sv[TS7][16], skr[TS7], sbr[TS7];
@@ -119,7 +134,7 @@ __global__ __launch_bounds__(256) void wkv7_kernel(Wkv7Args a) {
     const int stt = threadIdx.x >> 3, sc = (threadIdx.x & 7) * 8;   // staging role
     float *S = a.state + (size_t)h * HS7 * HS7 + (size_t)i * HS7 + 4 * g;
     f32x4 s = *(const f32x4 *)S;
-    Stage7<IN_F16> st;
+    Stage7<DT> st;
     auto fetch = [&](int t0) {
         const size_t o = (size_t)min(t0 + stt, T - 1) * C + h * HS7;   // rows past the end re-read the last one
         st.load8(a.r, o + sc, st.r);
@@ -134,9 +149,12 @@ __global__ __launch_bounds__(256) void wkv7_kernel(Wkv7Args a) {
             st.load8(a.w, o + sc, st.w);
         }
         const size_t ov = o + vb * 16 + 2 * (threadIdx.x & 7);
-        if (IN_F16) {
+        if (DT == RWKV_DT_F16) {
             const h16x2 x = *(const h16x2 *)((const rwkv_half *)a.v + ov);
             st.v[0] = (float)x[0]; st.v[1] = (float)x[1];
+        } else if (DT == RWKV_DT_BF16) {
+            const uint32_t x = *(const uint32_t *)((const uint16_t *)a.v + ov);
+            st.v[0] = __builtin_bit_cast(float, x << 16); st.v[1] = __builtin_bit_cast(float, x & 0xffff0000u);
         } else {
             st.v[0] = ((const float *)a.v)[ov]; st.v[1] = ((const float *)a.v)[ov + 1];
         }
@@ -204,7 +222,8 @@ __global__ __launch_bounds__(256) void wkv7_kernel(Wkv7Args a) {
             if (g == 0) {
                 const float y = yw + q.vi * q.kr + p * q.br;
                 const size_t o = (size_t)(t0 + tt) * C + h * HS7 + i;
-                if (MODEL || !IN_F16) ((float *)a.y)[o] = y;
+                if (MODEL || DT == RWKV_DT_F32) ((float *)a.y)[o] = y;
+                else if (DT == RWKV_DT_BF16) ((uint16_t *)a.y)[o] = f2bf(y);
                 else ((rwkv_half *)a.y)[o] = f2h(y);
             }
         };
@@ -548,14 +567,15 @@ extern "C" int rwkv_wkv7_forward(int64_t B, int64_t T, int64_t C, int64_t H, flo
     if (!state || !r || !w || !k || !v || !a || !b || !y) return RWKV_E_NULL;
     int rc = wkv7_check(B, T, C, H);
     if (rc) return rc;
-    if (dtype != RWKV_DT_F16 && dtype != RWKV_DT_F32) return RWKV_E_DTYPE;
+    if (dtype != RWKV_DT_F16 && dtype != RWKV_DT_F32 && dtype != RWKV_DT_BF16) return RWKV_E_DTYPE;
     if (!aligned16(state) || !aligned16(r) || !aligned16(w) || !aligned16(k) || !aligned16(a) || !aligned16(b) ||
         (((uintptr_t)v) & 3))
         return RWKV_E_LAYOUT;
     Wkv7Args q{(int)T, (int)C, state, r, w, k, v, a, b, y};
     const dim3 grid((unsigned)(4 * H)), block(256);
-    if (dtype == RWKV_DT_F16) hipLaunchKernelGGL((wkv7_kernel<true, false>), grid, block, 0, (hipStream_t)stream, q);
-    else hipLaunchKernelGGL((wkv7_kernel<false, false>), grid, block, 0, (hipStream_t)stream, q);
+    if (dtype == RWKV_DT_F16) hipLaunchKernelGGL((wkv7_kernel<RWKV_DT_F16, false>), grid, block, 0, (hipStream_t)stream, q);
+    else if (dtype == RWKV_DT_BF16) hipLaunchKernelGGL((wkv7_kernel<RWKV_DT_BF16, false>), grid, block, 0, (hipStream_t)stream, q);
+    else hipLaunchKernelGGL((wkv7_kernel<RWKV_DT_F32, false>), grid, block, 0, (hipStream_t)stream, q);
     RWKV_LAUNCH_CHECK();
     return RWKV_OK;
 }
@@ -719,7 +739,7 @@ extern "C" int rwkv_v7_forward(const rwkv_v7_model *m, const rwkv_v56_layer_stat
         }
         {
             Wkv7Args q{(int)T, C, s.att_kv, ws.r, ws.dec, ws.k, v, ws.an, ws.b, ws.y32};
-            hipLaunchKernelGGL((wkv7_kernel<true, true>), dim3((unsigned)(4 * H)), dim3(256), 0, st, q);
+            hipLaunchKernelGGL((wkv7_kernel<RWKV_DT_F16, true>), dim3((unsigned)(4 * H)), dim3(256), 0, st, q);
         }
         hipLaunchKernelGGL(gn7_kernel, dim3(head_waves), dim3(256), 0, st, (int)T, C, ws.y32, l.lnx_w, l.lnx_b, ws.rk, v,
                            ws.g, ws.att);

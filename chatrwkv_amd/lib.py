@@ -11,7 +11,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 # RWKV_HIP_LIB: another build of the same library (kernel tuning: two builds side by side)
 LIB_PATH = os.environ.get("RWKV_HIP_LIB") or os.path.join(HERE, "librwkv_hip.so")
 
-RWKV_DT_F16, RWKV_DT_F32 = 0, 1
+RWKV_DT_F16, RWKV_DT_F32, RWKV_DT_BF16 = 0, 1, 2
 
 _ERR = {
     -1: "RWKV_E_SHAPE: size not supported by the kernel",

@@ -259,17 +259,18 @@ def RUN_RWKV_6(B, T, C, H, state, r, k, v, w, u, state_layout=0):
 
 
 def RWKV7_OP(state, r, w, k, v, a, b):
-    """model.py:198-219 (WKV_7 / torch.ops.wkv7s.forward_fp16 | _fp32): the RWKV-7 state recurrence over T
-    tokens.  r, w, k, v, a, b: [T, C] fp16 or fp32 (one dtype), ``w`` the log-decay of model.py:537; state fp32
+    """model.py:198-219 (WKV_7 / torch.ops.wkv7s.forward_bf16 | _fp16 | _fp32): the RWKV-7 state recurrence over T
+    tokens.  r, w, k, v, a, b: [T, C] fp16, bf16 or fp32 (one dtype), ``w`` the log-decay of model.py:537; state fp32
     [H, 64, 64] laid out [head][value][key], updated in place.  Returns y [T, C] in the input dtype."""
     _need_cuda(state, r, w, k, v, a, b)
-    assert all(t.dtype == r.dtype for t in (w, k, v, a, b)) and r.dtype in (torch.float16, torch.float32)
+    assert all(t.dtype == r.dtype for t in (w, k, v, a, b)) and r.dtype in (torch.float16, torch.bfloat16, torch.float32)
     assert all(t.is_contiguous() for t in (r, w, k, v, a, b))      # as the reference asserts (model.py:207)
     assert state.dtype == torch.float32 and state.is_contiguous()
     T, C = r.shape
     H = state.shape[0]
     y = torch.empty((T, C), device=r.device, dtype=r.dtype)
     rc = _lib.load().rwkv_wkv7_forward(1, T, C, H, _ptr(state), _ptr(r), _ptr(w), _ptr(k), _ptr(v), _ptr(a), _ptr(b),
-                                       _ptr(y), F16 if r.dtype == torch.float16 else F32, _stream())
+                                       _ptr(y), {torch.float16: F16, torch.float32: F32, torch.bfloat16: _lib.RWKV_DT_BF16}[r.dtype],
+                                       _stream())
     _lib.check(rc, "rwkv_wkv7_forward")
     return y

@@ -43,6 +43,7 @@ typedef uint16_t rwkv_half;
 
 #define RWKV_DT_F16 0
 #define RWKV_DT_F32 1
+#define RWKV_DT_BF16 2   /* rwkv_wkv7_forward only */
 
 /* Library / device identification.  Returns the ABI version (currently 3). */
 int rwkv_abi_version(void);
@@ -301,10 +302,10 @@ int rwkv_v56_forward(const rwkv_v56_model *m, const rwkv_v56_layer_state *states
                      void *stream);
 
 /* ---------------------------------------------------------------------------------------
- * RWKV-7 state recurrence.  Replaces torch.ops.wkv7s.forward_fp16 / forward_fp32
- * (cuda/rwkv7_op.cpp:15-26, cuda/rwkv7.cu:9-58): per head, with row i of the state held per value index,
+ * RWKV-7 state recurrence.  Replaces torch.ops.wkv7s.forward_bf16 / forward_fp16 / forward_fp32
+ * (cuda/rwkv7_op.cpp:12-26, cuda/rwkv7.cu:9-58): per head, with row i of the state held per value index,
  *     sa_i = sum_j a_j S_ij ;  S_ij = S_ij * exp(-exp(w_j)) + k_j v_i + sa_i b_j ;  y_i = sum_j S_ij r_j
- * r, w, k, v, a, b, y: [T, C] in `dtype` (RWKV_DT_F16 or RWKV_DT_F32), w is the log-decay the reference
+ * r, w, k, v, a, b, y: [T, C] in `dtype` (RWKV_DT_F16, RWKV_DT_F32 or RWKV_DT_BF16), w is the log-decay the reference
  * passes (model.py:537-538); state fp32 [H][value i][key j] (model.py:288), updated in place; head size
  * C / H must be 64; B must be 1 (cuda/rwkv7.cu:17, 66).
  */

@@ -80,6 +80,39 @@ def test_wkv7_operator(dtype):
         assert np.abs(_np(S) - S_ref).max() <= 2e-5 * max(float(np.abs(S_ref).max()), 1.0), T
 
 
+def test_wkv7_operator_bf16():
+    """The bf16 form of the operator (torch.ops.wkv7s.forward_bf16, cuda/rwkv7_op.cpp:12-14): operands are bf16
+    values widened exactly to fp32, the recurrence runs in fp32, y is rounded to bf16 (nearest even).  Against the
+    oracle's fp32 recurrence on the same bf16-valued operands: y within one bf16 rounding step, state to fp32
+    accuracy; state carried over calls of 1, 37 and 70 tokens, through ops.RWKV7_OP."""
+    from chatrwkv_amd import ops
+    rng = np.random.Generator(np.random.PCG64(19))
+    H, N = 3, 64
+    C = H * N
+
+    def as_bf16(x):                                      # fp64 -> torch bf16 (round to nearest even) and its fp32 value
+        t = torch.from_numpy(x.astype(np.float32)).to(torch.bfloat16)
+        return t, t.float().numpy()
+    S_ref = (rng.standard_normal((H, N, N)) * 0.1).astype(np.float32)
+    S = torch.from_numpy(S_ref.copy()).cuda()
+    for T in (1, 37, 70):
+        r, k, v = (as_bf16(rng.standard_normal((T, C)) * 0.5) for _ in range(3))
+        kk = rng.standard_normal((T, C))
+        kk /= np.linalg.norm(kk.reshape(T, H, N), axis=-1, keepdims=True).repeat(N, -1).reshape(T, C)
+        a, b = as_bf16(-kk), as_bf16(kk * rng.random((T, C)))
+        w = as_bf16(rng.uniform(-4.0, -0.5, (T, C)))
+        y_ref, S_ref = model_v7.wkv7_kernel(S_ref, *(x[1] for x in (r, w, k, v, a, b)))   # fp32 operands of the same values
+        y = ops.RWKV7_OP(S, *(x[0].cuda() for x in (r, w, k, v, a, b)))
+        torch.cuda.synchronize()
+        assert y.dtype == torch.bfloat16 and tuple(y.shape) == (T, C)
+        got = y.float().cpu().numpy()
+        assert np.all(np.abs(got - y_ref) <= np.abs(y_ref) * 2.0 ** -8 + 1e-6), T      # half a bf16 step is 2**-9 relative
+        # and the rounding is to nearest: the result equals torch's own rounding of the fp32 reference almost everywhere
+        same = got == torch.from_numpy(y_ref).to(torch.bfloat16).float().numpy()
+        assert same.mean() > 0.99, (T, same.mean())
+        assert np.abs(_np(S) - S_ref).max() <= 2e-5 * max(float(np.abs(S_ref).max()), 1.0), T
+
+
 def test_rwkv7_op_wrapper():
     """ops.RWKV7_OP keeps the reference's call form (model.py:218-219)."""
     from chatrwkv_amd import ops
