@@ -371,7 +371,8 @@ template <bool W_U8, int TM, int TN> struct DmaCfg {
     static constexpr int AL = TM / 64, WL = W / 8192, LOADS = AL + WL;   // 1 KB loads per wave and tile
     static constexpr int MI = TM / 64, NI = TN / 128;                    // 32 x 32 blocks per wave (2 x 4 waves)
     static constexpr int STG_STRIDE = TN + 8;   // epilogue staging: 128 rows of TN floats, padded (see the epilogue)
-    static constexpr size_t LDS = (size_t)NST * STAGE > (size_t)128 * STG_STRIDE * 4 ? (size_t)NST * STAGE : (size_t)128 * STG_STRIDE * 4;
+    static constexpr size_t BODY = (size_t)NST * STAGE > (size_t)128 * STG_STRIDE * 4 ? (size_t)NST * STAGE : (size_t)128 * STG_STRIDE * 4;
+    static constexpr size_t LDS = BODY + (W_U8 ? 2 * TM * 4 : 0);   // past the stages: the tile rows' sums s0, s2 (GemmEpi::parts)
 };
 // s_waitcnt immediates: vmcnt(n) alone, vmcnt(n) with lgkmcnt(0), lgkmcnt(n) alone
 constexpr int vm_only(int n) { return 0x0F70 | (n & 15) | ((n >> 4) << 14); }
@@ -498,6 +499,33 @@ DEV void gemm_dma_body(int T, int N, int M, const h16 *__restrict__ A, int64_t l
     constexpr bool SPREAD = D_NST == 3;
     issue(0, 0, -1);
     issue(min(1, nk - 1), D_STAGE, -1);
+    // The input's row sums arrive as partial sums per column tile of the launch that produced it: this tile's rows
+    // are added up here, in index order, while the first two tiles are in flight (the waits for these loads cover the
+    // older tile loads too, so the counted waits below still hold).  Full depth: into LDS for the epilogue;
+    // K split: the first column tile's first split writes the totals out for the second pass.
+    bool lds_sums = false;
+    if constexpr (W_U8) {
+        if (ep.parts > 1 && (!SPLIT || (m0 == 0 && split == 0))) {
+            lds_sums = !SPLIT;
+            if (tid < 2 * TM) {
+                const int row = tid & (TM - 1), which = tid / TM, t = min(t0 + row, T - 1);
+                const float *p = (which ? ep.p2 : ep.p0) + (size_t)t * ep.parts;
+                float tot = 0.f;
+                for (int j = 0; j < ep.parts; j += 64) {   // parts % 4 == 0; up to 64 partial sums in flight per thread
+                    f32x4 q[16];
+#pragma unroll
+                    for (int u = 0; u < 16; ++u) q[u] = j + 4 * u < ep.parts ? *(const f32x4 *)(p + j + 4 * u) : f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int u = 0; u < 16; ++u) tot = (((tot + q[u][0]) + q[u][1]) + q[u][2]) + q[u][3];
+                }
+                if constexpr (SPLIT) {
+                    if (t0 + row < T) (which ? (float *)ep.s2 : (float *)ep.s0)[t] = tot;
+                } else {
+                    ((float *)(smem + Cfg::BODY))[tid] = tot;
+                }
+            }
+        }
+    }
     __builtin_amdgcn_s_waitcnt(vm_only(Cfg::LOADS));   // tile 0 has landed
     __builtin_amdgcn_s_barrier();
     int so = 0, sp = 2 * D_STAGE;   // the stage being read and (three stages) the one read before it
@@ -634,11 +662,15 @@ DEV void gemm_dma_body(int T, int N, int M, const h16 *__restrict__ A, int64_t l
     constexpr int CPR = TN / 8, RPI = 512 / CPR;   // 8-wide chunks per tile row; rows one pass of the workgroup covers
     const int cq = tid % CPR, col = m0 + cq * 8;
     const bool col_ok = col < M;   // M % 8 == 0
-    h16x8 rx8, mx8;
+    h16x8 rx8, mx8, ery8 = {}, emy8 = {};
     if (W_U8 && col_ok) { rx8 = *(const h16x8 *)(ep.rx + col); mx8 = *(const h16x8 *)(ep.mx + col); }
-    auto finish8 = [&](int t, float (&v)[8]) {
+    const bool emit = ep.emit_ry != nullptr;
+    if (emit && col_ok) { ery8 = *(const h16x8 *)(ep.emit_ry + col); emy8 = *(const h16x8 *)(ep.emit_my + col); }
+    const float *lsum = (const float *)(smem + Cfg::BODY);
+    // trow: the row within the tile; a0 / a2: this thread's share of the emitted row sums
+    auto finish8 = [&](int t, int trow, float (&v)[8], float &a0, float &a2) {
         if constexpr (W_U8) {
-            const float s0t = ep.s0[t], s2t = ep.s2[t];
+            const float s0t = lds_sums ? lsum[trow] : ep.s0[t], s2t = lds_sums ? lsum[TM + trow] : ep.s2[t];
 #pragma unroll
             for (int e = 0; e < 8; ++e) v[e] = epi_affine(v[e], (float)rx8[e], (float)mx8[e], s0t, s2t);
         }
@@ -654,7 +686,18 @@ DEV void gemm_dma_body(int T, int N, int M, const h16 *__restrict__ A, int64_t l
         float o[8];
 #pragma unroll
         for (int e = 0; e < 8; ++e) o[e] = epi_act(v[e], (float)res8[e], (float)gate8[e], ep);
-        if (ep.out_dtype == RWKV_DT_F32) {
+        if (emit) {
+            // what the scaling pass of the next product would make of the fp16 output: fp16(y * ry), sum y, sum y * my
+            h16x8 y8;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float yf = (float)(h16)o[e];
+                y8[e] = (h16)(yf * (float)ery8[e]);
+                a0 += yf;
+                a2 += yf * (float)emy8[e];
+            }
+            *(h16x8 *)((rwkv_half *)Y + (size_t)t * ldy + col) = y8;
+        } else if (ep.out_dtype == RWKV_DT_F32) {
             float *yo = (float *)Y + (size_t)t * ldy + col;
             *(f32x4 *)yo = f32x4{round_h(o[0]), round_h(o[1]), round_h(o[2]), round_h(o[3])};
             *(f32x4 *)(yo + 4) = f32x4{round_h(o[4]), round_h(o[5]), round_h(o[6]), round_h(o[7])};
@@ -702,10 +745,22 @@ DEV void gemm_dma_body(int T, int N, int M, const h16 *__restrict__ A, int64_t l
 #pragma unroll 1
             for (int it = 0; it < 128 / RPI; ++it) {
                 const int row = it * RPI + tid / CPR, t = t0 + h * 128 + row;
-                if (t < T && col_ok) {
+                const bool valid = t < T && col_ok;
+                float a0 = 0.f, a2 = 0.f;
+                if (valid) {
                     const f32x4 v0 = *(const f32x4 *)(stg + row * SW + cq * 8), v1 = *(const f32x4 *)(stg + row * SW + cq * 8 + 4);
                     float v[8] = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
-                    finish8(t, v);
+                    finish8(t, h * 128 + row, v, a0, a2);
+                }
+                if (emit) {   // the CPR threads of a row are neighbours in one wave; every lane takes part
+                    a0 = row16_sum(a0);
+                    a2 = row16_sum(a2);
+                    if constexpr (CPR == 32) { a0 += __shfl_xor(a0, 16, WAVE); a2 += __shfl_xor(a2, 16, WAVE); }
+                    if (valid && cq == 0) {
+                        const size_t pi = (size_t)t * ((M + TN - 1) / TN) + m0 / TN;
+                        ep.emit_s0[pi] = a0;
+                        ep.emit_s2[pi] = a2;
+                    }
                 }
             }
             __syncthreads();
@@ -1158,6 +1213,19 @@ int pick_cfg(int64_t T, int64_t N, int64_t M, bool w_u8, bool alone, bool dma, s
 }
 
 }  // namespace
+
+GemmPlan gemm_plan(bool w_u8, int64_t T, int64_t N, int64_t M, const rwkv_half *A, int64_t lda, const void *W,
+                   int64_t ldw, const void *Y, int64_t ldy, const GemmEpi &ep) {
+    if (skinny_ok(w_u8, T, N, A, lda, W, ldw, ep)) return GemmPlan{0, 0, 0, 1};
+    const int cfg = pick_cfg(T, N, M, w_u8, !ep.small_tiles, dma_ok(w_u8, N, M, A, lda, W, ldw, Y, ldy, ep),
+                             ep.splitk_ws ? ep.splitk_bytes : 0);
+    if (cfg != 14 && cfg != 15) return GemmPlan{1, 0, 0, 1};
+    const int tile = cfg == 14 ? 256 : 128;
+    const int64_t tiles = ((T + tile - 1) / tile) * ((M + tile - 1) / tile);
+    int ks = 1;   // as launch_dma decides it
+    if (ep.splitk_ws && (M & 3) == 0) ks = dma_split(tiles, (int)(N / BK), tile < 256, (size_t)T * M * sizeof(float), ep.splitk_bytes);
+    return GemmPlan{2, tile, tile, ks};
+}
 
 int gemm_launch(bool w_u8, int64_t T, int64_t N, int64_t M, const rwkv_half *A, int64_t lda, const void *W,
                 int64_t ldw, void *Y, int64_t ldy, const GemmEpi &ep, hipStream_t st) {

@@ -18,7 +18,24 @@ struct GemmEpi {
     size_t splitk_bytes;
     int small_tiles;               // 1: keep the 128 x 128 tile (the caller runs another contraction beside this one, and a
                                    // 256 x 256 tile's 128 KB of LDS would leave no room for it on the CU)
+    // Hand-over of a uint8 product's input without a scaling pass in between (direct-to-LDS launches; gemm_plan
+    // says which launches those are).
+    // Producer: emit_ry != NULL: the output y is stored as fp16(y * emit_ry[m]), already scaled for the next
+    //   product, and the sums of y and of y * emit_my over the columns of each tile go to
+    //   emit_s0 / emit_s2 [T][ceil(M / tile width)].
+    // Consumer: parts > 1: p0 / p2 [T][parts] hold such partial row sums; a row's totals are formed in index order
+    //   by the launch itself (the K-split form writes them to s0 / s2 for its second pass, so these name scratch).
+    const rwkv_half *emit_ry, *emit_my;
+    float *emit_s0, *emit_s2;
+    int parts;
+    const float *p0, *p2;
 };
+
+// How gemm_launch would run a product: kind 0 = the 2..16-row kernel, 1 = register-staged tiles, 2 = direct-to-LDS
+// tiles of tm x tn with K split ks ways.
+struct GemmPlan { int kind, tm, tn, ks; };
+GemmPlan gemm_plan(bool w_u8, int64_t T, int64_t N, int64_t M, const rwkv_half *A, int64_t lda, const void *W,
+                   int64_t ldw, const void *Y, int64_t ldy, const GemmEpi &ep);
 
 // Size of the split-K scratch the model-level entry points reserve in their workspaces.
 constexpr size_t RWKV_SPLITK_WS_BYTES = (size_t)64 << 20;

@@ -3,6 +3,7 @@
 //   -> WKV-4 over T (r gating fused) -> prepare -> GEMM Wo (+ residual)
 //   lnmix_seq (LN2, ...) -> GEMM Wr (sigmoid), GEMM Wk (relu^2) -> prepare -> GEMM Wv (gate, residual, /2)
 // and LN_out + head on the last row (GEMV) or on every row (GEMM) for full_output.
+#include <algorithm>
 #include <cstdlib>
 #include <mutex>
 #include "kernels.h"
@@ -334,10 +335,14 @@ struct SeqWs {
     rwkv_half *x, *xs[3], *r, *rwkv, *vx, *xsv, *xx_att, *xx_ffn;
     void *k, *v;       // fp16 (uint8 weights) or fp32 (fp16 weights)
     float *sums;       // 8 * T floats
+    float *parts;      // partial row sums handed from one product's epilogue to the next product: 2 * T * PARTS_MAX floats
     float *splitk;     // RWKV_SPLITK_WS_BYTES of split-K scratch for the contraction kernel
     float *wkv;        // chunk summaries of the WKV scan
     size_t total;
 };
+
+// most partial sums a row can have: one per 128 columns of the channel-mix key product, one per 64 channels of WKV
+int64_t parts_max(int64_t C, int64_t F) { return std::max((F + 127) / 128, (C + 63) / 64); }
 
 SeqWs carve(void *base, int64_t T, int64_t C, int64_t F) {
     SeqWs w;
@@ -355,6 +360,7 @@ SeqWs carve(void *base, int64_t T, int64_t C, int64_t F) {
     w.xx_att = (rwkv_half *)take((size_t)C * 2);
     w.xx_ffn = (rwkv_half *)take((size_t)C * 2);
     w.sums = (float *)take((size_t)T * 8 * sizeof(float));
+    w.parts = (float *)take((size_t)T * 2 * parts_max(C, F) * sizeof(float));
     w.splitk = (float *)take(RWKV_SPLITK_WS_BYTES);
     w.wkv = (float *)take(wkv4_scratch_bytes(T, C));
     w.total = (size_t)(p - (unsigned char *)base);
@@ -370,6 +376,24 @@ int run_gemm(const rwkv_mat &m, bool u8, int64_t T, const rwkv_half *A, const fl
     ep.s0 = s0;
     ep.s2 = s2;
     return gemm_launch(u8, T, m.N, m.M, A, m.N, m.w, m.ld, Y, ldy, ep, st);
+}
+
+// how run_gemm with the same arguments would be launched
+GemmPlan plan_gemm(const rwkv_mat &m, bool u8, int64_t T, const rwkv_half *A, const float *s0, const float *s2, const void *Y,
+                   int64_t ldy, GemmEpi ep, float *splitk) {
+    ep.splitk_ws = splitk;
+    ep.splitk_bytes = RWKV_SPLITK_WS_BYTES;
+    ep.mx = u8 ? m.mx : nullptr;
+    ep.rx = u8 ? m.rx : nullptr;
+    ep.s0 = s0;
+    ep.s2 = s2;
+    return gemm_plan(u8, T, m.N, m.M, A, m.N, m.w, m.ld, Y, ldy, ep);
+}
+
+// RWKV_HANDOVER=0 keeps the separate scaling passes (for A/B timing)
+bool handover_enabled() {
+    const char *e = getenv("RWKV_HANDOVER");
+    return !(e && *e == '0');
 }
 
 // Two side streams (default priority) for contractions that are independent of each other and too small
@@ -567,6 +591,7 @@ extern "C" int rwkv_v4_forward_seq(const rwkv_v4_model *m, const rwkv_v4_layer_s
         // (257 .. 384 tokens: +4 % at n_embd 4096; slower at 256 and from 385 on)
         ForkScope par2(ss, st, 1, !dma_seq && ((T / 128) * (C / 128) > 128 || ((T + 127) / 128 == 3 && C == 4096)));
         float *sk2 = par2 ? nullptr : ws.splitk;
+        int vparts = 0;   // > 0: the key product hands the value product its input with this many partial sums per row
         if (T <= 128 && !(C & 127) && !(F & 127)) {
             // short calls: receptance and key in one grouped launch
             const rwkv_half *xin[2] = {ws.xs[0], ws.xs[1]};
@@ -579,12 +604,32 @@ extern "C" int rwkv_v4_forward_seq(const rwkv_v4_model *m, const rwkv_v4_layer_s
         if ((rc = run_gemm(l.ffn_receptance, u8, T, ws.xs[0], s0[0], s2[0], ws.r, C, e, par2 ? ss->s[0] : st, sk2))) return rc;
         e.act = ACT_RELU_SQ;
         e.small_tiles = par2 ? 1 : 0;   // the receptance product runs beside this one
-        if ((rc = run_gemm(l.ffn_key, u8, T, ws.xs[1], s0[1], s2[1], ws.vx, F, e, st, sk2))) return rc;
+        // Where the key product runs at full depth through the direct-to-LDS kernel and the value product through that
+        // kernel too, the key product's epilogue writes relu(k)^2 already scaled for the value product, with the row
+        // sums as one partial sum per column tile: no scaling pass, and the unscaled [T, F] activation is never stored.
+        if (u8 && handover_enabled()) {
+            const GemmPlan pk = plan_gemm(l.ffn_key, true, T, ws.xs[1], s0[1], s2[1], ws.xsv, F, e, sk2);
+            GemmEpi ev{};
+            ev.out_scale = 1.f; ev.out_dtype = RWKV_DT_F16;
+            ev.act = ACT_GATED_RESIDUAL; ev.gate = ws.r; ev.ldgate = C; ev.res = ws.x; ev.ldres = C;
+            const GemmPlan pv = plan_gemm(l.ffn_value, true, T, ws.xsv, s0v, s2v, ws.x, C, ev, ws.splitk);
+            const int np = pk.kind == 2 ? (F + pk.tn - 1) / pk.tn : 0;
+            if (pk.kind == 2 && pk.ks == 1 && pv.kind == 2 && np > 1 && !(np & 3)) {
+                vparts = np;
+                e.emit_ry = l.ffn_value.ry; e.emit_my = l.ffn_value.my;
+                e.emit_s0 = ws.parts; e.emit_s2 = ws.parts + (size_t)T * np;
+            }
+        }
+        if ((rc = run_gemm(l.ffn_key, u8, T, ws.xs[1], s0[1], s2[1], vparts ? ws.xsv : ws.vx, F, e, st, sk2))) return rc;
         e.small_tiles = 0;
+        e.emit_ry = e.emit_my = nullptr; e.emit_s0 = e.emit_s2 = nullptr;
         if (!par2.join()) return (int)hipErrorUnknown;
         }
         const rwkv_half *a_v = ws.vx;
-        if (u8) {
+        if (vparts) {
+            a_v = ws.xsv;
+            e.parts = vparts; e.p0 = ws.parts; e.p2 = ws.parts + (size_t)T * vparts;
+        } else if (u8) {
             if ((rc = mm8_prepare_launch(T, F, ws.vx, F, l.ffn_value.ry, l.ffn_value.my, ws.xsv, s0v, s2v, st))) return rc;
             a_v = ws.xsv;
         }

@@ -200,6 +200,7 @@ __global__ __launch_bounds__(256) void v6_mix2x4_kernel(Mix2Args a) {
 struct Ws56 {
     rwkv_half *x, *xx, *sxd, *xxx, *t1, *mix[5], *d1, *d2, *r, *k, *v, *g, *att, *vx, *xs, *xx_att, *xx_ffn;
     float *sums, *splitk, *y32;
+    float *parts;            // partial row sums handed from the key product's epilogue to the value product
     rwkv_half *xs_side[3];   // scaled-activation scratch of the products that run beside the first one [T, C]
     float *sums_side[3];
     size_t total;
@@ -224,6 +225,7 @@ Ws56 carve56(void *base, int64_t T, int64_t C, int64_t F, int64_t lm, int64_t ld
     }
     w.splitk = (float *)take(RWKV_SPLITK_WS_BYTES);
     w.y32 = (float *)take(T >= 32 ? (size_t)T * C * 4 : 256);
+    w.parts = (float *)take(T > 1 ? (size_t)T * 2 * ((F + 127) / 128) * sizeof(float) : 256);
     w.total = (size_t)(p - (unsigned char *)base);
     return w;
 }
@@ -465,18 +467,24 @@ extern "C" int rwkv_v56_forward(const rwkv_v56_model *m, const rwkv_v56_layer_st
             ep[0].act = ACT_SIGMOID; ep[1].act = ACT_RELU_SQ;
             for (int j = 0; j < 2; ++j) { ep[j].out_scale = 1.f; ep[j].out_dtype = RWKV_DT_F16; }
             if ((rc = gemm_group_launch(u8, 2, T, C, xin, mats, outs, ep, nullptr, fs, ws.splitk, st))) return rc;
+            if ((rc = mm(c, l.ffn_value, u8, ws.vx, ACT_GATED_RESIDUAL, ws.x, ws.r, scale, ws.x))) return rc;
         } else {
-            // channel-mix receptance beside the key product
+            // channel-mix receptance beside the key product (one after the other in long calls); the key product
+            // hands the value product its input already scaled where both run through the direct-to-LDS kernel
             ForkScope par(ss, st, 1, !dma_seq);
             if ((rc = mm_scaled(par ? cs[0] : c, l.ffn_receptance, u8, fx[0], fs[0], fs[0] + T, ACT_SIGMOID, nullptr, nullptr,
                                 1.f, ws.r)))
                 return rc;
             Ctx ck = c;
             ck.small_tiles = par ? 1 : 0;
-            if ((rc = mm_scaled(ck, l.ffn_key, u8, fx[1], fs[1], fs[1] + T, ACT_RELU_SQ, nullptr, nullptr, 1.f, ws.vx))) return rc;
+            int np = 0;
+            if ((rc = mm_pair_first(ck, c, l.ffn_key, l.ffn_value, u8, fx[1], fs[1], fs[1] + T, ACT_RELU_SQ, ws.vx,
+                                    ACT_GATED_RESIDUAL, ws.x, ws.r, ws.x, ws.parts, &np)))
+                return rc;
             if (!par.join()) return (int)hipErrorUnknown;
+            if ((rc = mm_pair_second(c, l.ffn_key, l.ffn_value, u8, ws.vx, ACT_GATED_RESIDUAL, ws.x, ws.r, scale, ws.x, ws.parts, np)))
+                return rc;
         }
-        if ((rc = mm(c, l.ffn_value, u8, ws.vx, ACT_GATED_RESIDUAL, ws.x, ws.r, scale, ws.x))) return rc;
         RWKV_LAUNCH_CHECK();
     }
     // ---- head
