@@ -364,12 +364,18 @@ __global__ __launch_bounds__(64 * WT * WM) void gemm_kernel(int T, int N, int M,
 // one tile is in flight while one multiplies.
 // Tile TM x TN is 256 x 256 (wave tile 128 x 64: the long, wide products) or 128 x 128 (wave tile 64 x 32, a stage of
 // 24 KB: products with too few 256 x 256 tiles for the chip run at full depth with these instead of splitting K).
+// NW (waves per workgroup: 8, or 4 with 64 x 64 wave tiles) and NSTG (stages, 0 = the default above) exist for
+// tuning runs.  Measured on the 128 x 128 tile with uint8 weights: four waves of 64 x 64 (a third fewer fragment
+// reads per MFMA) 45.0 against 41.7 us on [1024 x 4096] x [4096 x 4096] and equal on launches of several rounds;
+// four and five stages (tiles three and four ahead) 42.6 against 42.8 us, and 4-6 % slower on launches of several
+// rounds, where only one workgroup then fits a CU.  Neither fragment reads nor load latency bound that tile.
 constexpr int DT = 256, DM = 256;
-template <bool W_U8, int TM, int TN> struct DmaCfg {
+template <bool W_U8, int TM, int TN, int NW = 8, int NSTG = 0> struct DmaCfg {
     static constexpr int A = TM * BK * 2, W = W_U8 ? TN * BK : TN * BK * 2, STAGE = A + W;
-    static constexpr int NST = (W_U8 || TM < 256) ? 3 : 2;
-    static constexpr int AL = TM / 64, WL = W / 8192, LOADS = AL + WL;   // 1 KB loads per wave and tile
-    static constexpr int MI = TM / 64, NI = TN / 128;                    // 32 x 32 blocks per wave (2 x 4 waves)
+    static constexpr int NST = NSTG ? NSTG : (W_U8 || TM < 256) ? 3 : 2;
+    static constexpr int AL = A / 1024 / NW, WL = W / 1024 / NW, LOADS = AL + WL;   // 1 KB loads per wave and tile
+    static constexpr int WR = 2, WC = NW / 2;                            // waves: 2 rows x 4 (or 2) columns
+    static constexpr int MI = TM / (32 * WR), NI = TN / (32 * WC);       // 32 x 32 blocks per wave
     static constexpr int STG_STRIDE = TN + 8;   // epilogue staging: 128 rows of TN floats, padded (see the epilogue)
     static constexpr size_t BODY = (size_t)NST * STAGE > (size_t)128 * STG_STRIDE * 4 ? (size_t)NST * STAGE : (size_t)128 * STG_STRIDE * 4;
     static constexpr size_t LDS = BODY + (W_U8 ? 2 * TM * 4 : 0);   // past the stages: the tile rows' sums s0, s2 (GemmEpi::parts)
@@ -379,15 +385,16 @@ constexpr int vm_only(int n) { return 0x0F70 | (n & 15) | ((n >> 4) << 14); }
 constexpr int vm_lgkm0(int n) { return 0x0070 | (n & 15) | ((n >> 4) << 14); }
 constexpr int lgkm_only(int n) { return 0xC07F | (n << 8); }
 
-template <bool W_U8, bool SPLIT, int TM, int TN>
+template <bool W_U8, bool SPLIT, int TM, int TN, int NW = 8, int NSTG = 0>
 DEV void gemm_dma_body(int T, int N, int M, const h16 *__restrict__ A, int64_t lda, const void *__restrict__ Wv, int64_t ldw,
                        void *__restrict__ Y, int64_t ldy, const GemmEpi &ep, int nk_split, float *__restrict__ part, int split) {
-    using Cfg = DmaCfg<W_U8, TM, TN>;
+    using Cfg = DmaCfg<W_U8, TM, TN, NW, NSTG>;
     constexpr int D_A = Cfg::A, D_STAGE = Cfg::STAGE, D_NST = Cfg::NST, AL = Cfg::AL, WL = Cfg::WL, MI = Cfg::MI, NI = Cfg::NI;
     static_assert((TM == 256 || TM == 128) && (TN == 256 || TN == 128), "tile");
+    static_assert((NW == 8 || NW == 4) && 2 * TM <= 64 * NW && MI >= 2 && MI <= 4 && NI >= 1 && NI <= 2, "waves");
     extern __shared__ __align__(1024) unsigned char smem[];
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wr = wave >> 2, wc = wave & 3;
+    const int wr = wave / Cfg::WC, wc = wave % Cfg::WC;
     const int tiles_t = (T + TM - 1) / TM;
     int bid = blockIdx.x;
     if ((gridDim.x & 7) == 0) bid = (bid & 7) * (gridDim.x >> 3) + (bid >> 3);
@@ -496,9 +503,12 @@ DEV void gemm_dma_body(int T, int N, int M, const h16 *__restrict__ A, int64_t l
     // issued in three parts between the MFMA steps, into the stage tile kt - 1 was read from (a burst of all of
     // them right after the barrier measured 2 % slower).  Two stages: tile kt + 2 can only go where tile kt is, so
     // its loads follow the barrier in one go.
-    constexpr bool SPREAD = D_NST == 3;
+    constexpr bool SPREAD = D_NST >= 3;
+    constexpr int PD = SPREAD ? D_NST - 1 : 2;   // tiles in flight ahead of the one being multiplied
     issue(0, 0, -1);
     issue(min(1, nk - 1), D_STAGE, -1);
+#pragma unroll
+    for (int p = 2; p < PD; ++p) issue(min(p, nk - 1), p * D_STAGE, -1);
     // The input's row sums arrive as partial sums per column tile of the launch that produced it: this tile's rows
     // are added up here, in index order, while the first two tiles are in flight (the waits for these loads cover the
     // older tile loads too, so the counted waits below still hold).  Full depth: into LDS for the epilogue;
@@ -526,9 +536,9 @@ DEV void gemm_dma_body(int T, int N, int M, const h16 *__restrict__ A, int64_t l
             }
         }
     }
-    __builtin_amdgcn_s_waitcnt(vm_only(Cfg::LOADS));   // tile 0 has landed
+    __builtin_amdgcn_s_waitcnt(vm_only((PD - 1) * Cfg::LOADS));   // tile 0 has landed
     __builtin_amdgcn_s_barrier();
-    int so = 0, sp = 2 * D_STAGE;   // the stage being read and (three stages) the one read before it
+    int so = 0, sp = (D_NST - 1) * D_STAGE;   // the stage being read and (three stages and more) the one read before it
     // Second schedule (uint8 weights, and the large tile with fp16 weights; measured: [1024 x 4096] x [4096 x 4096]
     // uint8 57 -> 50 us, the large tile 1-4 % faster, the small tile with fp16 weights 10-15 % slower):
     // fragments are read TWO steps ahead of their MFMAs and the uint8 -> fp16 widening of step s + 1 is issued
@@ -569,7 +579,7 @@ DEV void gemm_dma_body(int T, int N, int M, const h16 *__restrict__ A, int64_t l
         widen(0);
         for (int kt = 0; kt < nk; ++kt) {
             const int sn = so + D_STAGE >= D_NST * D_STAGE ? 0 : so + D_STAGE;
-            const int kl = min(kt + 2, nk - 1);
+            const int kl = min(kt + PD, nk - 1);
             // step 0
             mfmas(0);
             reads_done();
@@ -585,7 +595,7 @@ DEV void gemm_dma_body(int T, int N, int M, const h16 *__restrict__ A, int64_t l
             if (SPREAD) issue(kl, sp, 1);
             __builtin_amdgcn_sched_barrier(0);
             // my part of tile kt + 1 has landed (newer: the A loads of tile kt + 2) and all my reads of tile kt are back
-            __builtin_amdgcn_s_waitcnt(vm_lgkm0(SPREAD ? AL : 0));
+            __builtin_amdgcn_s_waitcnt(vm_lgkm0(SPREAD ? (PD - 2) * Cfg::LOADS + AL : 0));
             __builtin_amdgcn_s_barrier();
             if (!SPREAD) issue(kl, so, -1);
             // step 2
@@ -607,7 +617,7 @@ DEV void gemm_dma_body(int T, int N, int M, const h16 *__restrict__ A, int64_t l
         ldfrag(0, 0, 0);
         for (int kt = 0; kt < nk; ++kt) {
             const int sn = so + D_STAGE >= D_NST * D_STAGE ? 0 : so + D_STAGE;
-            const int kl = min(kt + 2, nk - 1);
+            const int kl = min(kt + PD, nk - 1);
             ldfrag(1, so, 1);
             if (SPREAD) issue(kl, sp, 0);
             __builtin_amdgcn_sched_barrier(0);
@@ -625,7 +635,7 @@ DEV void gemm_dma_body(int T, int N, int M, const h16 *__restrict__ A, int64_t l
             multiply(0);
             // all my reads of this stage have returned and my part of tile kt + 1 has landed (with three stages tile
             // kt + 2 is in flight)
-            __builtin_amdgcn_s_waitcnt(vm_lgkm0(SPREAD ? Cfg::LOADS : 0));
+            __builtin_amdgcn_s_waitcnt(vm_lgkm0(SPREAD ? (PD - 1) * Cfg::LOADS : 0));
             __builtin_amdgcn_s_barrier();
             if (!SPREAD) issue(kl, so, -1);
             ldfrag(0, sn, 0);
@@ -659,7 +669,7 @@ DEV void gemm_dma_body(int T, int N, int M, const h16 *__restrict__ A, int64_t l
     // Each thread finishes eight consecutive outputs of one row: 16-byte loads of the residual / gate rows, 16-byte
     // stores, and a body small enough to stay in the instruction cache (per-element code for 128 accumulators
     // does not).
-    constexpr int CPR = TN / 8, RPI = 512 / CPR;   // 8-wide chunks per tile row; rows one pass of the workgroup covers
+    constexpr int CPR = TN / 8, RPI = 64 * NW / CPR;   // 8-wide chunks per tile row; rows one pass of the workgroup covers
     const int cq = tid % CPR, col = m0 + cq * 8;
     const bool col_ok = col < M;   // M % 8 == 0
     h16x8 rx8, mx8, ery8 = {}, emy8 = {};
@@ -768,11 +778,11 @@ DEV void gemm_dma_body(int T, int N, int M, const h16 *__restrict__ A, int64_t l
     }
 }
 
-template <bool W_U8, bool SPLIT, int TM, int TN>
-__global__ __launch_bounds__(512) void gemm_dma_kernel(int T, int N, int M, const h16 *__restrict__ A, int64_t lda,
-                                                       const void *__restrict__ W, int64_t ldw, void *__restrict__ Y,
-                                                       int64_t ldy, GemmEpi ep, int nk_split, float *__restrict__ part) {
-    gemm_dma_body<W_U8, SPLIT, TM, TN>(T, N, M, A, lda, W, ldw, Y, ldy, ep, nk_split, part, SPLIT ? blockIdx.y : 0);
+template <bool W_U8, bool SPLIT, int TM, int TN, int NW, int NSTG>
+__global__ __launch_bounds__(64 * NW) void gemm_dma_kernel(int T, int N, int M, const h16 *__restrict__ A, int64_t lda,
+                                                           const void *__restrict__ W, int64_t ldw, void *__restrict__ Y,
+                                                           int64_t ldy, GemmEpi ep, int nk_split, float *__restrict__ part) {
+    gemm_dma_body<W_U8, SPLIT, TM, TN, NW, NSTG>(T, N, M, A, lda, W, ldw, Y, ldy, ep, nk_split, part, SPLIT ? blockIdx.y : 0);
 }
 
 // Up to four contractions [T, N] x [N, M_i] in one launch (blockIdx.y picks the operands), at full depth: short
@@ -1143,16 +1153,16 @@ int dma_split(int64_t tiles, int nk, bool small_tile, size_t out_bytes, size_t w
 
 // gemm_dma_kernel.  Fewer than 192 tiles (narrow outputs): the contraction is split over workgroups of the same
 // tile until about one workgroup per CU is in flight; slabs and the second pass as in launch_cfg.
-template <bool W_U8, int TM, int TN>
+template <bool W_U8, int TM, int TN, int NW = 8, int NSTG = 0>
 int launch_dma(int64_t T, int64_t N, int64_t M, const rwkv_half *A, int64_t lda, const void *W, int64_t ldw, void *Y,
                int64_t ldy, const GemmEpi &ep, hipStream_t st) {
-    constexpr size_t lds = DmaCfg<W_U8, TM, TN>::LDS;
+    constexpr size_t lds = DmaCfg<W_U8, TM, TN, NW, NSTG>::LDS;
     static PerDeviceOnce once;
     bool *attr_done = once.slot();
     if (!attr_done || !*attr_done) {
-        hipError_t e = hipFuncSetAttribute((const void *)gemm_dma_kernel<W_U8, false, TM, TN>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        hipError_t e = hipFuncSetAttribute((const void *)gemm_dma_kernel<W_U8, false, TM, TN, NW, NSTG>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e == hipSuccess)
-            e = hipFuncSetAttribute((const void *)gemm_dma_kernel<W_U8, true, TM, TN>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            e = hipFuncSetAttribute((const void *)gemm_dma_kernel<W_U8, true, TM, TN, NW, NSTG>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return (int)e;
         if (attr_done) *attr_done = true;
     }
@@ -1162,13 +1172,13 @@ int launch_dma(int64_t T, int64_t N, int64_t M, const rwkv_half *A, int64_t lda,
     int ks = 1;
     if (ep.splitk_ws && (M & 3) == 0) ks = dma_split(tiles, nk, TM < 256, (size_t)T * M * sizeof(float), ep.splitk_bytes);
     if (ks > 1) {
-        hipLaunchKernelGGL((gemm_dma_kernel<W_U8, true, TM, TN>), dim3((unsigned)tiles, (unsigned)ks), dim3(512), lds, st, (int)T, (int)N,
+        hipLaunchKernelGGL((gemm_dma_kernel<W_U8, true, TM, TN, NW, NSTG>), dim3((unsigned)tiles, (unsigned)ks), dim3(64 * NW), lds, st, (int)T, (int)N,
                            (int)M, (const h16 *)A, lda, W, ldw, Y, ldy, ep, nk / ks, ep.splitk_ws);
         const int64_t n = T * M;
         const unsigned blocks = (unsigned)((n + 2047) / 2048 < 16384 ? (n + 2047) / 2048 : 16384);
         hipLaunchKernelGGL(splitk_epilogue8_kernel, dim3(blocks), dim3(256), 0, st, (int)T, (int)M, ks, ep.splitk_ws, Y, ldy, ep);
     } else {
-        hipLaunchKernelGGL((gemm_dma_kernel<W_U8, false, TM, TN>), dim3((unsigned)tiles), dim3(512), lds, st, (int)T, (int)N, (int)M,
+        hipLaunchKernelGGL((gemm_dma_kernel<W_U8, false, TM, TN, NW, NSTG>), dim3((unsigned)tiles), dim3(64 * NW), lds, st, (int)T, (int)N, (int)M,
                            (const h16 *)A, lda, W, ldw, Y, ldy, ep, nk, (float *)nullptr);
     }
     RWKV_LAUNCH_CHECK();
