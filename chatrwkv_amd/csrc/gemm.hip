@@ -1062,6 +1062,75 @@ int skinny_launch(bool w_u8, int n, int64_t T, int64_t N, const SkinnyGroup &g, 
     return RWKV_OK;
 }
 
+// ---- narrow outputs: [T, N] x [N, M] with M of a LoRA rank and fp16 weights ------------------------------------
+// The first stage of a low-rank product (RWKV-6 mixing and decay LoRA, RWKV-7's four) has thousands of input columns
+// and a few dozen to a few hundred outputs: a handful of 128 x 128 tiles, which the tile kernels can only spread
+// over the chip by splitting K and adding the slabs in a second launch.  Here a workgroup of eight waves takes a
+// 16 x 16 block of the output and splits K over its waves: wave w owns the 32-wide k-chunks w, w + 8, ...; per
+// chunk a lane loads 16 bytes of one weight row and of one activation row (lane = row + 16 q: the four lanes of a
+// row cover 64 contiguous bytes), sixteen chunks in flight, and issues v_mfma_f32_16x16x32_f16 with the weights as
+// the first operand, so that lane (token j, q) ends with outputs 4 q .. 4 q + 3 of token j.  The eight partial
+// blocks are added in wave order through LDS (deterministic) and 64 threads round, apply the activation and store
+// 8 bytes each.  Operands come from L2: the weights are read once per 16 rows of the call, the activation once per
+// 16 outputs, so the kernel serves calls of up to NARROW_MAX_T rows ([256 x 4096] x [4096 x 160]: 9 us against
+// 14 us for the K-split tiles and their second pass; at 1024 rows the tiles win, 23 against 14 us).
+__global__ __launch_bounds__(512) void narrow_kernel(int T, int N, int M, const h16 *__restrict__ A, int64_t lda,
+                                                     const h16 *__restrict__ W, int64_t ldw, rwkv_half *__restrict__ Y,
+                                                     int64_t ldy, GemmEpi ep) {
+    __shared__ f32x4 red[8][64];
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int sub = lane & 15, q = lane >> 4;
+    const int t0 = blockIdx.x * 16, m0 = blockIdx.y * 16;
+    const h16 *arow = A + (size_t)min(t0 + sub, T - 1) * lda + 8 * q;
+    const h16 *wrow = W + (size_t)min(m0 + sub, M - 1) * ldw + 8 * q;
+    const int nchunks = N / 32;
+    constexpr int NB = 16;   // chunks in flight per wave: a 4096-wide row is one round
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    // chunks past the end repeat the last one and multiply zeros (no branch between the loads and their use)
+    for (int c0 = wave; c0 < nchunks; c0 += 8 * NB) {
+        h16x8 wv[NB], xv[NB];
+#pragma unroll
+        for (int i = 0; i < NB; ++i) {
+            const int c = min(c0 + 8 * i, nchunks - 1);
+            wv[i] = *(const h16x8 *)(wrow + (size_t)c * 32);
+            xv[i] = *(const h16x8 *)(arow + (size_t)c * 32);
+        }
+#pragma unroll
+        for (int i = 0; i < NB; ++i) {
+            if (c0 + 8 * i >= nchunks) xv[i] = h16x8{};
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(wv[i], xv[i], acc, 0, 0, 0);
+        }
+    }
+    red[wave][lane] = acc;
+    __syncthreads();
+    if (wave == 0) {
+        f32x4 v = red[0][lane];
+#pragma unroll
+        for (int w = 1; w < 8; ++w) v += red[w][lane];
+        const int t = t0 + sub, m = m0 + 4 * q;
+        if (t < T && m < M) {   // M % 4 == 0
+            h16x4 o;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) o[e] = (h16)epi_act(v[e], 0.f, 0.f, ep);
+            *(h16x4 *)((h16 *)Y + (size_t)t * ldy + m) = o;
+        }
+    }
+}
+
+// narrow_kernel's operands: fp16 weights, at most NARROW_MAX_M outputs, rows of whole 32-wide chunks laid out for
+// 16-byte loads, an epilogue without residual or gate, fp16 out.  RWKV_NO_NARROW=1 sends these through the tile
+// kernels (tuning).
+constexpr int NARROW_MAX_M = 192, NARROW_MAX_T = 512;
+bool narrow_ok(bool w_u8, int64_t T, int64_t N, int64_t M, const void *A, int64_t lda, const void *W, int64_t ldw, const void *Y,
+               int64_t ldy, const GemmEpi &ep) {
+    auto a16 = [](const void *p) { return (((uintptr_t)p) & 15) == 0; };
+    if (w_u8 || ep.rx || T <= SKINNY_MAX_ROWS || T > NARROW_MAX_T || M > NARROW_MAX_M || (M & 3) || N < 1024 || (N % 32)) return false;
+    if ((lda & 7) || (ldw & 7) || (ldy & 3) || !a16(A) || !a16(W) || (((uintptr_t)Y) & 7)) return false;
+    if (ep.act == ACT_RESIDUAL || ep.act == ACT_GATED_RESIDUAL || ep.raw_f32 || ep.out_dtype != RWKV_DT_F16) return false;
+    const char *e = getenv("RWKV_NO_NARROW");
+    return !(e && *e == '1');
+}
+
 }  // namespace
 
 namespace {
@@ -1244,6 +1313,12 @@ int gemm_launch(bool w_u8, int64_t T, int64_t N, int64_t M, const rwkv_half *A, 
         g.A[0] = (const h16 *)A; g.W[0] = W; g.Y[0] = Y; g.lda = lda; g.ldw[0] = ldw; g.ldy[0] = ldy; g.M[0] = (int)M; g.ep[0] = ep;
         return skinny_launch(w_u8, 1, T, N, g, st);
     }
+    if (narrow_ok(w_u8, T, N, M, A, lda, W, ldw, Y, ldy, ep)) {
+        hipLaunchKernelGGL(narrow_kernel, dim3((unsigned)((T + 15) / 16), (unsigned)((M + 15) / 16)), dim3(512), 0, st, (int)T, (int)N,
+                           (int)M, (const h16 *)A, lda, (const h16 *)W, ldw, (rwkv_half *)Y, ldy, ep);
+        RWKV_LAUNCH_CHECK();
+        return RWKV_OK;
+    }
     const int cfg = pick_cfg(T, N, M, w_u8, !ep.small_tiles, dma_ok(w_u8, N, M, A, lda, W, ldw, Y, ldy, ep),
                              ep.splitk_ws ? ep.splitk_bytes : 0);
     return w_u8 ? launch_pick<true>(cfg, T, N, M, A, lda, W, ldw, Y, ldy, ep, st)
@@ -1260,13 +1335,30 @@ int mm8_prepare_launch(int64_t T, int64_t N, const rwkv_half *x, int64_t ldx, co
 
 // n (2..4) products [T, N] x [N, M_i] of uint8 or fp16 weights with their own inputs, outputs and epilogues in one
 // launch.  uint8 with xs != NULL: x[i] is the unscaled activation and xs[i] / sums[i] (2 T floats) are scratch;
-// uint8 with xs == NULL: x[i] is already scaled by ry and sums[i] holds its row sums.
+// uint8 with xs == NULL: x[i] is already scaled by ry and sums[i] holds its row sums -- as 2 T totals, or with
+// parts > 1 (a multiple of four; direct-to-LDS launches only, see gemm_group_takes_parts) as 2 T floats of scratch
+// followed by [T][parts] partial sums of x and [T][parts] of x * my, which the launch adds up in index order.
 // Operands laid out for 16-byte loads: the direct-to-LDS kernel, tile size and K split (over splitk_ws,
 // RWKV_SPLITK_WS_BYTES of scratch, or NULL) from the cost model; otherwise register-staged 128 x 128 tiles at full depth.
+bool gemm_group_takes_parts(bool w_u8, int n, int64_t T, int64_t N, const rwkv_half *const *x, const rwkv_mat *const *mats,
+                            void *const *Y) {
+    if (!w_u8 || n < 2 || n > 4 || (N % BK)) return false;
+    const float one = 0.f;
+    bool skinny = true;
+    for (int i = 0; i < n; ++i) {
+        GemmEpi e{};
+        e.mx = mats[i]->mx; e.rx = mats[i]->rx; e.s0 = &one; e.s2 = &one; e.out_dtype = RWKV_DT_F16;
+        if (mats[i]->N != N || !dma_ok(true, N, mats[i]->M, x[i], N, mats[i]->w, mats[i]->ld, Y[i], mats[i]->M, e)) return false;
+        skinny = skinny && skinny_ok(true, T, N, x[i], N, mats[i]->w, mats[i]->ld, e);
+    }
+    return !skinny;
+}
+
 int gemm_group_launch(bool w_u8, int n, int64_t T, int64_t N, const rwkv_half *const *x, const rwkv_mat *const *mats,
                       void *const *Y, const GemmEpi *eps, rwkv_half *const *xs, float *const *sums, float *splitk_ws,
-                      hipStream_t st) {
+                      hipStream_t st, int parts) {
     if (n < 2 || n > 4 || (N % BK)) return RWKV_E_SHAPE;
+    if (parts > 1 && (xs || !w_u8 || (parts & 3))) return RWKV_E_SHAPE;
     GemmGroup g{};
     g.lda = N;
     const bool prep = w_u8 && xs;
@@ -1286,6 +1378,7 @@ int gemm_group_launch(bool w_u8, int n, int64_t T, int64_t N, const rwkv_half *c
         g.ep[i] = eps[i];
         g.ep[i].ldres = g.ep[i].ldgate = mats[i]->M;
         if (w_u8) { g.ep[i].mx = mats[i]->mx; g.ep[i].rx = mats[i]->rx; g.ep[i].s0 = sums[i]; g.ep[i].s2 = sums[i] + T; }
+        if (parts > 1) { g.ep[i].parts = parts; g.ep[i].p0 = sums[i] + 2 * T; g.ep[i].p2 = sums[i] + 2 * T + (size_t)T * parts; }
         const int64_t ts = ((T + 127) / 128) * ((mats[i]->M + 127) / 128), tb = ((T + DT - 1) / DT) * ((mats[i]->M + DM - 1) / DM);
         tiles = std::max(tiles, ts);
         tiles_big = std::max(tiles_big, tb);
@@ -1300,6 +1393,7 @@ int gemm_group_launch(bool w_u8, int n, int64_t T, int64_t N, const rwkv_half *c
         bool skinny = true;
         for (int i = 0; i < n; ++i) skinny = skinny && skinny_ok(w_u8, T, N, g.A[i], N, g.W[i], g.ldw[i], g.ep[i]);
         if (skinny) {
+            if (parts > 1) return RWKV_E_LAYOUT;
             SkinnyGroup sg{};
             sg.lda = N;
             for (int i = 0; i < n; ++i) {
@@ -1334,6 +1428,7 @@ int gemm_group_launch(bool w_u8, int n, int64_t T, int64_t N, const rwkv_half *c
         RWKV_LAUNCH_CHECK();
         return RWKV_OK;
     }
+    if (parts > 1) return RWKV_E_LAYOUT;   // partial sums only through the direct-to-LDS kernel
     constexpr size_t lds = 2 * (size_t)(128 + 128) * BK * sizeof(h16);
     const dim3 grid((unsigned)tiles, (unsigned)n);
     if (w_u8) hipLaunchKernelGGL((gemm_group_kernel<true, 128, 128, 2, 2, 4>), grid, dim3(256), lds, st, (int)T, (int)N, g);

@@ -45,7 +45,11 @@ int gemm_launch(bool w_u8, int64_t T, int64_t N, int64_t M, const rwkv_half *A, 
 // n (2..4) products [T, N] x [N, M_i] in one launch (short calls, where each alone would split K); see gemm.hip
 int gemm_group_launch(bool w_u8, int n, int64_t T, int64_t N, const rwkv_half *const *x, const rwkv_mat *const *mats,
                       void *const *Y, const GemmEpi *eps, rwkv_half *const *xs, float *const *sums, float *splitk_ws,
-                      hipStream_t st);
+                      hipStream_t st, int parts = 0);
+// true where that launch would go through the direct-to-LDS kernel, which can take the row sums of already scaled
+// inputs as `parts` partial sums per row (GemmEpi::parts)
+bool gemm_group_takes_parts(bool w_u8, int n, int64_t T, int64_t N, const rwkv_half *const *x, const rwkv_mat *const *mats,
+                            void *const *Y);
 int mm8_prepare_launch(int64_t T, int64_t N, const rwkv_half *x, int64_t ldx, const rwkv_half *ry,
                        const rwkv_half *my, rwkv_half *xs, float *s0, float *s2, hipStream_t st);
 int gemv_f16_launch(int64_t N, int64_t M, const rwkv_half *x, const rwkv_half *w, int64_t ldw, void *y,

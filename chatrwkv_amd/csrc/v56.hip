@@ -101,6 +101,12 @@ struct Mix2Args {
     const rwkv_half *prev;           // [C] token-shift state
     const rwkv_half *maa[5];         // w, k, v, r, g
     rwkv_half *out[5];               // [T, C] each
+    // v6_mix2x4_kernel, uint8 matrices: ry[j] != NULL: out[j] is stored as fp16(mix * ry[j]), the input of matrix j's
+    // product, and the sums of mix and mix * my[j] over each block of 1024 channels go to p0[j] / p2[j] [T][npart]
+    // (npart = the number of blocks rounded up to a multiple of four, the padding entries zero)
+    const rwkv_half *ry[5], *my[5];
+    float *p0[5], *p2[5];
+    int npart;
 };
 
 // grid (ceil(T / 16), C/256, 5): m_j[c] = sum_i t1[t, jR + i] * w2[j][i][c]; out_j = xx + sxd * (maa_j + m_j).
@@ -159,9 +165,12 @@ __global__ __launch_bounds__(256) void v6_mix2x4_kernel(Mix2Args a) {
         st1[r][tt] = tt < nt ? h2f(a.t1[(size_t)(t0 + tt) * 5 * R + j * R + r]) : 0.f;
     }
     __syncthreads();
-    if (c >= C) return;
-    const h16x4 maa = *(const h16x4 *)(a.maa[j] + c);
-    const rwkv_half *w = a.w2 + (size_t)j * R * C + c;
+    const bool scaled = a.ry[j] != nullptr;   // the same for the whole workgroup
+    if (c >= C && !scaled) return;
+    const bool live = c < C;
+    const int cl = live ? c : 0;              // channels past the end take part in the sums with zeros
+    const h16x4 maa = *(const h16x4 *)(a.maa[j] + cl);
+    const rwkv_half *w = a.w2 + (size_t)j * R * C + cl;
     f32x4 m[TT];
 #pragma unroll
     for (int tt = 0; tt < TT; ++tt) m[tt] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -182,18 +191,45 @@ __global__ __launch_bounds__(256) void v6_mix2x4_kernel(Mix2Args a) {
             }
         }
     }
+    h16x4 ry4 = {}, my4 = {};
+    if (scaled) { ry4 = *(const h16x4 *)(a.ry[j] + cl); my4 = *(const h16x4 *)(a.my[j] + cl); }
+    float sums[2 * TT];
 #pragma unroll
     for (int tt = 0; tt < TT; ++tt) {
-        const size_t o = (size_t)(t0 + min(tt, nt - 1)) * C + c;
+        const size_t o = (size_t)(t0 + min(tt, nt - 1)) * C + cl;
         const h16x4 xx4 = *(const h16x4 *)(a.xx + o), sd4 = *(const h16x4 *)(a.sxd + o);
         h16x4 out4;
+        float a0 = 0.f, a2 = 0.f;
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
             const float xx = (float)xx4[e];
             const float mm = round_h((float)maa[e] + round_h(m[tt][e]));
             out4[e] = (h16)(xx + round_h((float)sd4[e] * mm));
+            if (scaled) {
+                const float kf = (float)out4[e];
+                out4[e] = (h16)(kf * (float)ry4[e]);
+                a0 += kf;
+                a2 += kf * (float)my4[e];
+            }
         }
-        if (tt < nt) *(h16x4 *)(a.out[j] + o) = out4;
+        sums[2 * tt] = live ? a0 : 0.f;
+        sums[2 * tt + 1] = live ? a2 : 0.f;
+        if (tt < nt && live) *(h16x4 *)(a.out[j] + o) = out4;
+    }
+    if (scaled) {
+        __shared__ float red[2 * TT * 4];
+        block_sum_n<2 * TT>(sums, red);
+        if (threadIdx.x < nt) {
+            const size_t pi = (size_t)(t0 + threadIdx.x) * a.npart;
+            float s0 = 0.f, s2 = 0.f;
+#pragma unroll
+            for (int tt = 0; tt < TT; ++tt)
+                if (tt == (int)threadIdx.x) { s0 = sums[2 * tt]; s2 = sums[2 * tt + 1]; }
+            a.p0[j][pi + blockIdx.y] = s0;
+            a.p2[j][pi + blockIdx.y] = s2;
+            if (blockIdx.y == 0)
+                for (int q = gridDim.y; q < a.npart; ++q) { a.p0[j][pi + q] = 0.f; a.p2[j][pi + q] = 0.f; }
+        }
     }
 }
 
@@ -201,10 +237,14 @@ struct Ws56 {
     rwkv_half *x, *xx, *sxd, *xxx, *t1, *mix[5], *d1, *d2, *r, *k, *v, *g, *att, *vx, *xs, *xx_att, *xx_ffn;
     float *sums, *splitk, *y32;
     float *parts;            // partial row sums handed from the key product's epilogue to the value product
+    float *att_parts[4];     // RWKV-6: totals scratch + partial row sums of the scaled key / value / receptance / gate inputs
     rwkv_half *xs_side[3];   // scaled-activation scratch of the products that run beside the first one [T, C]
     float *sums_side[3];
     size_t total;
 };
+
+// partial sums per row that v6_mix2x4_kernel writes: one per block of 1024 channels, rounded up to a multiple of four
+int mix_parts(int64_t C) { return (int)((((C + 1023) / 1024) + 3) & ~(int64_t)3); }
 
 Ws56 carve56(void *base, int64_t T, int64_t C, int64_t F, int64_t lm, int64_t ld) {
     Ws56 w;
@@ -226,6 +266,7 @@ Ws56 carve56(void *base, int64_t T, int64_t C, int64_t F, int64_t lm, int64_t ld
     w.splitk = (float *)take(RWKV_SPLITK_WS_BYTES);
     w.y32 = (float *)take(T >= 32 ? (size_t)T * C * 4 : 256);
     w.parts = (float *)take(T > 1 ? (size_t)T * 2 * ((F + 127) / 128) * sizeof(float) : 256);
+    for (int j = 0; j < 4; ++j) w.att_parts[j] = (float *)take(T > 1 ? (size_t)T * (2 + 2 * mix_parts(C)) * sizeof(float) : 256);
     w.total = (size_t)(p - (unsigned char *)base);
     return w;
 }
@@ -319,6 +360,9 @@ extern "C" int rwkv_v56_forward(const rwkv_v56_model *m, const rwkv_v56_layer_st
         const bool dma_seq = T >= 512;
         const rwkv_half *kx, *vx, *rx, *gx = nullptr, *wx = nullptr;
         bool fuse_d1 = false, att_scaled = false;
+        int att_np = 0;   // RWKV-6: > 0 = the mixes arrive scaled, with this many partial row sums each
+        // receptance, key, value (and gate) as one grouped launch (see below)
+        const bool grouped = T > 1 && (T >= 256 || (!ss && ((T + 127) / 128) * (C / 128) <= 128)) && !(C & 127);
         float *att_sums[4] = {ws.sums, ws.sums_side[0], ws.sums_side[1], ws.sums_side[2]};   // of kx, vx, rx, gx
         if (v6) {
             Mix2Args b{};
@@ -340,6 +384,22 @@ extern "C" int rwkv_v56_forward(const rwkv_v56_model *m, const rwkv_v56_layer_st
             }
             b.T = (int)T; b.C = C; b.R = lm; b.t1 = ws.t1; b.w2 = l.tm_w2;
             for (int j = 0; j < 5; ++j) { b.maa[j] = l.att_mix[1 + j]; b.out[j] = ws.mix[j]; }
+            // uint8 matrices, the four products as one grouped direct-to-LDS launch: the mixing kernel writes their
+            // inputs already scaled, with partial row sums that the grouped launch adds up -- no scaling pass
+            if (T > 1 && u8 && grouped && !(C & 3) && lm <= 64 && handover_enabled()) {
+                const rwkv_half *xin[4] = {ws.mix[3], ws.mix[1], ws.mix[2], ws.mix[4]};
+                const rwkv_mat *mats[4] = {&l.att_receptance, &l.att_key, &l.att_value, &l.att_gate};
+                void *outs[4] = {ws.r, ws.k, ws.v, ws.g};
+                if (gemm_group_takes_parts(true, 4, T, C, xin, mats, outs)) {
+                    att_np = mix_parts(C);
+                    const rwkv_mat *mj[5] = {nullptr, &l.att_key, &l.att_value, &l.att_receptance, &l.att_gate};
+                    b.npart = att_np;
+                    for (int j = 1; j < 5; ++j) {
+                        b.ry[j] = mj[j]->ry; b.my[j] = mj[j]->my;
+                        b.p0[j] = ws.att_parts[j - 1] + 2 * T; b.p2[j] = b.p0[j] + (size_t)T * att_np;
+                    }
+                }
+            }
             if (T == 1) hipLaunchKernelGGL(v6_mix2_kernel<1>, dim3(1, (unsigned)((C + 255) / 256), 5), dim3(256), 0, st, b);
             else if (!(C & 3) && lm <= 64) {
                 if (T <= 512) hipLaunchKernelGGL(v6_mix2x4_kernel<4>, dim3((unsigned)((T + 3) / 4), (unsigned)((C + 1023) / 1024), 5), dim3(256), 0, st, b);
@@ -384,7 +444,7 @@ extern "C" int rwkv_v56_forward(const rwkv_v56_model *m, const rwkv_v56_layer_st
             // One grouped launch at full depth for receptance, key, value (and gate): in short calls, where each
             // product alone would split K and need a reduction pass, and from 256 rows on, where the group goes
             // through the direct-to-LDS kernel (256 x 256 tiles, K split while the group has few tiles).
-            if ((T >= 256 || (!ss && ((T + 127) / 128) * (C / 128) <= 128)) && !(C & 127)) {
+            if (grouped) {
                 const int n = gated ? 4 : 3;
                 const rwkv_half *xin[4] = {rx, kx, vx, gx};
                 const rwkv_mat *mats[4] = {&l.att_receptance, &l.att_key, &l.att_value, &l.att_gate};
@@ -398,9 +458,11 @@ extern "C" int rwkv_v56_forward(const rwkv_v56_model *m, const rwkv_v56_layer_st
                     ep[j].ldres = C; ep[j].ldgate = C;
                 }
                 float *smx[4] = {att_sums[2], att_sums[0], att_sums[1], att_sums[3]};
-                if ((rc = gemm_group_launch(u8, n, T, C, xin, mats, outs, ep, att_scaled ? nullptr : xsc, att_scaled ? smx : sm,
-                                            ws.splitk, st)))
-                    return rc;
+                float *smp[4] = {ws.att_parts[2], ws.att_parts[0], ws.att_parts[1], ws.att_parts[3]};
+                if (att_np) rc = gemm_group_launch(u8, n, T, C, xin, mats, outs, ep, nullptr, smp, ws.splitk, st, att_np);
+                else rc = gemm_group_launch(u8, n, T, C, xin, mats, outs, ep, att_scaled ? nullptr : xsc, att_scaled ? smx : sm,
+                                            ws.splitk, st);
+                if (rc) return rc;
             } else if (att_scaled) {
                 if ((rc = mm_scaled(c, l.att_receptance, u8, rx, att_sums[2], att_sums[2] + T, ACT_NONE, nullptr, nullptr, 1.f, ws.r)) ||
                     (rc = mm_scaled(c, l.att_key, u8, kx, att_sums[0], att_sums[0] + T, ACT_NONE, nullptr, nullptr, 1.f, ws.k)) ||
