@@ -664,6 +664,36 @@ def test_full_width_oracle_parity(shape, V, capsys):
         assert np.abs(_np(s) - ref).max() <= 1e-2 * scale, (i, np.abs(_np(s) - ref).max(), scale)
 
 
+@pytest.mark.parametrize("shape", ["v4-7b", "v6-7b"])
+def test_handover_against_scaling_pass(shape, monkeypatch):
+    """Sequence calls at the 7B widths with uint8 weights hand the channel-mix value product (and RWKV-6's four
+    time-mix products) their input already scaled, with the row sums as partial sums that the consuming launch adds
+    up; RWKV_HANDOVER=0 keeps the separate scaling passes, whose results the oracle tests pin.  Same arithmetic per
+    element, another summation order for the row sums: logits and states of the two forms agree far inside the
+    parity tolerance, in calls of 256 (small tiles, K split, partial sums in two rounds) and 1024 tokens (large
+    tiles), and each form is deterministic."""
+    version, _, C, F, _ = synth.SHAPES[shape]
+    V = 5003
+    ck = synth.make_checkpoint(version=version, n_layer=2, n_embd=C, n_ffn=F, vocab=V, seed=23, affine=True, device="cuda:0")
+    m = _rwkv()(ck, "cuda fp16i8", verbose=False)
+    del ck
+    for T in (256, 1024):
+        toks = synth.random_tokens(T, V, seed=T)
+        monkeypatch.setenv("RWKV_HANDOVER", "0")
+        ref, rst = m.forward(toks, None)
+        monkeypatch.delenv("RWKV_HANDOVER")
+        out, st = m.forward(toks, None)
+        out2, st2 = m.forward(toks, None)
+        assert torch.equal(out, out2)
+        for a, b in zip(st, st2):
+            assert torch.equal(a, b)
+        scale = float(ref.abs().max())
+        assert float((out - ref).abs().max()) <= 2e-3 * max(scale, 1.0), (T, float((out - ref).abs().max()), scale)
+        for i, (a, b) in enumerate(zip(st, rst)):
+            s = max(float(b.float().abs().max()), 1.0)
+            assert float((a.float() - b.float()).abs().max()) <= 2e-3 * s, (T, i)
+
+
 @pytest.mark.parametrize("L", [8, 32])
 def test_depth_oracle_parity(L, capsys):
     """Eight layers, and all 32 layers, of the 7B RWKV-4 shape under 'cuda fp16i8' against the oracle (short vocabulary;

@@ -187,7 +187,11 @@ def test_mm8_linearity_full_size():
                                    (4096, 4096, 1024), (4096, 8192, 520), (128, 4096, 1024),
                                    (128, 200, 37), (192, 1000, 300), (64, 8, 2),
                                    # 2 .. 16 rows: the streaming kernel
-                                   (768, 768, 3), (4096, 4096, 16), (16384, 4096, 5), (2560, 10240, 11), (128, 211, 2), (2048, 512, 6)])
+                                   (768, 768, 3), (4096, 4096, 16), (16384, 4096, 5), (2560, 10240, 11), (128, 211, 2), (2048, 512, 6),
+                                   # narrow outputs of a LoRA's first stage (17 .. 512 rows, up to 192 outputs, fp16 out):
+                                   # ragged rows, an output count that is no multiple of 16, a row length that is no
+                                   # multiple of the 512 values one round of the eight waves covers, the row limit
+                                   (4096, 160, 256), (4096, 64, 37), (5120, 100, 300), (1056, 192, 512), (4096, 128, 17)])
 @pytest.mark.parametrize("out_dtype", [torch.float16, torch.float32])
 def test_gemm_f16(N, M, B, out_dtype):
     ops = _ops()
