@@ -39,35 +39,73 @@ struct Prep7Args {
     float *rk;                                // [T, H] bonus factor, fp16-rounded
 };
 
-// One wave per (token, head), lane = channel of the head.  Every step rounds to fp16 where an fp16
-// tensor operation of the reference does.
+// Eight adjacent channels per lane (16-byte accesses), so the eight lanes of a row of eight own one head of one
+// token: grid-stride over the T * C / 8 chunks.  Every step rounds to fp16 where an fp16 tensor operation of the
+// reference does; the two sums over a head run over a lane's eight channels in index order and then over the
+// eight lanes in three DPP steps.
+DEV float head8_sum(float v) {
+    v += dpp_mov<0xB1>(v);    // quad_perm [1,0,3,2]
+    v += dpp_mov<0x4E>(v);    // quad_perm [2,3,0,1]
+    v += dpp_mov<0x141>(v);   // row_half_mirror: the other quad of the eight
+    return v;
+}
+
 __global__ __launch_bounds__(256) void prep7_kernel(Prep7Args a) {
-    const int64_t wave = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (wave >= (int64_t)a.T * a.H) return;
-    const int lane = threadIdx.x & 63;
-    const int64_t t = wave / a.H;
-    const int h = (int)(wave - t * a.H);
-    const int c = h * HS7 + lane;
-    const size_t o = (size_t)t * a.C + c;
-    const float r = h2f(a.r[o]), k = h2f(a.k[o]);
-    float v = h2f(a.v[o]);
-    const float av = round_h(sigmoidf_(round_h(h2f(a.a0[c]) + h2f(a.a_raw[o]))));
-    const float kku = round_h(k * h2f(a.k_k[c]));
-    const float nrm = fmaxf(round_h(sqrtf(wave_sum(kku * kku))), 1e-12f);
-    const float kk = round_h(kku / nrm);
-    const float k2 = round_h(k * round_h(1.f + round_h(round_h(av - 1.f) * h2f(a.k_a[c]))));
-    if (a.vg_raw) {
-        const float sg = round_h(sigmoidf_(round_h(h2f(a.v0[c]) + h2f(a.vg_raw[o]))));
-        v = round_h(v + round_h(round_h(h2f(a.v_first[o]) - v) * sg));
-        a.v[o] = f2h(v);
+    const int64_t nchunk = (int64_t)a.T * a.C / 8;
+    const int cpr = a.C / 8;   // chunks per token row
+    // whole waves take part in the DPP sums: chunks past the end repeat the last one and store nothing
+    for (int64_t i0 = (int64_t)blockIdx.x * 256; i0 < nchunk; i0 += (int64_t)gridDim.x * 256) {
+        const int64_t i = i0 + threadIdx.x;
+        const bool live = i < nchunk;
+        const int64_t ic = live ? i : nchunk - 1;
+        const int64_t t = ic / cpr;
+        const int c = (int)(ic - t * cpr) * 8;
+        const size_t o = (size_t)t * a.C + c;
+        const h16x8 r8 = *(const h16x8 *)(a.r + o), k8 = *(const h16x8 *)(a.k + o), v8 = *(const h16x8 *)(a.v + o);
+        const h16x8 ar8 = *(const h16x8 *)(a.a_raw + o), wr8 = *(const h16x8 *)(a.w_raw + o);
+        h16x8 vg8 = {}, vf8 = {}, v08 = {};
+        if (a.vg_raw) { vg8 = *(const h16x8 *)(a.vg_raw + o); vf8 = *(const h16x8 *)(a.v_first + o); v08 = *(const h16x8 *)(a.v0 + c); }
+        const h16x8 a08 = *(const h16x8 *)(a.a0 + c), kk8 = *(const h16x8 *)(a.k_k + c), ka8 = *(const h16x8 *)(a.k_a + c);
+        const h16x8 w08 = *(const h16x8 *)(a.w0 + c), rk8 = *(const h16x8 *)(a.r_k + c);
+        float av[8], kku[8], k2[8], ss = 0.f, rks = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const float k = (float)k8[e];
+            av[e] = round_h(sigmoidf_(round_h((float)a08[e] + (float)ar8[e])));
+            kku[e] = round_h(k * (float)kk8[e]);
+            ss += kku[e] * kku[e];
+            k2[e] = round_h(k * round_h(1.f + round_h(round_h(av[e] - 1.f) * (float)ka8[e])));
+            rks += round_h(round_h((float)r8[e] * k2[e]) * (float)rk8[e]);
+        }
+        const float nrm = fmaxf(round_h(sqrtf(head8_sum(ss))), 1e-12f);
+        rks = head8_sum(rks);
+        h16x8 ko, ano, bo, vo = v8;
+        f32x4 d0, d1;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const float kk = round_h(kku[e] / nrm);
+            if (a.vg_raw) {
+                const float v = (float)v8[e];
+                const float sg = round_h(sigmoidf_(round_h((float)v08[e] + (float)vg8[e])));
+                vo[e] = (h16)(v + round_h(round_h((float)vf8[e] - v) * sg));
+            }
+            const float z = round_h((float)w08[e] + (float)wr8[e]);
+            const float dec = __expf(-0.606531f * sigmoidf_(z));
+            if (e < 4) d0[e] = dec; else d1[e - 4] = dec;
+            ko[e] = (h16)k2[e];
+            ano[e] = (h16)(-kk);
+            bo[e] = (h16)(kk * av[e]);
+        }
+        if (live) {
+            if (a.vg_raw) *(h16x8 *)(a.v + o) = vo;
+            *(f32x4 *)(a.dec + o) = d0;
+            *(f32x4 *)(a.dec + o + 4) = d1;
+            *(h16x8 *)(a.k + o) = ko;
+            *(h16x8 *)(a.an + o) = ano;
+            *(h16x8 *)(a.b + o) = bo;
+            if (!(c & (HS7 - 1))) a.rk[t * a.H + c / HS7] = round_h(rks);
+        }
     }
-    const float z = round_h(h2f(a.w0[c]) + h2f(a.w_raw[o]));
-    a.dec[o] = __expf(-0.606531f * sigmoidf_(z));
-    a.k[o] = f2h(k2);
-    a.an[o] = f2h(-kk);
-    a.b[o] = f2h(kk * av);
-    const float rk = wave_sum(round_h(round_h(r * k2) * h2f(a.r_k[c])));
-    if (lane == 0) a.rk[wave] = round_h(rk);
 }
 
 struct Wkv7Args {
@@ -735,7 +773,8 @@ extern "C" int rwkv_v7_forward(const rwkv_v7_model *m, const rwkv_v56_layer_stat
             a.vg_raw = i > 0 ? ws.vg_raw : nullptr; a.v_first = i > 0 ? ws.v_first : nullptr;
             a.w0 = l.w0; a.a0 = l.a0; a.v0 = l.v0; a.k_k = l.k_k; a.k_a = l.k_a; a.r_k = l.r_k;
             a.an = ws.an; a.b = ws.b; a.dec = ws.dec; a.rk = ws.rk;
-            hipLaunchKernelGGL(prep7_kernel, dim3(head_waves), dim3(256), 0, st, a);
+            const int64_t blocks = ((int64_t)T * C / 8 + 255) / 256;
+            hipLaunchKernelGGL(prep7_kernel, dim3((unsigned)std::min<int64_t>(blocks, 65535)), dim3(256), 0, st, a);
         }
         {
             Wkv7Args q{(int)T, C, s.att_kv, ws.r, ws.dec, ws.k, v, ws.an, ws.b, ws.y32};
