@@ -756,16 +756,65 @@ extern "C" int rwkv_v7_forward(const rwkv_v7_model *m, const rwkv_v56_layer_stat
         if ((rc = mm(cm, l.att_key, false, xk, ACT_NONE, nullptr, nullptr, 1.f, ws.k))) return rc;
         if ((rc = mm(cv, l.att_value, false, xv, ACT_NONE, nullptr, nullptr, 1.f, v))) return rc;
         }
-        if ((rc = mm(cl, lora_first(l, 0, m->lora_w), false, xw, ACT_TANH, nullptr, nullptr, 1.f, ws.lw))) return rc;
-        if ((rc = mm(cl, lora_second(l, 0, m->lora_w), false, ws.lw, ACT_NONE, nullptr, nullptr, 1.f, ws.w_raw))) return rc;
-        if ((rc = mm(cl, lora_first(l, o_a, m->lora_a), false, xa, ACT_NONE, nullptr, nullptr, 1.f, ws.la))) return rc;
-        if ((rc = mm(cl, lora_second(l, o_a, m->lora_a), false, ws.la, ACT_NONE, nullptr, nullptr, 1.f, ws.a_raw))) return rc;
-        if (i > 0) {
-            if ((rc = mm(cl, lora_first(l, o_v, m->lora_v), false, xv, ACT_NONE, nullptr, nullptr, 1.f, ws.lv))) return rc;
-            if ((rc = mm(cl, lora_second(l, o_v, m->lora_v), false, ws.lv, ACT_NONE, nullptr, nullptr, 1.f, ws.vg_raw))) return rc;
+        // The LoRA products: the first stages (same input width, their own inputs, ranks and activations) as one
+        // grouped launch, then the second stages -- those of equal rank as one grouped launch, the others one by one.
+        // RWKV_V7_LORA_GROUPS=0 launches all eight one by one (tuning).
+        {
+            const bool has_v = i > 0;
+            struct Stage { const rwkv_half *x; int off, d, act; rwkv_half *l1, *out; };
+            const Stage sg[4] = {{xw, 0, m->lora_w, ACT_TANH, ws.lw, ws.w_raw},
+                                 {xa, o_a, m->lora_a, ACT_NONE, ws.la, ws.a_raw},
+                                 {xv, o_v, m->lora_v, ACT_NONE, ws.lv, ws.vg_raw},
+                                 {xg, o_g, m->lora_g, ACT_SIGMOID, ws.lg, ws.g}};
+            const char *env = getenv("RWKV_V7_LORA_GROUPS");
+            const bool groups = !(env && *env == '0') && !(C & 7);
+            bool first_done[4] = {false, false, false, false}, second_done[4] = {false, false, false, false};
+            if (groups) {
+                const rwkv_half *xin[4];
+                rwkv_mat mt[4];
+                const rwkv_mat *mp[4];
+                void *outs[4];
+                GemmEpi ep[4] = {};
+                int n = 0, idx[4];
+                for (int q = 0; q < 4; ++q) {
+                    if (q == 2 && !has_v) continue;
+                    xin[n] = sg[q].x; mt[n] = lora_first(l, sg[q].off, sg[q].d); mp[n] = &mt[n]; outs[n] = sg[q].l1;
+                    ep[n].act = sg[q].act; ep[n].out_scale = 1.f; ep[n].out_dtype = RWKV_DT_F16;
+                    idx[n++] = q;
+                }
+                if ((rc = gemm_group_launch(false, n, T, C, xin, mp, outs, ep, nullptr, nullptr, cl.splitk, cl.st))) return rc;
+                for (int q = 0; q < n; ++q) first_done[idx[q]] = true;
+                // second stages of the most common rank together
+                int best = -1, best_n = 0;
+                for (int q = 0; q < 4; ++q) {
+                    if (q == 2 && !has_v) continue;
+                    int cnt = 0;
+                    for (int r = 0; r < 4; ++r) cnt += (r != 2 || has_v) && sg[r].d == sg[q].d;
+                    if (cnt > best_n) { best_n = cnt; best = q; }
+                }
+                if (best_n >= 2 && !(sg[best].d % 64)) {
+                    n = 0;
+                    for (int q = 0; q < 4; ++q) {
+                        if ((q == 2 && !has_v) || sg[q].d != sg[best].d) continue;
+                        xin[n] = sg[q].l1; mt[n] = lora_second(l, sg[q].off, sg[q].d); mp[n] = &mt[n]; outs[n] = sg[q].out;
+                        ep[n] = GemmEpi{};
+                        ep[n].act = ACT_NONE; ep[n].out_scale = 1.f; ep[n].out_dtype = RWKV_DT_F16;
+                        idx[n++] = q;
+                    }
+                    if ((rc = gemm_group_launch(false, n, T, sg[best].d, xin, mp, outs, ep, nullptr, nullptr, cl.splitk, cl.st))) return rc;
+                    for (int q = 0; q < n; ++q) second_done[idx[q]] = true;
+                }
+            }
+            for (int q = 0; q < 4; ++q) {
+                if (q == 2 && !has_v) continue;
+                if (!first_done[q] &&
+                    (rc = mm(cl, lora_first(l, sg[q].off, sg[q].d), false, sg[q].x, sg[q].act, nullptr, nullptr, 1.f, sg[q].l1)))
+                    return rc;
+                if (!second_done[q] &&
+                    (rc = mm(cl, lora_second(l, sg[q].off, sg[q].d), false, sg[q].l1, ACT_NONE, nullptr, nullptr, 1.f, sg[q].out)))
+                    return rc;
+            }
         }
-        if ((rc = mm(cl, lora_first(l, o_g, m->lora_g), false, xg, ACT_SIGMOID, nullptr, nullptr, 1.f, ws.lg))) return rc;
-        if ((rc = mm(cl, lora_second(l, o_g, m->lora_g), false, ws.lg, ACT_NONE, nullptr, nullptr, 1.f, ws.g))) return rc;
         if (!par.join()) return (int)hipErrorUnknown;
         {
             Prep7Args a{};
