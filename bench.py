@@ -5,7 +5,7 @@
 Workload (the headline configuration): random-init 32-layer / n_embd 4096 / ffn 16384 / vocab
 50277 model, prefill of 1024 uniform-random tokens in one call, then greedy decode.  A "step"
 is one decoded token (one pass of forward([token], state)); W untimed steps, then exactly K
-timed steps with the next token taken on the device (argmax) so the loop has no host
+timed steps with the next token taken on the device (rwkv_greedy_token: argmax of the logits) so the loop has no host
 synchronisation; the same K steps are also timed with a host sync per token.
 
 One JSON line is printed:
@@ -316,6 +316,8 @@ def main():
     ap.add_argument("--chunk", type=int, default=0, help="prefill in calls of this many tokens (0: one call)")
     ap.add_argument("--layers", type=int, default=None, help="debug: fewer layers (result is then not the headline)")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--select", choices=["greedy", "torch"], default="greedy",
+                    help="next token on the device by rwkv_greedy_token (one launch) or by torch's argmax + conversion")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run five plain 1 GiB device copies (a kernel of known HBM traffic, for scaling "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE counters)")
@@ -376,18 +378,23 @@ def main():
     prefill_flops = 2.0 * args.prefill * (wbytes / (1 if u8 else 2) - C * V) + 2.0 * C * V
 
     # ---- decode: W warm-up + K timed greedy steps, token stays on the device
-    tok = out.argmax().reshape(1).to(torch.int32)
+    if args.select == "greedy":
+        from chatrwkv_amd.sampling import greedy_token as pick
+    else:
+        def pick(logits, into=None):
+            return logits.argmax().reshape(1).to(torch.int32)
+    tok = pick(out)
     def one_step():
         nonlocal out, state, tok
         out, state = model.forward(tok, state)
-        tok = out.argmax().reshape(1).to(torch.int32)
+        tok = pick(out, tok)
     for _ in range(args.warmup):
         one_step()
     n_spin = spin_up(one_step, args.spinup, sync_every=64)
     t0 = time.perf_counter()
     for _ in range(args.steps):
         out, state = model.forward(tok, state)
-        tok = out.argmax().reshape(1).to(torch.int32)
+        tok = pick(out, tok)
     torch.cuda.synchronize()
     t_dev = time.perf_counter() - t0
 
@@ -448,7 +455,9 @@ def main():
         "config": {"workload": f"RWKV-{int(version)} {args.shape} ({L} layers, n_embd {C}, ffn {F}, vocab {V}) '{args.strategy}', "
                                f"batch 1: prefill {args.prefill} tokens in {'one call' if chunk >= args.prefill else f'calls of {chunk}'}, "
                                f"then greedy decode" + (" (BASELINE.json configs[2])" if args.shape == "v4-7b" else ""),
-                   "strategy": args.strategy, "prefill_tokens": args.prefill},
+                   "strategy": args.strategy, "prefill_tokens": args.prefill,
+                   "next_token": "rwkv_greedy_token (argmax of the logits, one launch, id stays on the device)"
+                                 if args.select == "greedy" else "torch argmax + conversion to int32 on the device"},
         "roofline": roof,
         "decode_hbm": {"weight_bytes_per_token": wbytes, "achieved_GBps": wbytes * tok_s / 1e9,
                        "frac_of_peak": wbytes * tok_s / HBM_PEAK},

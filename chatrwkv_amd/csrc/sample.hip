@@ -190,6 +190,52 @@ __global__ __launch_bounds__(STHREADS) void sample_kernel(SampleArgs a) {
 
 }  // namespace
 
+// The temperature-0 draw without penalties or bans: the index of the largest logit, the lowest such index on
+// ties (NaN entries are never chosen).  One workgroup; each thread scans a strided share of the vocabulary with
+// eight loads in flight, then (value, index) pairs are reduced by wave shuffles and across the 16 waves in LDS.
+template <bool F16>
+__global__ __launch_bounds__(STHREADS) void greedy_kernel(const void *__restrict__ logits_, int V, int32_t *__restrict__ token) {
+    const float *lf = (const float *)logits_;
+    const rwkv_half *lh = (const rwkv_half *)logits_;
+    __shared__ float rv[SWAVES];
+    __shared__ int ri[SWAVES];
+    float best = -__builtin_inff();
+    int bi = 0x7fffffff;
+    auto take = [&](float v, int i) {
+        if (v > best || (v == best && i < bi)) { best = v; bi = i; }
+    };
+    for (int i0 = threadIdx.x; i0 < V; i0 += 8 * STHREADS) {
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int i = min(i0 + u * STHREADS, V - 1);
+            v[u] = F16 ? h2f(lh[i]) : lf[i];
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            if (i0 + u * STHREADS < V) take(v[u], i0 + u * STHREADS);
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) take(__shfl_xor(best, o, WAVE), __shfl_xor(bi, o, WAVE));
+    const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
+    if (lane == 0) { rv[wid] = best; ri[wid] = bi; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < SWAVES; ++w) take(rv[w], ri[w]);
+        *token = bi == 0x7fffffff ? 0 : bi;
+    }
+}
+
+extern "C" int rwkv_greedy_token(const void *logits, int dtype, int64_t V, int32_t *token, void *stream) {
+    if (!logits || !token) return RWKV_E_NULL;
+    if (V <= 0 || V > 0x7fffffff) return RWKV_E_SHAPE;
+    if (dtype == RWKV_DT_F32) hipLaunchKernelGGL(greedy_kernel<false>, dim3(1), dim3(STHREADS), 0, (hipStream_t)stream, logits, (int)V, token);
+    else if (dtype == RWKV_DT_F16) hipLaunchKernelGGL(greedy_kernel<true>, dim3(1), dim3(STHREADS), 0, (hipStream_t)stream, logits, (int)V, token);
+    else return RWKV_E_DTYPE;
+    RWKV_LAUNCH_CHECK();
+    return RWKV_OK;
+}
+
 extern "C" int rwkv_sample_logits(const float *logits, int64_t V, float temperature, float top_p, int32_t top_k,
                                   const int32_t *token_ban, int32_t n_ban, uint8_t *seen, float *occurrence,
                                   const float *token_weight, float alpha_presence, float alpha_frequency,

@@ -40,6 +40,7 @@ SIGNATURES = {
     "rwkv_gemm_f16": (_int, [_i64, _i64, _i64, _vp, _i64, _vp, _i64, _i64, _vp, _i64, _int, _vp]),
     "rwkv_gemm_f16_batched": (_int, [_i64, _i64, _i64, _i64, _vp, _i64, _i64, _vp, _i64, _i64, _i64, _vp, _i64, _i64, _int, _vp]),
     "rwkv_release_stream": (_int, [_vp]),
+    "rwkv_greedy_token": (_int, [_vp, _int, _i64, _vp, _vp]),
     "rwkv_wkv4_forward": (_int, [_i64, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _int, _vp, _vp, _vp, _vp]),
     "rwkv_wkv5_forward": (_int, [_i64, _i64, _i64, _i64, _vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "rwkv_wkv6_forward": (_int, [_i64, _i64, _i64, _i64, _vp, _int, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),

@@ -85,6 +85,19 @@ class Sampler:
         return self.token
 
 
+def greedy_token(logits, out=None):
+    """The temperature-0 draw of sample_logits (utils.py:56-58) without penalties, i.e. ``logits.argmax()``, as one
+    launch: returns the int32 device tensor [1] with the index of the largest logit (``out`` if given), which the
+    next ``forward`` takes as its token without a copy to the host."""
+    if logits.dtype not in (torch.float32, torch.float16) or not logits.is_cuda or logits.dim() != 1 or not logits.is_contiguous():
+        raise _lib.RwkvHipError("greedy_token() takes the contiguous fp32 or fp16 logits [vocab] on the GPU")
+    if out is None:
+        out = torch.empty(1, dtype=torch.int32, device=logits.device)
+    dt = _lib.RWKV_DT_F32 if logits.dtype == torch.float32 else _lib.RWKV_DT_F16
+    _lib.check(_lib.load().rwkv_greedy_token(logits.data_ptr(), dt, logits.numel(), out.data_ptr(), _stream()), "rwkv_greedy_token")
+    return out
+
+
 def sample_logits(logits, temperature=1.0, top_p=0.85, top_k=0, generator_seed=None):
     """PIPELINE.sample_logits (utils.py:55-88): returns the drawn id as a Python int."""
     s = Sampler(logits.numel(), device=logits.device, seed=generator_seed)

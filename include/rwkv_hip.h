@@ -188,6 +188,13 @@ int rwkv_sample_logits(const float *logits, int64_t V, float temperature, float 
                        const float *token_weight, float alpha_presence, float alpha_frequency, float alpha_decay,
                        const float *u, float *probs, int32_t *token, void *stream);
 
+/* The temperature-0 case of the same step without bans or penalties (rwkv/utils.py:56-58: top_p = 0 keeps the
+ * largest probability alone; what a greedy caller writes as logits.argmax()): token <- the index of the
+ * largest of logits [V] (dtype RWKV_DT_F32, or RWKV_DT_F16 as RWKV-7 returns them), the lowest such index on
+ * ties; NaN entries are never chosen.  One launch, no host synchronisation; token is a device int32 that the
+ * next one-token forward call can read. */
+int rwkv_greedy_token(const void *logits, int dtype, int64_t V, int32_t *token, void *stream);
+
 /* =======================================================================================
  * Model-level entry points: one call runs RWKV.forward (model.py:1443-1677) for RWKV-4 on
  * one GPU, with the elementwise chains of att_one / ffn_one / cuda_att_seq / ffn_seq

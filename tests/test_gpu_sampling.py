@@ -135,3 +135,31 @@ def test_generate_ids_on_tiny_model():
     stop = a[5]
     cut, _ = generate_ids(m, ctx, 24, PIPELINE_ARGS(temperature=1.0, top_p=0.8, token_ban=[0], token_stop=[stop]), seed=5)
     assert cut == a[:a.index(stop)]
+
+
+@pytest.mark.parametrize("vocab", [1, 7, 1000, 8192, 50277, 65536, 70001])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_greedy_token(vocab, dtype):
+    """rwkv_greedy_token, the temperature-0 draw without penalties (utils.py:56-58), against numpy's argmax (first
+    index of the maximum): random logits, the maximum repeated at several indices, NaN and -inf entries, all entries
+    equal; fp32 logits and the fp16 logits RWKV-7 returns; the id is written to the tensor given."""
+    from chatrwkv_amd import lib, sampling
+    x = logits_for(vocab, vocab, 3.0)
+    cases = [x.copy()]
+    if vocab >= 7:
+        y = x.copy(); y[[vocab - 1, vocab // 2, 3]] = 50.0; cases.append(y)            # ties: the lowest index
+        y = x.copy(); y[::3] = np.nan; y[1] = -np.inf; cases.append(y)                    # NaN is never chosen
+        y = x.copy(); y[vocab - 1] = 60.0; cases.append(y)                                # the last entry
+    cases.append(np.full(vocab, -1.25, np.float32))                                       # all equal: index 0
+    out = torch.full((1,), -7, dtype=torch.int32, device=DEV)
+    for c in cases:
+        t = torch.from_numpy(c).to(DEV).to(dtype)
+        ref = c.astype(np.float16 if dtype == torch.float16 else np.float32)
+        want = int(np.argmax(np.where(np.isnan(ref), -np.inf, ref)))
+        got = sampling.greedy_token(t, out)
+        assert got is out and int(out) == want, (vocab, int(out), want)
+        assert int(sampling.greedy_token(t)) == want
+    L = lib.load()
+    assert L.rwkv_greedy_token(None, lib.RWKV_DT_F32, 8, out.data_ptr(), None) == -3
+    assert L.rwkv_greedy_token(out.data_ptr(), lib.RWKV_DT_F32, 0, out.data_ptr(), None) == -1
+    assert L.rwkv_greedy_token(out.data_ptr(), 7, 8, out.data_ptr(), None) == -5
