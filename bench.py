@@ -383,7 +383,7 @@ def main():
     else:
         def pick(logits, into=None):
             return logits.argmax().reshape(1).to(torch.int32)
-    tok = pick(out)
+    tok = pick(out, model.token_slot)   # the id is written where the one-token step reads it: no copy per step
     def one_step():
         nonlocal out, state, tok
         out, state = model.forward(tok, state)

@@ -544,7 +544,8 @@ class RWKV:
 
     def _forward_one(self, token, state):
         if isinstance(token, torch.Tensor):
-            self._token_dev.copy_(token.reshape(1), non_blocking=True)
+            if token.data_ptr() != self._token_dev.data_ptr():   # the caller wrote the id into token_slot: nothing to copy
+                self._token_dev.copy_(token.reshape(1), non_blocking=True)
         else:
             # the id travels as a kernel argument of the fill: no host buffer that a later call
             # could overwrite while this one is still queued
@@ -627,6 +628,13 @@ class RWKV:
             _lib.check(rc, "forward (sequence mode)")
         self._run_segments(call)
         return logits, state
+
+    @property
+    def token_slot(self):
+        """The int32 device tensor [1] the one-token step reads its id from.  A sampler that writes the next id
+        here (``greedy_token(out, model.token_slot)``, ``Sampler.sample`` followed by a copy) and passes this
+        tensor to ``forward`` saves the step its copy of the id."""
+        return self._token_dev
 
     def forward(self, tokens, state, full_output=False):
         """model.py:1443-1677.  Returns (logits fp32 [vocab] or [T, vocab], state)."""

@@ -222,10 +222,18 @@ class RWKV_x070:
                                          torch.cuda.current_stream().cuda_stream)
         _lib.check(rc, "rwkv_v7_forward")
 
+    @property
+    def token_slot(self):
+        """The int32 device tensor [1] the one-token step reads its id from.  A sampler that writes the next id
+        here (``greedy_token(out, model.token_slot)``, ``Sampler.sample`` followed by a copy) and passes this
+        tensor to ``forward`` saves the step its copy of the id."""
+        return self._token_dev
+
     def forward_one(self, idx, state):
         """model.py:336-363."""
         if isinstance(idx, torch.Tensor):
-            self._token_dev.copy_(idx.reshape(1), non_blocking=True)
+            if idx.data_ptr() != self._token_dev.data_ptr():   # the caller wrote the id into token_slot: nothing to copy
+                self._token_dev.copy_(idx.reshape(1), non_blocking=True)
         else:
             idx = int(idx)
             if idx < 0 or idx >= self._model.vocab:

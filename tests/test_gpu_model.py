@@ -67,6 +67,30 @@ def test_converted_weights_match_oracle(tiny_models, strat):
         assert kw.stride(0) == 1  # input-contiguous storage
 
 
+def test_greedy_loop_through_the_token_slot(tiny_models):
+    """A greedy loop that writes each id into the model's token_slot with greedy_token and feeds that tensor back
+    draws the same ids and ends with the same logits and state as the loop that fetches int(out.argmax()) to the
+    host every step; a device tensor other than the slot is copied in as before."""
+    from chatrwkv_amd.sampling import greedy_token
+    m, _ = tiny_models["cuda fp16i8"]
+    toks = synth.random_tokens(7, TINY["vocab"], seed=PROMPT_SEED + 5)
+    out, st = m.forward(toks, None)
+    ids_host, o, s = [], out, st
+    for _ in range(12):
+        ids_host.append(int(o.argmax()))
+        o, s = m.forward([ids_host[-1]], s)
+    out, st = m.forward(toks, None)
+    ids_dev, o2, s2 = [], out, st
+    for i in range(12):
+        tok = greedy_token(o2, m.token_slot) if i % 3 else greedy_token(o2)   # every third id from a tensor of its own
+        ids_dev.append(int(tok))
+        o2, s2 = m.forward(tok, s2)
+    assert ids_dev == ids_host
+    assert torch.equal(o, o2)
+    for x, y in zip(s, s2):
+        assert torch.equal(x, y)
+
+
 @pytest.mark.parametrize("strat", ["cuda fp16i8", "cuda fp16"])
 def test_tiny_forward_parity(tiny_models, strat):
     m, o = tiny_models[strat]
