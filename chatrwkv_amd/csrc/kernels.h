@@ -72,10 +72,7 @@ int wkv56_fused_launch(bool v6, int T, int C, int H, float *state, const rwkv_ha
                        const rwkv_half *v, const void *w, const float *t_decay, const float *u, const float *lnx_w,
                        const float *lnx_b, const rwkv_half *gate, rwkv_half *out, hipStream_t st,
                        const rwkv_half *dw2 = nullptr, int ld = 0,  // dw2: v6 with w = tanh(. @ D1), product with D2 in-kernel
-                       float *y32 = nullptr,  // fp32 [T, C] scratch: calls of >= 32 tokens split each head over 4 workgroups
-                       const Wkv4Emit *emit = nullptr);  // those calls only (wkv56_can_emit): out scaled for the next
-                                                         // product (xs), partial sums per head in p0 / p2 [T][H]
-bool wkv56_can_emit(int64_t T);
+                       float *y32 = nullptr);  // fp32 [T, C] scratch: calls of >= 32 tokens split each head over 4 workgroups
 // Row-wise LayerNorm + token shift + mixes for up to 6 consumers over a [T, C] activation (seq_v4.hip).
 struct SeqMixArgs {
     int T, C;

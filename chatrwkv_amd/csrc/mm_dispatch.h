@@ -131,34 +131,6 @@ inline int mm_pair_second(const Ctx &c2, const rwkv_mat &m1, const rwkv_mat &m2,
     return gemm_launch(true, c2.T, M1, M2, c2.xs, M1, m2.w, m2.ld, out, M2, e2, c2.st);
 }
 
-// Sequence calls, uint8 matrix: would mm() run this product through the direct-to-LDS kernel, which can take the row
-// sums of an already scaled input as partial sums (mm_parts)?
-inline bool mm_takes_parts(const Ctx &c, const rwkv_mat &m, bool mat_u8, int act, const rwkv_half *res, const rwkv_half *gate,
-                           const rwkv_half *out) {
-    if (!mat_u8 || c.T <= 1 || !handover_enabled()) return false;
-    const int N = (int)m.N, M = (int)m.M;
-    GemmEpi e{};
-    e.act = act; e.res = res; e.ldres = M; e.gate = gate; e.ldgate = M; e.out_scale = 1.f;
-    e.out_dtype = RWKV_DT_F16; e.splitk_ws = c.splitk; e.splitk_bytes = RWKV_SPLITK_WS_BYTES;
-    e.small_tiles = c.small_tiles;
-    e.mx = m.mx; e.rx = m.rx; e.s0 = c.s0; e.s2 = c.s2;
-    return gemm_plan(true, c.T, N, M, c.xs, N, m.w, m.ld, out, M, e).kind == 2;
-}
-
-// The product of mm() for an input that arrives scaled in c.xs with np partial row sums per row in parts
-// ([T][np] of x, then [T][np] of x * my); np a multiple of four.
-inline int mm_parts(const Ctx &c, const rwkv_mat &m, const float *parts, int np, int act, const rwkv_half *res,
-                    const rwkv_half *gate, float out_scale, rwkv_half *out) {
-    const int N = (int)m.N, M = (int)m.M;
-    GemmEpi e{};
-    e.act = act; e.res = res; e.ldres = M; e.gate = gate; e.ldgate = M; e.out_scale = out_scale;
-    e.out_dtype = RWKV_DT_F16; e.splitk_ws = c.splitk; e.splitk_bytes = RWKV_SPLITK_WS_BYTES;
-    e.small_tiles = c.small_tiles;
-    e.mx = m.mx; e.rx = m.rx; e.s0 = c.s0; e.s2 = c.s2;
-    e.parts = np; e.p0 = parts; e.p2 = parts + (size_t)c.T * np;
-    return gemm_launch(true, c.T, N, M, c.xs, N, m.w, m.ld, out, M, e, c.st);
-}
-
 inline size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
 inline rwkv_mat lora_mat(const rwkv_half *w, int64_t N, int64_t M) {

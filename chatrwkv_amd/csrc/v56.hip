@@ -265,7 +265,7 @@ Ws56 carve56(void *base, int64_t T, int64_t C, int64_t F, int64_t lm, int64_t ld
     }
     w.splitk = (float *)take(RWKV_SPLITK_WS_BYTES);
     w.y32 = (float *)take(T >= 32 ? (size_t)T * C * 4 : 256);
-    w.parts = (float *)take(T > 1 ? (size_t)T * 2 * std::max<int64_t>((F + 127) / 128, C / 64) * sizeof(float) : 256);
+    w.parts = (float *)take(T > 1 ? (size_t)T * 2 * ((F + 127) / 128) * sizeof(float) : 256);
     for (int j = 0; j < 4; ++j) w.att_parts[j] = (float *)take(T > 1 ? (size_t)T * (2 + 2 * mix_parts(C)) * sizeof(float) : 256);
     w.total = (size_t)(p - (unsigned char *)base);
     return w;
@@ -484,19 +484,12 @@ extern "C" int rwkv_v56_forward(const rwkv_v56_model *m, const rwkv_v56_layer_st
         }
         // one token of v6: the second decay LoRA product is done inside the WKV kernel
         const bool d2_fused = v6 && T == 1;
-        // Calls that run GroupNorm as a launch of its own, output product through the direct-to-LDS kernel: that launch
-        // writes the product's input scaled, with one partial row sum per head -- no scaling pass.
-        Wkv4Emit em{};
-        const bool out_parts = wkv56_can_emit(T) && !(H & 3) && mm_takes_parts(c, l.att_output, u8, ACT_RESIDUAL, ws.x, nullptr, ws.x);
-        if (out_parts) em = Wkv4Emit{l.att_output.ry, l.att_output.my, c.xs, ws.parts, ws.parts + (size_t)T * H};
         if ((rc = wkv56_fused_launch(v6, (int)T, C, H, s.att_kv, ws.r, ws.k, ws.v,
                                      v6 ? (const void *)(d2_fused ? ws.d1 : ws.d2) : (const void *)l.time_decay, l.time_decay,
                                      l.time_first, l.lnx_w, l.lnx_b, gated ? ws.g : nullptr, ws.att, st,
-                                     d2_fused ? l.td_w2 : nullptr, ld, ws.y32, out_parts ? &em : nullptr)))
+                                     d2_fused ? l.td_w2 : nullptr, ld, ws.y32)))
             return rc;
-        if (out_parts) rc = mm_parts(c, l.att_output, ws.parts, H, ACT_RESIDUAL, ws.x, nullptr, 1.f, ws.x);
-        else rc = mm(c, l.att_output, u8, ws.att, ACT_RESIDUAL, ws.x, nullptr, 1.f, ws.x);
-        if (rc) return rc;
+        if ((rc = mm(c, l.att_output, u8, ws.att, ACT_RESIDUAL, ws.x, nullptr, 1.f, ws.x))) return rc;
         // ---- channel mix
         const float scale = (m->rescale_layer > 0 && (i + 1) % m->rescale_layer == 0) ? 0.5f : 1.f;
         if (T == 1) {

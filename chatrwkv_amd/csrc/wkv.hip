@@ -469,12 +469,9 @@ __global__ __launch_bounds__(256) void wkv56_split_kernel(Wkv56Args a) {
 }
 
 // GroupNorm over each head's 64 outputs (eps 64e-5), affine, fp16 rounding, gate: one wave per (token, head).
-// em.ry != NULL: the result goes out as fp16(value * ry) for the output product, with the sums of the value and of
-// value * my over the head in em.p0 / em.p2 [T][H].
 __global__ __launch_bounds__(256) void wkv56_gn_kernel(int T, int C, const float *__restrict__ y,
                                                        const float *__restrict__ lnx_w, const float *__restrict__ lnx_b,
-                                                       const rwkv_half *__restrict__ gate, rwkv_half *__restrict__ out,
-                                                       Wkv4Emit em) {
+                                                       const rwkv_half *__restrict__ gate, rwkv_half *__restrict__ out) {
     const int H = C / HS;
     const int64_t wave = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (wave >= (int64_t)T * H) return;
@@ -489,15 +486,9 @@ __global__ __launch_bounds__(256) void wkv56_gn_kernel(int T, int C, const float
     float gq = d * rsqrtf(var + 64e-5f) * lnx_w[h * HS + c] + lnx_b[h * HS + c];
     gq = round_h(gq);
     if (gate) gq = gq * h2f(gate[o]);
-    if (!em.ry) { out[o] = f2h(gq); return; }
-    const float yh = round_h(gq);
-    em.xs[o] = f2h(yh * h2f(em.ry[h * HS + c]));
-    const float a0 = wave_sum(yh), a2 = wave_sum(yh * h2f(em.my[h * HS + c]));
-    if (c == 0) { em.p0[wave] = a0; em.p2[wave] = a2; }
+    out[o] = f2h(gq);
 }
 
-
-bool wkv56_can_emit(int64_t T) { return T >= 32; }   // the calls that run GroupNorm as a launch of its own
 
 size_t wkv4_scratch_bytes(int64_t T, int64_t C) {
     if (T < 64) return 256;
@@ -561,9 +552,8 @@ static int wkv56_launch(bool v6, int64_t B, int64_t T, int64_t C, int64_t H, flo
 int wkv56_fused_launch(bool v6, int T, int C, int H, float *state, const rwkv_half *r, const rwkv_half *k,
                        const rwkv_half *v, const void *w, const float *t_decay, const float *u, const float *lnx_w,
                        const float *lnx_b, const rwkv_half *gate, rwkv_half *out, hipStream_t st,
-                       const rwkv_half *dw2, int ld, float *y32, const Wkv4Emit *emit) {
+                       const rwkv_half *dw2, int ld, float *y32) {
     if (C != H * HS) return RWKV_E_SHAPE;
-    if (emit && !(wkv56_can_emit(T) && y32 && emit->ry && emit->my && emit->xs && emit->p0 && emit->p2)) return RWKV_E_SHAPE;
     Wkv56Args a{};
     a.T = T; a.C = C; a.state = state; a.state_layout = 1;
     a.r = r; a.k = k; a.v = v; a.w = w; a.u = u; a.t_decay = t_decay;
@@ -575,7 +565,7 @@ int wkv56_fused_launch(bool v6, int T, int C, int H, float *state, const rwkv_ha
         else hipLaunchKernelGGL((wkv56_split_kernel<0>), dim3((unsigned)(4 * H)), dim3(256), 0, st, a);
         const int64_t waves = (int64_t)T * H;
         hipLaunchKernelGGL(wkv56_gn_kernel, dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, st, T, C, y32, lnx_w, lnx_b,
-                           gate, out, emit ? *emit : Wkv4Emit{});
+                           gate, out);
     } else if (v6 && dw2) {
         if (ld <= 0 || (ld & 7)) return RWKV_E_SHAPE;
         hipLaunchKernelGGL((wkv56_kernel<true, 3, true>), dim3((unsigned)H), dim3(256), 0, st, a);
