@@ -55,18 +55,9 @@ int mm8_prepare_launch(int64_t T, int64_t N, const rwkv_half *x, int64_t ldx, co
 int gemv_f16_launch(int64_t N, int64_t M, const rwkv_half *x, const rwkv_half *w, int64_t ldw, void *y,
                     int y_dtype, hipStream_t st);
 // kv_f32: k, v are fp32 (fp16-weight strategy) instead of fp16.
-// Output of the chunked scan as the scaled input of a uint8 product (GemmEpi::parts): xs = fp16(y * ry) instead of
-// y, and per token the sums of y and y * my over each block of 64 channels in p0 / p2 [T][C / 64].
-struct Wkv4Emit {
-    const rwkv_half *ry, *my;
-    rwkv_half *xs;
-    float *p0, *p2;
-};
-bool wkv4_can_emit(int64_t T, int64_t C);   // the chunked scan runs (T >= 64) and C is a multiple of 64
 int wkv4_fused_launch(int T, int C, const float *w, const float *u, const void *k, const void *v, int kv_f32,
                       const rwkv_half *r, rwkv_half *y, float *aa, float *bb, float *pp, hipStream_t st,
-                      float *scratch = nullptr,  // scratch (wkv4_scratch_bytes): long calls run as a chunked scan
-                      const Wkv4Emit *emit = nullptr);
+                      float *scratch = nullptr);  // scratch (wkv4_scratch_bytes): long calls run as a chunked scan
 size_t wkv4_scratch_bytes(int64_t T, int64_t C);
 int wkv56_fused_launch(bool v6, int T, int C, int H, float *state, const rwkv_half *r, const rwkv_half *k,
                        const rwkv_half *v, const void *w, const float *t_decay, const float *u, const float *lnx_w,

@@ -563,30 +563,17 @@ extern "C" int rwkv_v4_forward_seq(const rwkv_v4_model *m, const rwkv_v4_layer_s
         if ((rc = run_gemm(l.att_receptance, u8, T, ws.xs[2], s0[2], s2[2], ws.r, C, e, sr, sk))) return rc;
         if (!par.join()) return (int)hipErrorUnknown;
         }
-        // Where the chunked scan runs and the output product goes through the direct-to-LDS kernel, the scan writes
-        // r * wkv already scaled for that product, with one partial row sum per 64 channels: no scaling pass.
-        int aparts = 0;
-        Wkv4Emit em{};
-        e.act = ACT_RESIDUAL; e.res = ws.x; e.ldres = C;
-        if (u8 && wkv4_can_emit(T, C) && !((C >> 6) & 3) && handover_enabled() &&
-            plan_gemm(l.att_output, true, T, ws.xs[0], s0[0], s2[0], ws.x, C, e, ws.splitk).kind == 2) {
-            aparts = C >> 6;
-            em = Wkv4Emit{l.att_output.ry, l.att_output.my, ws.xs[0], ws.parts, ws.parts + (size_t)T * aparts};
-        }
         if ((rc = wkv4_fused_launch((int)T, C, l.time_decay, l.time_first, ws.k, ws.v, u8 ? 0 : 1, ws.r, ws.rwkv, s.aa,
-                                    s.bb, s.pp, st, ws.wkv, aparts ? &em : nullptr)))
+                                    s.bb, s.pp, st, ws.wkv)))
             return rc;
         const rwkv_half *a_out = ws.rwkv;
-        if (aparts) {
-            a_out = ws.xs[0];
-            e.parts = aparts; e.p0 = em.p0; e.p2 = em.p2;
-        } else if (u8) {
+        if (u8) {
             if ((rc = mm8_prepare_launch(T, C, ws.rwkv, C, l.att_output.ry, l.att_output.my, ws.xs[0], s0[0], s2[0], st)))
                 return rc;
             a_out = ws.xs[0];
         }
+        e.act = ACT_RESIDUAL; e.res = ws.x; e.ldres = C;
         if ((rc = run_gemm(l.att_output, u8, T, a_out, s0[0], s2[0], ws.x, C, e, st, ws.splitk))) return rc;
-        e.parts = 0; e.p0 = e.p2 = nullptr;
         // ---- channel mix
         {
             SeqMixArgs a{};

@@ -149,23 +149,10 @@ template <int MODE>
 __global__ __launch_bounds__(64) void wkv4_chunk_apply_kernel(int T, int C, int L, const float *__restrict__ w_,
                                                               const float *__restrict__ u_, Wkv4IO<MODE> io,
                                                               float *__restrict__ aa_, float *__restrict__ bb_,
-                                                              float *__restrict__ pp_, const float *__restrict__ scratch,
-                                                              Wkv4Emit em) {
+                                                              float *__restrict__ pp_, const float *__restrict__ scratch) {
     constexpr int UNR = 8;
     const int c = blockIdx.x * 64 + threadIdx.x, j = blockIdx.y;
     if (c >= C) return;
-    const bool emit = MODE != 0 && em.ry != nullptr;   // whole waves then (C % 64 == 0)
-    const float ryc = emit ? h2f(em.ry[c]) : 0.f, myc = emit ? h2f(em.my[c]) : 0.f;
-    const int np = C >> 6;
-    // the gated output of one token: stored as it is, or scaled for the next product with this wave's partial sums
-    auto store = [&](int t, float out, float rr) {
-        const size_t o = (size_t)t * C + c;
-        if (!emit) { io.st(o, out, rr); return; }
-        const float yh = round_h(rr * round_h(out));
-        em.xs[o] = f2h(yh * ryc);
-        const float a0 = wave_sum(yh), a2 = wave_sum(yh * myc);
-        if (threadIdx.x == 0) { em.p0[(size_t)t * np + blockIdx.x] = a0; em.p2[(size_t)t * np + blockIdx.x] = a2; }
-    };
     const float u = u_[c], w = w_[c];
     const int t0 = j * L, t1 = min(T, t0 + L);
     float aa = scratch[c], bb = scratch[C + c], pp = scratch[2 * C + c];
@@ -187,7 +174,7 @@ __global__ __launch_bounds__(64) void wkv4_chunk_apply_kernel(int T, int C, int 
         for (int i = 0; i < UNR; ++i) {
             float out;
             wkv4_step(kk[i], vv[i], u, w, aa, bb, pp, out);
-            store(t + i, out, rr[i]);
+            io.st((size_t)(t + i) * C + c, out, rr[i]);
         }
     }
     for (; t < t1; ++t) {
@@ -195,7 +182,7 @@ __global__ __launch_bounds__(64) void wkv4_chunk_apply_kernel(int T, int C, int 
         float out;
         const float rr = io.ldr(o);
         wkv4_step(io.ldk(o), io.ldv(o), u, w, aa, bb, pp, out);
-        store(t, out, rr);
+        io.st(o, out, rr);
     }
     if (t1 == T) { aa_[c] = aa; bb_[c] = bb; pp_[c] = pp; }
 }
@@ -496,35 +483,27 @@ size_t wkv4_scratch_bytes(int64_t T, int64_t C) {
     return (size_t)((T + L - 1) / L + 1) * 3 * (size_t)C * sizeof(float);
 }
 
-bool wkv4_can_emit(int64_t T, int64_t C) { return T >= 64 && !(C & 63); }
-
 template <int MODE>
 static void wkv4_fused_run(int T, int C, const float *w, const float *u, Wkv4IO<MODE> io, float *aa, float *bb, float *pp,
-                           float *scratch, hipStream_t st, const Wkv4Emit &em) {
+                           float *scratch, hipStream_t st) {
     if (T >= 64 && scratch) {
         const int L = wkv4_chunk_len(T);
         const dim3 grid((unsigned)((C + 63) / 64), (unsigned)((T + L - 1) / L));
         hipLaunchKernelGGL(wkv4_chunk_summary_kernel<MODE>, grid, dim3(64), 0, st, T, C, L, w, io, aa, bb, pp, scratch);
-        hipLaunchKernelGGL(wkv4_chunk_apply_kernel<MODE>, grid, dim3(64), 0, st, T, C, L, w, u, io, aa, bb, pp, scratch, em);
+        hipLaunchKernelGGL(wkv4_chunk_apply_kernel<MODE>, grid, dim3(64), 0, st, T, C, L, w, u, io, aa, bb, pp, scratch);
     } else {
         hipLaunchKernelGGL(wkv4_kernel<MODE>, dim3((unsigned)((C + 63) / 64), 1), dim3(64), 0, st, T, C, w, u, io, aa, bb, pp);
     }
 }
 
 int wkv4_fused_launch(int T, int C, const float *w, const float *u, const void *k, const void *v, int kv_f32,
-                      const rwkv_half *r, rwkv_half *y, float *aa, float *bb, float *pp, hipStream_t st, float *scratch,
-                      const Wkv4Emit *emit) {
-    Wkv4Emit em{};
-    if (emit) {
-        if (!scratch || !wkv4_can_emit(T, C) || !emit->ry || !emit->my || !emit->xs || !emit->p0 || !emit->p2) return RWKV_E_SHAPE;
-        em = *emit;
-    }
+                      const rwkv_half *r, rwkv_half *y, float *aa, float *bb, float *pp, hipStream_t st, float *scratch) {
     if (kv_f32) {
         Wkv4IO<2> io{(const float *)k, (const float *)v, y, r};
-        wkv4_fused_run<2>(T, C, w, u, io, aa, bb, pp, scratch, st, em);
+        wkv4_fused_run<2>(T, C, w, u, io, aa, bb, pp, scratch, st);
     } else {
         Wkv4IO<1> io{(const rwkv_half *)k, (const rwkv_half *)v, y, r};
-        wkv4_fused_run<1>(T, C, w, u, io, aa, bb, pp, scratch, st, em);
+        wkv4_fused_run<1>(T, C, w, u, io, aa, bb, pp, scratch, st);
     }
     RWKV_LAUNCH_CHECK();
     return RWKV_OK;

@@ -690,8 +690,8 @@ def test_full_width_oracle_parity(shape, V, capsys):
 
 @pytest.mark.parametrize("shape", ["v4-7b", "v6-7b"])
 def test_handover_against_scaling_pass(shape, monkeypatch):
-    """Sequence calls at the 7B widths with uint8 weights hand the channel-mix value product, RWKV-4's time-mix
-    output product (and RWKV-6's four time-mix products) their input already scaled, with the row sums as partial sums that the consuming launch adds
+    """Sequence calls at the 7B widths with uint8 weights hand the channel-mix value product (and RWKV-6's four
+    time-mix products) their input already scaled, with the row sums as partial sums that the consuming launch adds
     up; RWKV_HANDOVER=0 keeps the separate scaling passes, whose results the oracle tests pin.  Same arithmetic per
     element, another summation order for the row sums: logits and states of the two forms agree far inside the
     parity tolerance, in calls of 256 (small tiles, K split, partial sums in two rounds) and 1024 tokens (large
@@ -713,9 +713,9 @@ def test_handover_against_scaling_pass(shape, monkeypatch):
             assert torch.equal(a, b)
         scale = float(ref.abs().max())
         assert float((out - ref).abs().max()) <= 2e-3 * max(scale, 1.0), (T, float((out - ref).abs().max()), scale)
-        for i, (a, b) in enumerate(zip(st, rst)):          # the WKV sums amplify an fp16 step of a key: 1 % as in the oracle tests
+        for i, (a, b) in enumerate(zip(st, rst)):
             s = max(float(b.float().abs().max()), 1.0)
-            assert float((a.float() - b.float()).abs().max()) <= 1e-2 * s, (T, i)
+            assert float((a.float() - b.float()).abs().max()) <= 2e-3 * s, (T, i)
 
 
 @pytest.mark.parametrize("L", [8, 32])
