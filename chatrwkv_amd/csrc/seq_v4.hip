@@ -2,9 +2,9 @@
 //   lnmix_seq (LN1, token shift, k/v/r mixes, ry scaling, row sums) -> 3 MFMA GEMMs (sigmoid fused for r)
 //   -> WKV-4 over T (r gating fused) -> GEMM Wo (+ residual)
 //   lnmix_seq (LN2, ...) -> GEMM Wr (sigmoid), GEMM Wk (relu^2) -> GEMM Wv (gate, residual, /2)
-// With uint8 weights the input of Wo and of Wv arrives scaled by the matrix's ry, with partial row sums, from the
-// launch that produces it (long calls through the direct-to-LDS kernel); otherwise a scaling pass (mm8_prepare)
-// sits in front of those two products.
+// With uint8 weights a scaling pass (mm8_prepare) sits in front of Wo; the input of Wv arrives scaled by that
+// matrix's ry, with partial row sums, from the epilogue of the Wk product (long calls through the direct-to-LDS
+// kernel; otherwise it has a scaling pass too).
 // and LN_out + head on the last row (GEMV) or on every row (GEMM) for full_output.
 #include <algorithm>
 #include <cstdlib>
