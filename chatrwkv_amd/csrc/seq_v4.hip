@@ -189,7 +189,10 @@ __global__ __launch_bounds__(256) void lnmix_seq_fast_kernel(SeqMixArgs a) {
     for (int c = 0; c < CH; ++c)
         if ((int)threadIdx.x + c * 256 < nch) {
 #pragma unroll
-            for (int e = 0; e < 8; ++e) { st[0] += (float)xv[c][e]; st[1] += (float)pxv[c][e]; st[2] += (float)lv[c][e]; }
+            for (int e = 0; e < 8; ++e) { st[0] += (float)xv[c][e]; st[1] += (float)pxv[c][e]; }
+            if (commit)   // the last row's statistics: only the workgroup that writes the new state needs them
+#pragma unroll
+                for (int e = 0; e < 8; ++e) st[2] += (float)lv[c][e];
         }
     block_sum_n<3>(st, red);
     const float mean = st[0] / C, pmean = st[1] / C, lmean = st[2] / C;
@@ -199,11 +202,16 @@ __global__ __launch_bounds__(256) void lnmix_seq_fast_kernel(SeqMixArgs a) {
         if ((int)threadIdx.x + c * 256 < nch) {
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-                const float d = (float)xv[c][e] - mean, pd = (float)pxv[c][e] - pmean, ld = (float)lv[c][e] - lmean;
+                const float d = (float)xv[c][e] - mean, pd = (float)pxv[c][e] - pmean;
                 st[0] += d * d;
                 st[1] += pd * pd;
-                st[2] += ld * ld;
             }
+            if (commit)
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const float ld = (float)lv[c][e] - lmean;
+                    st[2] += ld * ld;
+                }
         }
     block_sum_n<3>(st, red);
     const float rstd = rsqrtf(st[0] / C + LN_EPS), prstd = rsqrtf(st[1] / C + LN_EPS), lrstd = rsqrtf(st[2] / C + LN_EPS);
