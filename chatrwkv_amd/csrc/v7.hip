@@ -294,28 +294,44 @@ __global__ __launch_bounds__(256) void wkv7_kernel(Wkv7Args a) {
     *(f32x4 *)S = s;
 }
 
-// GroupNorm over each head's 64 outputs (eps 64e-5) on the fp16-rounded read-out, + bonus * v, * g:
-// one wave per (token, head).
+// GroupNorm over each head's 64 outputs (eps 64e-5) on the fp16-rounded read-out, + bonus * v, * g.  Four adjacent
+// channels per lane (16-byte loads of y, 8-byte accesses to v, g and the output): a row of 16 lanes owns one head
+// of one token, its two sums are DPP row sums; grid-stride over the T * C / 4 chunks.
 __global__ __launch_bounds__(256) void gn7_kernel(int T, int C, const float *__restrict__ y,
                                                   const rwkv_half *__restrict__ lnx_w,
                                                   const rwkv_half *__restrict__ lnx_b, const float *__restrict__ rk,
                                                   const rwkv_half *__restrict__ v, const rwkv_half *__restrict__ gate,
                                                   rwkv_half *__restrict__ out) {
-    const int H = C / HS7;
-    const int64_t wave = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (wave >= (int64_t)T * H) return;
-    const int lane = threadIdx.x & 63;
-    const int64_t t = wave / H;
-    const int h = (int)(wave - t * H);
-    const int c = h * HS7 + lane;
-    const size_t o = (size_t)t * C + c;
-    const float yv = round_h(y[o]);
-    const float mean = wave_sum(yv) * (1.f / HS7);
-    const float d = yv - mean;
-    const float var = wave_sum(d * d) * (1.f / HS7);
-    float q = round_h(d * rsqrtf(var + 64e-5f) * h2f(lnx_w[c]) + h2f(lnx_b[c]));
-    q = round_h(q + round_h(rk[wave] * h2f(v[o])));
-    out[o] = f2h(q * h2f(gate[o]));
+    const int64_t nchunk = (int64_t)T * C / 4;   // a multiple of 16: whole rows of lanes are live or idle together
+    const int cpr = C / 4, H = C / HS7;
+    for (int64_t i0 = (int64_t)blockIdx.x * 256; i0 < nchunk; i0 += (int64_t)gridDim.x * 256) {
+        const int64_t i = i0 + threadIdx.x;
+        const bool live = i < nchunk;
+        const int64_t ic = live ? i : nchunk - 1;
+        const int64_t t = ic / cpr;
+        const int c = (int)(ic - t * cpr) * 4;
+        const size_t o = (size_t)t * C + c;
+        const f32x4 y4 = *(const f32x4 *)(y + o);
+        const h16x4 w4 = *(const h16x4 *)(lnx_w + c), b4 = *(const h16x4 *)(lnx_b + c);
+        const h16x4 v4 = *(const h16x4 *)(v + o), g4 = *(const h16x4 *)(gate + o);
+        const float bonus = rk[t * H + c / HS7];
+        float yv[4], sum = 0.f;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) { yv[e] = round_h(y4[e]); sum += yv[e]; }
+        const float mean = row16_sum(sum) * (1.f / HS7);
+        float sq = 0.f;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) { const float d = yv[e] - mean; sq += d * d; }
+        const float rstd = rsqrtf(row16_sum(sq) * (1.f / HS7) + 64e-5f);
+        h16x4 o4;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            float q = round_h((yv[e] - mean) * rstd * (float)w4[e] + (float)b4[e]);
+            q = round_h(q + round_h(bonus * (float)v4[e]));
+            o4[e] = (h16)(q * (float)g4[e]);
+        }
+        if (live) *(h16x4 *)(out + o) = o4;
+    }
 }
 
 // ---- one-token kernels ---------------------------------------------------------------------
@@ -671,7 +687,6 @@ extern "C" int rwkv_v7_forward(const rwkv_v7_model *m, const rwkv_v56_layer_stat
     Ws7 ws = carve7(workspace, T, m);
     // the fp16 path needs no scaled-activation scratch or row sums
     Ctx c{st, false, T, num_cu(), nullptr, nullptr, nullptr, ws.splitk, 0};
-    const unsigned head_waves = (unsigned)(((int64_t)T * H + 3) / 4);
 
     const int max_rank = std::max(std::max(m->lora_w, m->lora_a), std::max(m->lora_v, m->lora_g));
     const int o_a = m->lora_w, o_v = o_a + m->lora_a, o_g = o_v + m->lora_v, rtot = o_g + m->lora_g;
@@ -829,7 +844,7 @@ extern "C" int rwkv_v7_forward(const rwkv_v7_model *m, const rwkv_v56_layer_stat
             Wkv7Args q{(int)T, C, s.att_kv, ws.r, ws.dec, ws.k, v, ws.an, ws.b, ws.y32};
             hipLaunchKernelGGL((wkv7_kernel<RWKV_DT_F16, true>), dim3((unsigned)(4 * H)), dim3(256), 0, st, q);
         }
-        hipLaunchKernelGGL(gn7_kernel, dim3(head_waves), dim3(256), 0, st, (int)T, C, ws.y32, l.lnx_w, l.lnx_b, ws.rk, v,
+        hipLaunchKernelGGL(gn7_kernel, dim3((unsigned)std::min<int64_t>(((int64_t)T * C / 4 + 255) / 256, 65535)), dim3(256), 0, st, (int)T, C, ws.y32, l.lnx_w, l.lnx_b, ws.rk, v,
                            ws.g, ws.att);
         if ((rc = mm(c, l.att_output, false, ws.att, ACT_RESIDUAL, ws.x, nullptr, 1.f, ws.x))) return rc;
         // ---- channel mix
