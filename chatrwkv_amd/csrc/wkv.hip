@@ -1,4 +1,5 @@
 // WKV recurrences: RWKV-4 (per channel, running-maximum form) and RWKV-5/6 (per-head 64x64 state).
+#include <algorithm>
 #include "gemv_core.h"
 #include "kernels.h"
 
@@ -455,25 +456,38 @@ __global__ __launch_bounds__(256) void wkv56_split_kernel(Wkv56Args a) {
     for (int e = 0; e < 4; ++e) S[(4 * g + e) * HS + i] = s[e];
 }
 
-// GroupNorm over each head's 64 outputs (eps 64e-5), affine, fp16 rounding, gate: one wave per (token, head).
+// GroupNorm over each head's 64 outputs (eps 64e-5), affine, fp16 rounding, gate.  Four adjacent channels per lane
+// (16-byte loads of y and of the affine vectors, 8-byte accesses to the gate and the output): a row of 16 lanes owns
+// one head of one token, its two sums are DPP row sums; grid-stride over the T * C / 4 chunks.
 __global__ __launch_bounds__(256) void wkv56_gn_kernel(int T, int C, const float *__restrict__ y,
                                                        const float *__restrict__ lnx_w, const float *__restrict__ lnx_b,
                                                        const rwkv_half *__restrict__ gate, rwkv_half *__restrict__ out) {
-    const int H = C / HS;
-    const int64_t wave = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (wave >= (int64_t)T * H) return;
-    const int c = threadIdx.x & 63;
-    const int64_t t = wave / H;
-    const int h = (int)(wave - t * H);
-    const size_t o = (size_t)t * C + h * HS + c;
-    const float v = y[o];
-    const float mean = wave_sum(v) * (1.f / HS);
-    const float d = v - mean;
-    const float var = wave_sum(d * d) * (1.f / HS);
-    float gq = d * rsqrtf(var + 64e-5f) * lnx_w[h * HS + c] + lnx_b[h * HS + c];
-    gq = round_h(gq);
-    if (gate) gq = gq * h2f(gate[o]);
-    out[o] = f2h(gq);
+    const int64_t nchunk = (int64_t)T * C / 4;   // a multiple of 16: whole rows of lanes are live or idle together
+    const int cpr = C / 4;
+    for (int64_t i0 = (int64_t)blockIdx.x * 256; i0 < nchunk; i0 += (int64_t)gridDim.x * 256) {
+        const int64_t i = i0 + threadIdx.x;
+        const bool live = i < nchunk;
+        const int64_t ic = live ? i : nchunk - 1;
+        const int64_t t = ic / cpr;
+        const int c = (int)(ic - t * cpr) * 4;
+        const size_t o = (size_t)t * C + c;
+        const f32x4 y4 = *(const f32x4 *)(y + o), w4 = *(const f32x4 *)(lnx_w + c), b4 = *(const f32x4 *)(lnx_b + c);
+        h16x4 g4 = {};
+        if (gate) g4 = *(const h16x4 *)(gate + o);
+        const float mean = row16_sum((y4[0] + y4[1]) + (y4[2] + y4[3])) * (1.f / HS);
+        float sq = 0.f;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) { const float d = y4[e] - mean; sq += d * d; }
+        const float rstd = rsqrtf(row16_sum(sq) * (1.f / HS) + 64e-5f);
+        h16x4 o4;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            float gq = round_h((y4[e] - mean) * rstd * w4[e] + b4[e]);
+            if (gate) gq = gq * (float)g4[e];
+            o4[e] = (h16)gq;
+        }
+        if (live) *(h16x4 *)(out + o) = o4;
+    }
 }
 
 
@@ -542,9 +556,8 @@ int wkv56_fused_launch(bool v6, int T, int C, int H, float *state, const rwkv_ha
         a.y = y32;
         if (v6) hipLaunchKernelGGL((wkv56_split_kernel<2>), dim3((unsigned)(4 * H)), dim3(256), 0, st, a);
         else hipLaunchKernelGGL((wkv56_split_kernel<0>), dim3((unsigned)(4 * H)), dim3(256), 0, st, a);
-        const int64_t waves = (int64_t)T * H;
-        hipLaunchKernelGGL(wkv56_gn_kernel, dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, st, T, C, y32, lnx_w, lnx_b,
-                           gate, out);
+        hipLaunchKernelGGL(wkv56_gn_kernel, dim3((unsigned)std::min<int64_t>(((int64_t)T * C / 4 + 255) / 256, 65535)), dim3(256), 0, st,
+                           T, C, y32, lnx_w, lnx_b, gate, out);
     } else if (v6 && dw2) {
         if (ld <= 0 || (ld & 7)) return RWKV_E_SHAPE;
         hipLaunchKernelGGL((wkv56_kernel<true, 3, true>), dim3((unsigned)H), dim3(256), 0, st, a);
