@@ -751,11 +751,13 @@ extern "C" int rwkv_v7_forward(const rwkv_v7_model *m, const rwkv_v56_layer_stat
                         *xg = ws.mix[5];
         rwkv_half *v = i == 0 ? ws.v_first : ws.v;
         // The three C x C products and the LoRA chain are independent of each other.  From 256 rows on receptance,
-        // key and value are one grouped launch of the direct-to-LDS kernel; where that group fills three quarters
-        // of the chip without splitting K, the eight small LoRA products (which do split K: one user of the split-K
-        // scratch at a time) run beside it on a side stream, on the CUs the group leaves free.
+        // key and value are one grouped launch of the direct-to-LDS kernel; where that group is more than one round
+        // of large tiles (2048 tokens at n_embd 4096), the LoRA launches (which do split K: one user of the split-K
+        // scratch at a time) run beside it on a side stream.  Measured with the LoRA stages grouped: 46.0K against
+        // 45.7K tok/s in calls of 2048, but 42.3K against 43.3K in calls of 1024, where the group is one round and
+        // the two streams only slow each other down.
         const bool dma_seq = true;
-        ForkScope par(ss, st, 1, dma_seq && 3 * ((T + 255) / 256) * ((C + 255) / 256) >= 192);
+        ForkScope par(ss, st, 1, dma_seq && 3 * ((T + 255) / 256) * ((C + 255) / 256) >= 384);
         Ctx cm = c, cv = c, cl = c;
         if (par) cl.st = ss->s[0];
         if (dma_seq && !(C & 7)) {
