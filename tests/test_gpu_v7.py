@@ -344,6 +344,29 @@ def test_v7_full_width_oracle_parity():
         assert np.abs(_np(s) - ref.astype(np.float32)).max() <= 1e-2 * scale, i
 
 
+def test_v7_long_call_with_lora_side_stream():
+    """At the 7B width a call of 2048 tokens runs the grouped LoRA launches on a side stream beside the receptance /
+    key / value group (calls of 1024 keep everything on the caller's stream): its logits and states must agree with
+    the same tokens fed as two calls of 1024, and a second identical call must reproduce it bit for bit."""
+    C, F, V = 4096, 16384, 1003
+    ck = synth.make_checkpoint_v7(n_layer=2, n_embd=C, n_ffn=F, vocab=V, seed=29, device="cuda:0")
+    m = _x070()(ck, "cuda fp16")
+    del ck
+    toks = synth.random_tokens(2048, V, seed=30)
+    out, st = m.forward(toks, None)
+    out_b, st_b = m.forward(toks, None)
+    assert torch.equal(out, out_b)
+    for x, y in zip(st, st_b):
+        assert torch.equal(x, y)
+    st2 = None
+    for a in range(0, 2048, 1024):
+        out2, st2 = m.forward(toks[a:a + 1024], st2)
+    assert float((out.float() - out2.float()).abs().max()) <= LOGIT_TOL
+    for i, (s, s2) in enumerate(zip(st, st2)):
+        scale = max(float(s2.float().abs().max()), 1.0)
+        assert float((s.float() - s2.float()).abs().max()) <= 1e-2 * scale, i
+
+
 def test_v7_side_stream_path(tiny7):
     """A call of 256 tokens or more runs the independent products of a layer on three streams; its logits and
     states must match the oracle and the same prompt fed in shorter calls (which stay on one stream)."""
